@@ -1,0 +1,214 @@
+"""ctypes binding of the C ABI in include/f2cgt.h (libf2cgt_hip.so).
+
+This is the binding a non-pybind caller would write: raw device pointers, sizes and a
+hipStream_t.  The helpers at the bottom accept torch tensors only to extract
+`data_ptr()` and torch's current stream; they allocate the output with torch and call
+the C entry point.  No computation happens on the Python side and there is no fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_int, c_int64, c_void_p
+
+from . import capi_path
+
+DT_U8, DT_I8, DT_I16, DT_I32, DT_I64, DT_F16, DT_F32, DT_F64 = range(8)
+METRIC_L2, METRIC_COSINE = 0, 1
+
+P, I, L = c_void_p, c_int, c_int64
+
+SIGNATURES = {
+    "f2cgt_version": ([], c_int),
+    "f2cgt_last_error": ([], c_char_p),
+    "f2cgt_num_cus": ([], c_int),
+    "f2cgt_packbits": ([P, P, L, L, I, P], c_int),
+    "f2cgt_unpackbits": ([P, P, L, L, L, I, P], c_int),
+    "f2cgt_sq_compress": ([P, P, P, L, L, L, I, L, P], c_int),
+    "f2cgt_sq_decompress": ([P, I, P, P, L, L, L, L, I, L, P], c_int),
+    "f2cgt_sq_affine_decompress": ([P, P, P, L, L, L, L, I, P], c_int),
+    "f2cgt_vq_decompress": ([P, I, P, I, P, L, L, L, L, L, P], c_int),
+    "f2cgt_spmm_csr": ([P, I, P, P, P, I, L, L, L, L, P], c_int),
+    "f2cgt_vq_decompress_spmm_csr": ([P, I, P, P, P, I, P, L, L, L, L, L, L, L, P], c_int),
+    "f2cgt_sq_decompress_spmm_csr": ([P, I, P, P, P, I, P, L, L, L, L, L, L, I, L, P], c_int),
+    "f2cgt_sq_affine_decompress_spmm_csr": ([P, P, L, P, P, I, P, L, L, L, L, L, I, P], c_int),
+    "f2cgt_hybrid_decompress_spmm_csr":
+        ([P, P, P, L, P, P, P, P, I, P, L, L, L, L, L, L, L, L, L, P], c_int),
+    "f2cgt_pairwise_distance": ([P, P, P, L, L, L, I, P], c_int),
+    "f2cgt_kmeans_predict": ([P, P, P, P, L, L, L, I, P], c_int),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded libf2cgt_hip.so with argument types declared."""
+    global _lib
+    if _lib is None:
+        import torch  # noqa: F401  (loads the HIP runtime the library links against)
+        handle = ctypes.CDLL(capi_path())
+        for name, (argtypes, restype) in SIGNATURES.items():
+            fn = getattr(handle, name)  # AttributeError if the symbol is not exported
+            fn.argtypes = argtypes
+            fn.restype = restype
+        _lib = handle
+    return _lib
+
+
+class F2CGTError(RuntimeError):
+    pass
+
+
+def _check(rc, name):
+    if rc != 0:
+        raise F2CGTError("%s failed (%d): %s" % (name, rc, lib().f2cgt_last_error().decode()))
+
+
+def _tag(t):
+    import torch
+    return {torch.uint8: DT_U8, torch.int8: DT_I8, torch.int16: DT_I16, torch.int32: DT_I32,
+            torch.int64: DT_I64, torch.float16: DT_F16, torch.float32: DT_F32,
+            torch.float64: DT_F64}[t.dtype]
+
+
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+# ---- tensor-level helpers (tests, benchmark) ---------------------------------------------
+def packbits(unpack, bits):
+    import torch
+    per = 8 // bits
+    out = torch.empty((unpack.shape[0], (unpack.shape[1] + per - 1) // per), dtype=torch.uint8,
+                      device=unpack.device)
+    _check(lib().f2cgt_packbits(_ptr(unpack), _ptr(out), unpack.shape[0], unpack.shape[1], bits,
+                                _stream()), "packbits")
+    return out
+
+
+def unpackbits(pack, bits, unpack_dim):
+    import torch
+    out = torch.empty((pack.shape[0], unpack_dim), dtype=torch.uint8, device=pack.device)
+    _check(lib().f2cgt_unpackbits(_ptr(pack), _ptr(out), pack.shape[0], pack.shape[1], unpack_dim,
+                                  bits, _stream()), "unpackbits")
+    return out
+
+
+def sq_compress(src, codebooks, bits, column_slice):
+    import torch
+    out = torch.empty_like(src)
+    _check(lib().f2cgt_sq_compress(_ptr(src), _ptr(out), _ptr(codebooks), src.shape[0], src.shape[1],
+                                   codebooks.shape[0], bits, column_slice, _stream()), "sq_compress")
+    return out
+
+
+def sq_decompress(codes, codebooks, bits, column_slice, feat_dim):
+    import torch
+    out = torch.empty((codes.shape[0], feat_dim), dtype=torch.float32, device=codes.device)
+    _check(lib().f2cgt_sq_decompress(_ptr(codes), _tag(codes), _ptr(out), _ptr(codebooks),
+                                     codes.shape[0], codes.shape[1], feat_dim, codebooks.shape[0], bits,
+                                     column_slice, _stream()), "sq_decompress")
+    return out
+
+
+def sq_affine_decompress(codes, params, bits, feat_dim):
+    import torch
+    out = torch.empty((codes.shape[0], feat_dim), dtype=torch.float32, device=codes.device)
+    _check(lib().f2cgt_sq_affine_decompress(_ptr(codes), _ptr(out), _ptr(params), params.shape[1],
+                                            codes.shape[0], codes.shape[1], feat_dim, bits, _stream()),
+           "sq_affine_decompress")
+    return out
+
+
+def vq_decompress(codes, codebooks, feat_dim):
+    import torch
+    out = torch.empty((codes.shape[0], feat_dim), dtype=torch.float32, device=codes.device)
+    _check(lib().f2cgt_vq_decompress(_ptr(codes), _tag(codes), _ptr(codebooks), _tag(codebooks),
+                                     _ptr(out), codes.shape[0], feat_dim, codebooks.shape[0],
+                                     codebooks.shape[1], codebooks.shape[2], _stream()), "vq_decompress")
+    return out
+
+
+def spmm_csr(feat, indptr, indices, out=None):
+    import torch
+    rows = indptr.numel() - 1
+    if out is None:
+        out = torch.empty((rows, feat.shape[1]), dtype=feat.dtype, device=feat.device)
+    _check(lib().f2cgt_spmm_csr(_ptr(feat), _tag(feat), _ptr(out), _ptr(indptr), _ptr(indices),
+                                _tag(indptr), rows, indices.numel(), feat.shape[0], feat.shape[1],
+                                _stream()), "spmm_csr")
+    return out
+
+
+def vq_decompress_spmm_csr(codes, codebooks, indptr, indices, feat_dim, out=None):
+    import torch
+    rows = indptr.numel() - 1
+    if out is None:
+        out = torch.empty((rows, feat_dim), dtype=torch.float32, device=codes.device)
+    _check(lib().f2cgt_vq_decompress_spmm_csr(
+        _ptr(codes), _tag(codes), _ptr(codebooks), _ptr(indptr), _ptr(indices), _tag(indptr), _ptr(out),
+        rows, indices.numel(), codes.shape[0], feat_dim, codebooks.shape[0], codebooks.shape[1],
+        codebooks.shape[2], _stream()), "vq_decompress_spmm_csr")
+    return out
+
+
+def sq_decompress_spmm_csr(codes, codebooks, indptr, indices, bits, column_slice, feat_dim, out=None):
+    import torch
+    rows = indptr.numel() - 1
+    if out is None:
+        out = torch.empty((rows, feat_dim), dtype=torch.float32, device=codes.device)
+    _check(lib().f2cgt_sq_decompress_spmm_csr(
+        _ptr(codes), _tag(codes), _ptr(codebooks), _ptr(indptr), _ptr(indices), _tag(indptr), _ptr(out),
+        rows, indices.numel(), codes.shape[0], codes.shape[1], feat_dim, codebooks.shape[0], bits,
+        column_slice, _stream()), "sq_decompress_spmm_csr")
+    return out
+
+
+def sq_affine_decompress_spmm_csr(codes, params, indptr, indices, bits, feat_dim, out=None):
+    import torch
+    rows = indptr.numel() - 1
+    if out is None:
+        out = torch.empty((rows, feat_dim), dtype=torch.float32, device=codes.device)
+    _check(lib().f2cgt_sq_affine_decompress_spmm_csr(
+        _ptr(codes), _ptr(params), params.shape[1], _ptr(indptr), _ptr(indices), _tag(indptr), _ptr(out),
+        rows, indices.numel(), codes.shape[0], codes.shape[1], feat_dim, bits, _stream()),
+        "sq_affine_decompress_spmm_csr")
+    return out
+
+
+def hybrid_decompress_spmm_csr(row_map, sq_codes, sq_params, vq_codes, vq_codebooks, indptr, indices,
+                               feat_dim, out=None):
+    import torch
+    rows = indptr.numel() - 1
+    if out is None:
+        out = torch.empty((rows, feat_dim), dtype=torch.float32, device=row_map.device)
+    _check(lib().f2cgt_hybrid_decompress_spmm_csr(
+        _ptr(row_map), _ptr(sq_codes), _ptr(sq_params), sq_params.shape[1], _ptr(vq_codes),
+        _ptr(vq_codebooks), _ptr(indptr), _ptr(indices), _tag(indptr), _ptr(out), rows, indices.numel(),
+        row_map.numel(), sq_codes.shape[0], vq_codes.shape[0], feat_dim, vq_codebooks.shape[0],
+        vq_codebooks.shape[1], vq_codebooks.shape[2], _stream()), "hybrid_decompress_spmm_csr")
+    return out
+
+
+def pairwise_distance(x, y, metric):
+    import torch
+    out = torch.empty((x.shape[0], y.shape[0]), dtype=torch.float32, device=x.device)
+    _check(lib().f2cgt_pairwise_distance(_ptr(x), _ptr(y), _ptr(out), x.shape[0], y.shape[0], x.shape[1],
+                                         METRIC_COSINE if metric == "cosine" else METRIC_L2, _stream()),
+           "pairwise_distance")
+    return out
+
+
+def kmeans_predict(x, centers, metric, u8=False, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((x.shape[0],), dtype=torch.uint8 if u8 else torch.int64, device=x.device)
+    _check(lib().f2cgt_kmeans_predict(_ptr(x), _ptr(centers), None if u8 else _ptr(out),
+                                      _ptr(out) if u8 else None, x.shape[0], centers.shape[0], x.shape[1],
+                                      METRIC_COSINE if metric == "cosine" else METRIC_L2, _stream()),
+           "kmeans_predict")
+    return out

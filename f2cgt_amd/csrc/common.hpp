@@ -1,0 +1,102 @@
+// Shared host/device helpers of libf2cgt_hip.so (gfx950 only, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/f2cgt.h"
+
+namespace f2cgt {
+
+constexpr int kWave = 64;
+
+// ---- error reporting ---------------------------------------------------------
+char* error_buffer();  // thread-local, 512 bytes (defined in runtime.hip)
+
+inline int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// Checks the launch that was just enqueued; returns 0 or the hipError_t (> 0).
+inline int launch_status(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return 0;
+  snprintf(error_buffer(), 512, "%s: %s", what, hipGetErrorString(e));
+  return (int)e;
+}
+
+#define F2CGT_REQUIRE(cond, code, ...) \
+  do {                                 \
+    if (!(cond)) return ::f2cgt::fail((code), __VA_ARGS__); \
+  } while (0)
+
+int num_cus();  // compute units of the current device (cached per device)
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+__host__ __device__ constexpr int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+inline int pow2_ceil(int v) {
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+// ---- device helpers ----------------------------------------------------------
+template <typename Idx>
+__device__ __forceinline__ int64_t clamp_idx(Idx v, int64_t hi_exclusive) {
+  int64_t x = (int64_t)v;
+  x = x < 0 ? 0 : x;
+  return x >= hi_exclusive ? hi_exclusive - 1 : x;
+}
+
+// Edge range of CSC row r, clamped to [0, num_edges] and made monotone.
+template <typename Idx>
+__device__ __forceinline__ void row_range(const Idx* __restrict__ indptr, int64_t r,
+                                          int64_t num_edges, int64_t& b, int64_t& e) {
+  int64_t b0 = (int64_t)indptr[r];
+  int64_t e0 = (int64_t)indptr[r + 1];
+  b0 = b0 < 0 ? 0 : (b0 > num_edges ? num_edges : b0);
+  e0 = e0 < b0 ? b0 : (e0 > num_edges ? num_edges : e0);
+  b = b0;
+  e = e0;
+}
+
+// Non-temporal stores: the aggregation output is written once and never re-read by
+// the kernel, so it should not displace gathered code rows from L2 / MALL.
+__device__ __forceinline__ void store_nt(float* p, float v) { __builtin_nontemporal_store(v, p); }
+__device__ __forceinline__ void store_nt2(float* p, float a, float b) {
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  f2 v = {a, b};
+  __builtin_nontemporal_store(v, reinterpret_cast<f2*>(p));
+}
+__device__ __forceinline__ void store_nt4(float* p, float a, float b, float c, float d) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  f4 v = {a, b, c, d};
+  __builtin_nontemporal_store(v, reinterpret_cast<f4*>(p));
+}
+
+// Correctly rounded fp32 exp2 / log2: the fp64 library result rounded once.
+__device__ __forceinline__ float exp2_cr(float x) { return (float)exp2((double)x); }
+__device__ __forceinline__ float log2_cr(float x) { return (float)log2((double)x); }
+
+// Decoded value of one log-domain SQ code (bits > 1).  `signed_code` is the code after
+// removing the storage bias; fp32, product and sum rounded separately.
+__device__ __forceinline__ float sq_log_decode(float signed_code, float k, float emin) {
+  float v = signed_code + 0.5f;
+  float s = v >= 0.f ? 1.f : -1.f;
+  float t = __fadd_rn(__fmul_rn(fabsf(v), k), emin);
+  return exp2_cr(t) * s;
+}
+
+}  // namespace f2cgt

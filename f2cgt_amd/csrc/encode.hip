@@ -1,0 +1,360 @@
+// VQ encode: pairwise distance and nearest-centre assignment.
+//
+// pairwise_distance materialises the [m,n] matrix and is bounded by that write; it
+// evaluates the unexpanded form sum((x-y)^2) (or 1 - cos) on the vector ALUs so the
+// numbers carry no cancellation error.
+//
+// kmeans_predict never writes the matrix.  A wave owns 32 rows of x and walks the
+// centres 32 at a time with fp32 MFMA (v_mfma_f32_32x32x2_f32): A = centre tile,
+// B = x tile, so every lane holds 16 centre scores of ONE x row and the running
+// arg-min stays in registers.  Scores use the expanded form (|c|^2 - 2 x.c, the row
+// constant |x|^2 dropped); rows whose two best scores are closer than the rounding
+// bound of that form are re-evaluated exactly in fp64 by the whole wave, so the label
+// is the true first minimum.
+#include "common.hpp"
+
+#include <cfloat>
+#include <climits>
+
+namespace f2cgt {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// ---- exact assignment of one row by a whole wave (fp64) ------------------------------
+__device__ int exact_argmin_row(const float* __restrict__ xrow, const float* __restrict__ centers,
+                                int n, int k, int metric, int lane) {
+  double bestv = DBL_MAX;
+  int besti = INT_MAX;
+  double xn = 0.0;
+  if (metric == F2CGT_METRIC_COSINE)
+    for (int t = 0; t < k; ++t) xn += (double)xrow[t] * (double)xrow[t];
+  for (int c = lane; c < n; c += kWave) {
+    const float* cr = centers + (int64_t)c * k;
+    double d;
+    if (metric == F2CGT_METRIC_COSINE) {
+      double dot = 0.0, cn = 0.0;
+      for (int t = 0; t < k; ++t) {
+        dot += (double)xrow[t] * (double)cr[t];
+        cn += (double)cr[t] * (double)cr[t];
+      }
+      double den = sqrt(xn) * sqrt(cn);
+      den = den > 1e-8 ? den : 1e-8;
+      d = 1.0 - dot / den;
+    } else {
+      d = 0.0;
+      for (int t = 0; t < k; ++t) {
+        const double df = (double)xrow[t] - (double)cr[t];
+        d += df * df;
+      }
+    }
+    if (d < bestv) { bestv = d; besti = c; }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const double ov = __shfl_xor(bestv, off);
+    const int oi = __shfl_xor(besti, off);
+    if (ov < bestv || (ov == bestv && oi < besti)) { bestv = ov; besti = oi; }
+  }
+  return besti;
+}
+
+// ---- general fallback: one wave per row, exact -------------------------------------------
+__global__ __launch_bounds__(256) void predict_exact_kernel(const float* __restrict__ x,
+                                                            const float* __restrict__ centers,
+                                                            int64_t* __restrict__ lab64,
+                                                            uint8_t* __restrict__ lab8, int64_t m,
+                                                            int n, int k, int metric) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  for (int64_t row = wave; row < m; row += stride) {
+    const int best = exact_argmin_row(x + row * k, centers, n, k, metric, lane);
+    if (lane == 0) {
+      if (lab64) lab64[row] = best;
+      if (lab8) lab8[row] = (uint8_t)best;
+    }
+  }
+}
+
+// ---- MFMA path ----------------------------------------------------------------------------
+// KH = per-half register depth: the k dimensions are split in two halves of
+// khalf = ceil(k/2); lanes 0-31 feed half 0, lanes 32-63 half 1 (zero padded to KH).
+template <int KH>
+__global__ __launch_bounds__(256) void predict_mfma_kernel(const float* __restrict__ x,
+                                                           const float* __restrict__ centers,
+                                                           int64_t* __restrict__ lab64,
+                                                           uint8_t* __restrict__ lab8, int64_t m,
+                                                           int n, int k, int metric, int n_pad) {
+  extern __shared__ float smem[];
+  float* cT = smem;                   // [2*KH][n_pad]  centre coordinates, transposed
+  float* bias = cT + 2 * KH * n_pad;  // [n_pad]  score = bias + mul * dot
+  float* mul = bias + n_pad;          // [n_pad]
+  int* cmax_bits = reinterpret_cast<int*>(mul + n_pad);  // max |c|^2 as ordered int bits
+
+  const int khalf = (k + 1) / 2;
+  if (threadIdx.x == 0) *cmax_bits = 0;
+  __syncthreads();
+  for (int j = threadIdx.x; j < n_pad; j += blockDim.x) {
+    float cn = 0.f;
+#pragma unroll 4
+    for (int kk = 0; kk < 2 * KH; ++kk) {
+      const int h = kk / KH, t = kk - h * KH;
+      const int dim = h * khalf + t;
+      const bool ok = j < n && t < khalf && dim < k;
+      const float v = ok ? centers[(int64_t)j * k + dim] : 0.f;
+      cT[kk * n_pad + j] = v;
+      cn += v * v;
+    }
+    if (j >= n) {
+      bias[j] = INFINITY;
+      mul[j] = 0.f;
+    } else if (metric == F2CGT_METRIC_COSINE) {
+      const float nr = sqrtf(cn);
+      bias[j] = 0.f;
+      mul[j] = -1.f / (nr > 1e-30f ? nr : 1e-30f);
+    } else {
+      bias[j] = cn;
+      mul[j] = -2.f;
+      atomicMax(cmax_bits, __float_as_int(cn));
+    }
+  }
+  __syncthreads();
+  const float cmax = __int_as_float(*cmax_bits);
+
+  const int lane = threadIdx.x & 63;
+  const int j = lane & 31;
+  const int h = lane >> 5;
+  const int64_t n_tiles = (m + 31) / 32;
+  const float unit = 5.9604645e-8f * (float)(4 * k + 16);
+  const bool vec4 = (k % 8 == 0) && (KH % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+
+  for (int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); tile < n_tiles;
+       tile += (int64_t)gridDim.x * 4) {
+    const int64_t row = tile * 32 + j;
+    const bool valid = row < m;
+    float xr[KH];
+    float xn = 0.f;
+    const float* xp = x + row * k + h * khalf;
+    if (vec4) {
+#pragma unroll
+      for (int t = 0; t < KH; t += 4) {
+        float4 q = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (valid && t < khalf) q = *reinterpret_cast<const float4*>(xp + t);
+        xr[t] = q.x; xr[t + 1] = q.y; xr[t + 2] = q.z; xr[t + 3] = q.w;
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < KH; ++t) {
+        const int dim = h * khalf + t;
+        xr[t] = (valid && t < khalf && dim < k) ? xp[t] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < KH; ++t) xn += xr[t] * xr[t];
+    xn += __shfl_xor(xn, 32);
+
+    float best = INFINITY, second = INFINITY;
+    int besti = 0;
+    for (int ct = 0; ct < n_pad; ct += 32) {
+      floatx16 acc;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+      const float* ap = cT + (h * KH) * n_pad + ct + j;
+#pragma unroll
+      for (int t = 0; t < KH; ++t)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[t * n_pad], xr[t], acc, 0, 0, 0);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int ci = ct + 8 * (v / 4) + 4 * h + (v % 4);
+        const float s = bias[ci] + mul[ci] * acc[v];
+        if (s < best) {
+          second = best;
+          best = s;
+          besti = ci;
+        } else if (s < second) {
+          second = s;
+        }
+      }
+    }
+    {  // merge the two halves of the wave (same x row, disjoint centres)
+      const float ob = __shfl_xor(best, 32);
+      const float os = __shfl_xor(second, 32);
+      const int oi = __shfl_xor(besti, 32);
+      if (ob < best || (ob == best && oi < besti)) {
+        second = fminf(best, os);
+        best = ob;
+        besti = oi;
+      } else {
+        second = fminf(second, ob);
+      }
+    }
+    const float scale = metric == F2CGT_METRIC_COSINE ? sqrtf(xn) : xn + cmax;
+    const bool near_tie = valid && h == 0 && !((second - best) > unit * scale);
+    uint64_t todo = __ballot(near_tie);
+    while (todo) {
+      const int src = __ffsll((unsigned long long)todo) - 1;
+      todo &= todo - 1;
+      const int64_t rrow = tile * 32 + (src & 31);
+      const int exact = exact_argmin_row(x + rrow * k, centers, n, k, metric, lane);
+      if (lane == src) besti = exact;
+    }
+    if (valid && h == 0) {
+      if (lab64) lab64[row] = besti;
+      if (lab8) lab8[row] = (uint8_t)besti;
+    }
+  }
+}
+
+// ---- pairwise distance --------------------------------------------------------------------
+constexpr int kTile = 64;   // rows of x and of y per workgroup
+constexpr int kChunk = 32;  // k dimensions staged per pass
+
+__global__ __launch_bounds__(256) void pairwise_kernel(const float* __restrict__ x,
+                                                       const float* __restrict__ y,
+                                                       float* __restrict__ dist, int64_t m, int64_t n,
+                                                       int k, int metric) {
+  __shared__ float xs[kChunk][kTile + 1];
+  __shared__ float ys[kChunk][kTile + 1];
+  const int tx = threadIdx.x & 15;  // 4 y rows each
+  const int ty = threadIdx.x >> 4;  // 4 x rows each
+  const int64_t n_tiles_n = (n + kTile - 1) / kTile;
+  const int64_t n_tiles = ((m + kTile - 1) / kTile) * n_tiles_n;
+  for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+    const int64_t i0 = (tile / n_tiles_n) * kTile;
+    const int64_t j0 = (tile % n_tiles_n) * kTile;
+    float acc[4][4], xn[4], yn[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      xn[a] = 0.f;
+      yn[a] = 0.f;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) acc[a][b] = 0.f;
+    }
+    for (int k0 = 0; k0 < k; k0 += kChunk) {
+      __syncthreads();
+      for (int t = threadIdx.x; t < kTile * kChunk; t += 256) {
+        const int r = t / kChunk, c = t % kChunk;
+        const bool kin = k0 + c < k;
+        xs[c][r] = (kin && i0 + r < m) ? x[(i0 + r) * k + k0 + c] : 0.f;
+        ys[c][r] = (kin && j0 + r < n) ? y[(j0 + r) * k + k0 + c] : 0.f;
+      }
+      __syncthreads();
+      const int kc = (k - k0) < kChunk ? (k - k0) : kChunk;
+      for (int c = 0; c < kc; ++c) {
+        float xv[4], yv[4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          xv[a] = xs[c][ty * 4 + a];
+          yv[a] = ys[c][tx * 4 + a];
+        }
+        if (metric == F2CGT_METRIC_COSINE) {
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            xn[a] += xv[a] * xv[a];
+            yn[a] += yv[a] * yv[a];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) acc[a][b] += xv[a] * yv[b];
+          }
+        } else {
+#pragma unroll
+          for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+              const float d = xv[a] - yv[b];
+              acc[a][b] += d * d;
+            }
+        }
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int64_t i = i0 + ty * 4 + a;
+      if (i >= m) continue;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int64_t j = j0 + tx * 4 + b;
+        if (j >= n) continue;
+        float v = acc[a][b];
+        if (metric == F2CGT_METRIC_COSINE) {
+          float den = sqrtf(xn[a]) * sqrtf(yn[b]);
+          den = den > 1e-8f ? den : 1e-8f;
+          v = 1.f - v / den;
+        }
+        dist[i * n + j] = v;
+      }
+    }
+  }
+}
+
+template <int KH>
+int launch_mfma(const float* x, const float* centers, int64_t* l64, uint8_t* l8, int64_t m, int n,
+                int k, int metric, int n_pad, size_t lds, hipStream_t st) {
+  auto kern = predict_mfma_kernel<KH>;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail((int)e, "kmeans_predict: cannot reserve %zu B of LDS", lds);
+  }
+  int per_cu = (int)((144 * 1024) / lds);
+  per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
+  int64_t need = ceil_div(ceil_div(m, 32), 4);
+  int64_t cap = (int64_t)num_cus() * per_cu;
+  const int grid = (int)(need < cap ? need : cap);
+  kern<<<grid, 256, lds, st>>>(x, centers, l64, l8, m, n, k, metric, n_pad);
+  return launch_status("kmeans_predict");
+}
+
+}  // namespace
+}  // namespace f2cgt
+
+using namespace f2cgt;
+
+extern "C" int f2cgt_pairwise_distance(const float* x, const float* y, float* dist, int64_t m,
+                                       int64_t n, int64_t k, int metric, void* stream) {
+  F2CGT_REQUIRE(m >= 0 && n >= 0 && k >= 0, F2CGT_E_INVALID, "pairwise_distance: negative size");
+  F2CGT_REQUIRE(k < (1 << 24), F2CGT_E_UNSUPPORTED, "pairwise_distance: k too large");
+  F2CGT_REQUIRE(metric == F2CGT_METRIC_L2 || metric == F2CGT_METRIC_COSINE, F2CGT_E_INVALID,
+                "pairwise_distance: unknown metric %d", metric);
+  if (m * n == 0) return 0;
+  F2CGT_REQUIRE(dist && (k == 0 || (x && y)), F2CGT_E_INVALID, "pairwise_distance: null buffer");
+  const int64_t tiles = ceil_div(m, kTile) * ceil_div(n, kTile);
+  const int64_t cap = (int64_t)num_cus() * 8;
+  pairwise_kernel<<<(int)(tiles < cap ? tiles : cap), 256, 0, as_stream(stream)>>>(x, y, dist, m, n,
+                                                                                  (int)k, metric);
+  return launch_status("pairwise_distance");
+}
+
+extern "C" int f2cgt_kmeans_predict(const float* x, const float* centers, int64_t* labels_i64,
+                                    uint8_t* labels_u8, int64_t m, int64_t n, int64_t k, int metric,
+                                    void* stream) {
+  F2CGT_REQUIRE(m >= 0 && n > 0 && k > 0, F2CGT_E_INVALID,
+                "kmeans_predict: need m >= 0, n > 0 centres, k > 0 dimensions");
+  F2CGT_REQUIRE(n <= 65536 && k < (1 << 20), F2CGT_E_UNSUPPORTED, "kmeans_predict: n or k too large");
+  F2CGT_REQUIRE(metric == F2CGT_METRIC_L2 || metric == F2CGT_METRIC_COSINE, F2CGT_E_INVALID,
+                "kmeans_predict: unknown metric %d", metric);
+  F2CGT_REQUIRE(labels_u8 == nullptr || n <= 256, F2CGT_E_INVALID,
+                "kmeans_predict: uint8 labels need n <= 256 centres");
+  if (m == 0) return 0;
+  F2CGT_REQUIRE(x && centers && (labels_i64 || labels_u8), F2CGT_E_INVALID,
+                "kmeans_predict: null buffer");
+  hipStream_t st = as_stream(stream);
+  const int khalf = (int)((k + 1) / 2);
+  int kh = pow2_ceil(khalf);
+  if (kh < 4) kh = 4;
+  const int n_pad = (int)ceil_div(n, 32) * 32;
+  const size_t lds = ((size_t)2 * kh * n_pad + 2 * (size_t)n_pad + 4) * sizeof(float);
+  if (kh <= 32 && lds <= 96 * 1024) {
+    switch (kh) {
+      case 4: return launch_mfma<4>(x, centers, labels_i64, labels_u8, m, (int)n, (int)k, metric, n_pad, lds, st);
+      case 8: return launch_mfma<8>(x, centers, labels_i64, labels_u8, m, (int)n, (int)k, metric, n_pad, lds, st);
+      case 16: return launch_mfma<16>(x, centers, labels_i64, labels_u8, m, (int)n, (int)k, metric, n_pad, lds, st);
+      default: return launch_mfma<32>(x, centers, labels_i64, labels_u8, m, (int)n, (int)k, metric, n_pad, lds, st);
+    }
+  }
+  int64_t need = ceil_div(m, 4);
+  int64_t cap = (int64_t)num_cus() * 8;
+  predict_exact_kernel<<<(int)(need < cap ? need : cap), 256, 0, st>>>(x, centers, labels_i64, labels_u8, m,
+                                                                      (int)n, (int)k, metric);
+  return launch_status("kmeans_predict");
+}

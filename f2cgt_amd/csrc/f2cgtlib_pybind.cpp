@@ -1,0 +1,460 @@
+// Python module `F2CGTLib`: the operator surface of the reference's pybind module
+// (src/pybind.cu:7-48: same function names, keyword names, argument order, tensor
+// layouts and return types) on top of the C ABI of libf2cgt_hip.so.
+//
+// This file holds no device code.  It validates arguments (TORCH_CHECK -> RuntimeError
+// where the reference aborts or reads out of bounds), allocates the result with torch,
+// picks up torch's current HIP stream and forwards raw pointers.
+#include <pybind11/pybind11.h>
+#include <torch/extension.h>
+
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include <string>
+
+#include "../../include/f2cgt.h"
+
+namespace py = pybind11;
+
+namespace {
+
+void* current_stream() { return static_cast<void*>(c10::hip::getCurrentHIPStream().stream()); }
+
+void check_rc(int rc, const char* op) {
+  TORCH_CHECK(rc == 0, op, " failed (", rc, "): ", f2cgt_last_error());
+}
+
+torch::Tensor dev_contig(const torch::Tensor& t, const char* name) {
+  TORCH_CHECK(t.defined(), name, " is undefined");
+  TORCH_CHECK(t.device().is_cuda(), name, " must be a GPU tensor");
+  return t.contiguous();
+}
+
+int dtype_tag(const torch::Tensor& t, const char* name) {
+  switch (t.scalar_type()) {
+    case torch::kUInt8: return F2CGT_DT_U8;
+    case torch::kInt8: return F2CGT_DT_I8;
+    case torch::kInt16: return F2CGT_DT_I16;
+    case torch::kInt32: return F2CGT_DT_I32;
+    case torch::kInt64: return F2CGT_DT_I64;
+    case torch::kFloat16: return F2CGT_DT_F16;
+    case torch::kFloat32: return F2CGT_DT_F32;
+    case torch::kFloat64: return F2CGT_DT_F64;
+    default: TORCH_CHECK(false, name, " has an unsupported dtype ", t.scalar_type());
+  }
+  return -1;
+}
+
+// CSC index tensors: int32/int64 go straight through; the narrower integer types the
+// reference also dispatches on (src/common.h:33-53) are widened to int32 first.
+struct Graph {
+  torch::Tensor indptr, indices;
+  int tag;
+  int64_t rows, edges;
+};
+
+Graph graph_of(const torch::Tensor& indptr_in, const torch::Tensor& indices_in) {
+  Graph g;
+  g.indptr = dev_contig(indptr_in, "indptr");
+  g.indices = dev_contig(indices_in, "indices");
+  TORCH_CHECK(g.indptr.dim() == 1 && g.indptr.numel() >= 1, "indptr must be 1-D with at least one entry");
+  TORCH_CHECK(g.indices.dim() == 1, "indices must be 1-D");
+  TORCH_CHECK(g.indptr.scalar_type() == g.indices.scalar_type(),
+              "indptr and indices must share one integer dtype");
+  auto st = g.indptr.scalar_type();
+  TORCH_CHECK(st == torch::kInt64 || st == torch::kInt32 || st == torch::kInt16 || st == torch::kInt8 ||
+                  st == torch::kUInt8,
+              "indptr/indices must be int64, int32, int16, int8 or uint8");
+  if (st != torch::kInt64 && st != torch::kInt32) {
+    g.indptr = g.indptr.to(torch::kInt32);
+    g.indices = g.indices.to(torch::kInt32);
+  }
+  g.tag = g.indptr.scalar_type() == torch::kInt64 ? F2CGT_DT_I64 : F2CGT_DT_I32;
+  g.rows = g.indptr.numel() - 1;
+  g.edges = g.indices.numel();
+  return g;
+}
+
+torch::Tensor empty_f32(std::initializer_list<int64_t> shape, const torch::Tensor& like) {
+  return torch::empty(shape, torch::TensorOptions().dtype(torch::kFloat32).device(like.device()));
+}
+
+int metric_tag(const std::string& metric) {
+  // "cosine" selects cosine; every other string selects squared L2 (src/kmeans.cu:108-112).
+  return metric == "cosine" ? F2CGT_METRIC_COSINE : F2CGT_METRIC_L2;
+}
+
+// ---- reference operator surface -----------------------------------------------------
+
+torch::Tensor packbits(torch::Tensor unpack, int64_t target_bits) {
+  unpack = dev_contig(unpack, "unpack");
+  TORCH_CHECK(unpack.dim() == 2, "unpack must be 2-D");
+  TORCH_CHECK(unpack.scalar_type() == torch::kUInt8 || unpack.scalar_type() == torch::kInt8,
+              "unpack must be uint8");
+  TORCH_CHECK(target_bits == 1 || target_bits == 2 || target_bits == 4,
+              "packbits: target_bits must be 1, 2 or 4");
+  c10::DeviceGuard guard(unpack.device());
+  const int64_t per = 8 / target_bits;
+  const int64_t pack_dim = (unpack.size(1) + per - 1) / per;
+  auto pack = torch::empty({unpack.size(0), pack_dim},
+                           torch::TensorOptions().dtype(torch::kUInt8).device(unpack.device()));
+  check_rc(f2cgt_packbits(static_cast<const uint8_t*>(unpack.data_ptr()),
+                          static_cast<uint8_t*>(pack.data_ptr()), unpack.size(0), unpack.size(1),
+                          (int)target_bits, current_stream()),
+           "packbits");
+  return pack;
+}
+
+torch::Tensor unpackbits(torch::Tensor pack, int64_t target_bits, int64_t unpack_dim) {
+  pack = dev_contig(pack, "pack");
+  TORCH_CHECK(pack.dim() == 2, "pack must be 2-D");
+  TORCH_CHECK(pack.scalar_type() == torch::kUInt8 || pack.scalar_type() == torch::kInt8,
+              "pack must be uint8");
+  TORCH_CHECK(target_bits == 1 || target_bits == 2 || target_bits == 4,
+              "unpackbits: target_bits must be 1, 2 or 4");
+  TORCH_CHECK(unpack_dim >= 0 && unpack_dim <= pack.size(1) * (8 / target_bits),
+              "unpackbits: unpack_dim does not fit the packed row");
+  c10::DeviceGuard guard(pack.device());
+  auto unpack = torch::empty({pack.size(0), unpack_dim},
+                             torch::TensorOptions().dtype(torch::kUInt8).device(pack.device()));
+  check_rc(f2cgt_unpackbits(static_cast<const uint8_t*>(pack.data_ptr()),
+                            static_cast<uint8_t*>(unpack.data_ptr()), pack.size(0), pack.size(1),
+                            unpack_dim, (int)target_bits, current_stream()),
+           "unpackbits");
+  return unpack;
+}
+
+torch::Tensor sq_codebooks_checked(torch::Tensor codebooks) {
+  codebooks = dev_contig(codebooks, "codebooks");
+  TORCH_CHECK(codebooks.scalar_type() == torch::kFloat32, "codebooks must be float32");
+  TORCH_CHECK(codebooks.dim() == 2 && codebooks.size(1) == 5 && codebooks.size(0) >= 1,
+              "SQ codebooks must be [n_codebooks, 5] = fmin,fmax,emin,emax,mean");
+  return codebooks;
+}
+
+torch::Tensor sq_compress(torch::Tensor src, torch::Tensor codebooks, int64_t target_bits,
+                          int64_t column_slice) {
+  src = dev_contig(src, "src");
+  TORCH_CHECK(src.dim() == 2 && src.scalar_type() == torch::kFloat32, "src must be float32 [rows, feat_dim]");
+  codebooks = sq_codebooks_checked(codebooks);
+  c10::DeviceGuard guard(src.device());
+  auto out = torch::empty_like(src);
+  check_rc(f2cgt_sq_compress(src.data_ptr<float>(), out.data_ptr<float>(), codebooks.data_ptr<float>(),
+                             src.size(0), src.size(1), codebooks.size(0), (int)target_bits, column_slice,
+                             current_stream()),
+           "sq_compress");
+  return out;
+}
+
+torch::Tensor sq_decompress(torch::Tensor compress_data, torch::Tensor codebooks, int64_t target_bits,
+                            int64_t column_slice, int64_t feat_dim) {
+  compress_data = dev_contig(compress_data, "compress_data");
+  TORCH_CHECK(compress_data.dim() == 2, "compress_data must be 2-D");
+  codebooks = sq_codebooks_checked(codebooks);
+  c10::DeviceGuard guard(compress_data.device());
+  auto out = empty_f32({compress_data.size(0), feat_dim}, compress_data);
+  check_rc(f2cgt_sq_decompress(compress_data.data_ptr(), dtype_tag(compress_data, "compress_data"),
+                               out.data_ptr<float>(), codebooks.data_ptr<float>(), compress_data.size(0),
+                               compress_data.size(1), feat_dim, codebooks.size(0), (int)target_bits,
+                               column_slice, current_stream()),
+           "sq_decompress");
+  return out;
+}
+
+torch::Tensor vq_decompress(torch::Tensor index_tensor, torch::Tensor codebooks, int64_t feat_dim) {
+  index_tensor = dev_contig(index_tensor, "index_tensor");
+  codebooks = dev_contig(codebooks, "codebooks");
+  TORCH_CHECK(index_tensor.dim() == 2, "index_tensor must be [rows, n_codebooks]");
+  TORCH_CHECK(codebooks.dim() == 3, "VQ codebooks must be [n_codebooks, K, width]");
+  TORCH_CHECK(index_tensor.size(1) == codebooks.size(0), "index_tensor has ", index_tensor.size(1),
+              " columns but there are ", codebooks.size(0), " codebooks");
+  c10::DeviceGuard guard(index_tensor.device());
+  auto out = empty_f32({index_tensor.size(0), feat_dim}, index_tensor);
+  check_rc(f2cgt_vq_decompress(index_tensor.data_ptr(), dtype_tag(index_tensor, "index_tensor"),
+                               codebooks.data_ptr(), dtype_tag(codebooks, "codebooks"),
+                               out.data_ptr<float>(), index_tensor.size(0), feat_dim, codebooks.size(0),
+                               codebooks.size(1), codebooks.size(2), current_stream()),
+           "vq_decompress");
+  return out;
+}
+
+torch::Tensor spmm_csr(torch::Tensor feat, torch::Tensor indptr, torch::Tensor indices) {
+  feat = dev_contig(feat, "feat");
+  TORCH_CHECK(feat.dim() == 2, "feat must be 2-D");
+  Graph g = graph_of(indptr, indices);
+  c10::DeviceGuard guard(feat.device());
+  auto out = torch::empty({g.rows, feat.size(1)}, feat.options());
+  check_rc(f2cgt_spmm_csr(feat.data_ptr(), dtype_tag(feat, "feat"), out.data_ptr(), g.indptr.data_ptr(),
+                          g.indices.data_ptr(), g.tag, g.rows, g.edges, feat.size(0), feat.size(1),
+                          current_stream()),
+           "spmm_csr");
+  return out;
+}
+
+torch::Tensor vq_decompress_spmm_csr(torch::Tensor compress_feat, torch::Tensor codebooks,
+                                     torch::Tensor indptr, torch::Tensor indices, int64_t feat_dim) {
+  compress_feat = dev_contig(compress_feat, "compress_feat");
+  codebooks = dev_contig(codebooks, "codebooks");
+  TORCH_CHECK(compress_feat.dim() == 2, "compress_feat must be [rows, n_codebooks]");
+  TORCH_CHECK(codebooks.dim() == 3 && codebooks.scalar_type() == torch::kFloat32,
+              "VQ codebooks must be float32 [n_codebooks, K, width]");
+  TORCH_CHECK(compress_feat.size(1) == codebooks.size(0), "compress_feat has ", compress_feat.size(1),
+              " columns but there are ", codebooks.size(0), " codebooks");
+  Graph g = graph_of(indptr, indices);
+  c10::DeviceGuard guard(compress_feat.device());
+  auto out = empty_f32({g.rows, feat_dim}, compress_feat);
+  check_rc(f2cgt_vq_decompress_spmm_csr(compress_feat.data_ptr(), dtype_tag(compress_feat, "compress_feat"),
+                                        codebooks.data_ptr<float>(), g.indptr.data_ptr(),
+                                        g.indices.data_ptr(), g.tag, out.data_ptr<float>(), g.rows, g.edges,
+                                        compress_feat.size(0), feat_dim, codebooks.size(0),
+                                        codebooks.size(1), codebooks.size(2), current_stream()),
+           "vq_decompress_spmm_csr");
+  return out;
+}
+
+torch::Tensor sq_decompress_spmm_csr(torch::Tensor compress_feat, torch::Tensor codebooks,
+                                     torch::Tensor indptr, torch::Tensor indices, int64_t target_bit,
+                                     int64_t column_slice, int64_t feat_dim) {
+  compress_feat = dev_contig(compress_feat, "compress_feat");
+  TORCH_CHECK(compress_feat.dim() == 2, "compress_feat must be 2-D");
+  codebooks = sq_codebooks_checked(codebooks);
+  Graph g = graph_of(indptr, indices);
+  c10::DeviceGuard guard(compress_feat.device());
+  auto out = empty_f32({g.rows, feat_dim}, compress_feat);
+  check_rc(f2cgt_sq_decompress_spmm_csr(compress_feat.data_ptr(), dtype_tag(compress_feat, "compress_feat"),
+                                        codebooks.data_ptr<float>(), g.indptr.data_ptr(),
+                                        g.indices.data_ptr(), g.tag, out.data_ptr<float>(), g.rows, g.edges,
+                                        compress_feat.size(0), compress_feat.size(1), feat_dim,
+                                        codebooks.size(0), (int)target_bit, column_slice, current_stream()),
+           "sq_decompress_spmm_csr");
+  return out;
+}
+
+torch::Tensor kmeans_predict_impl(torch::Tensor x, torch::Tensor centers, const std::string& metric,
+                                  bool as_u8) {
+  x = dev_contig(x, "data");
+  centers = dev_contig(centers, "centers");
+  TORCH_CHECK(x.dim() == 2 && centers.dim() == 2 && x.size(1) == centers.size(1),
+              "data [m,k] and centers [n,k] must share k");
+  TORCH_CHECK(x.scalar_type() == torch::kFloat32 && centers.scalar_type() == torch::kFloat32,
+              "data and centers must be float32");
+  c10::DeviceGuard guard(x.device());
+  auto labels = torch::empty({x.size(0)}, torch::TensorOptions()
+                                              .dtype(as_u8 ? torch::kUInt8 : torch::kInt64)
+                                              .device(x.device()));
+  check_rc(f2cgt_kmeans_predict(x.data_ptr<float>(), centers.data_ptr<float>(),
+                                as_u8 ? nullptr : labels.data_ptr<int64_t>(),
+                                as_u8 ? static_cast<uint8_t*>(labels.data_ptr()) : nullptr, x.size(0),
+                                centers.size(0), x.size(1), metric_tag(metric), current_stream()),
+           "kmeans_predict");
+  return labels;
+}
+
+torch::Tensor pairwise_distance(torch::Tensor x, torch::Tensor y, std::string metric) {
+  x = dev_contig(x, "x");
+  y = dev_contig(y, "y");
+  TORCH_CHECK(x.dim() == 2 && y.dim() == 2 && x.size(1) == y.size(1), "x [m,k] and y [n,k] must share k");
+  TORCH_CHECK(x.scalar_type() == torch::kFloat32 && y.scalar_type() == torch::kFloat32,
+              "x and y must be float32");
+  c10::DeviceGuard guard(x.device());
+  auto dist = empty_f32({x.size(0), y.size(0)}, x);
+  check_rc(f2cgt_pairwise_distance(x.data_ptr<float>(), y.data_ptr<float>(), dist.data_ptr<float>(),
+                                   x.size(0), y.size(0), x.size(1), metric_tag(metric), current_stream()),
+           "pairwise_distance");
+  return dist;
+}
+
+// Counterpart of the reference's raft-backed KMeans (src/kmeans.h:13-31, src/kmeans.cu).
+// predict() is the fused MFMA distance + arg-min kernel.  fit() is Lloyd's algorithm on
+// top of it with centres initialised from randomly chosen rows (raft's k-means++ and its
+// RNG stream are not reproduced; fit() is not a bit-parity target).
+class KMeans {
+ public:
+  KMeans(int64_t n_cluster, int64_t feat_dim, std::string metric, int max_iter, double tol, int n_init,
+         double oversampling_factor, int batch_samples, int batch_centroids, bool inertia_check)
+      : metric_(std::move(metric)), max_iter_(max_iter), tol_(tol), n_clusters_(n_cluster) {
+    (void)n_init; (void)oversampling_factor; (void)batch_samples; (void)batch_centroids; (void)inertia_check;
+    TORCH_CHECK(n_cluster > 0 && feat_dim > 0, "KMeans: n_cluster and feat_dim must be positive");
+    centers_ = torch::zeros({n_cluster, feat_dim},
+                            torch::TensorOptions().dtype(torch::kFloat32).device(torch::kCUDA));
+  }
+  KMeans(torch::Tensor centers, std::string metric, int max_iter, double tol, int n_init,
+         double oversampling_factor, int batch_samples, int batch_centroids, bool inertia_check)
+      : metric_(std::move(metric)), max_iter_(max_iter), tol_(tol) {
+    (void)n_init; (void)oversampling_factor; (void)batch_samples; (void)batch_centroids; (void)inertia_check;
+    TORCH_CHECK(centers.device().is_cuda(), "centers must be a CUDA tensor");
+    TORCH_CHECK(centers.dim() == 2 && centers.scalar_type() == torch::kFloat32,
+                "centers must be float32 [n_cluster, feat_dim]");
+    centers_ = centers.contiguous();
+    n_clusters_ = centers.size(0);
+  }
+
+  void fit(torch::Tensor x) {
+    TORCH_CHECK(x.device().is_cuda(), "x must be a CUDA tensor");
+    x = x.contiguous().to(torch::kFloat32);
+    TORCH_CHECK(x.dim() == 2 && x.size(1) == centers_.size(1), "fit: data must be [n, feat_dim]");
+    TORCH_CHECK(x.size(0) >= n_clusters_, "fit: fewer samples than clusters");
+    c10::DeviceGuard guard(x.device());
+    auto pick = torch::randperm(x.size(0), torch::TensorOptions().dtype(torch::kInt64).device(x.device()))
+                    .slice(0, 0, n_clusters_);
+    centers_.copy_(x.index_select(0, pick));
+    auto ones = torch::ones({x.size(0)}, x.options());
+    for (int it = 0; it < max_iter_; ++it) {
+      auto labels = kmeans_predict_impl(x, centers_, metric_, false);
+      auto sums = torch::zeros_like(centers_).index_add_(0, labels, x);
+      auto cnt = torch::zeros({n_clusters_}, x.options()).index_add_(0, labels, ones);
+      auto fresh = sums / cnt.clamp_min(1.0).unsqueeze(1);
+      auto next = torch::where(cnt.unsqueeze(1) > 0, fresh, centers_);
+      const double shift = (next - centers_).pow(2).sum().item<double>();
+      centers_.copy_(next);
+      if (shift < tol_) break;
+    }
+  }
+
+  torch::Tensor predict(torch::Tensor x, bool normalize_weights) {
+    (void)normalize_weights;  // sample weights only scale raft's inertia, never the labels
+    TORCH_CHECK(x.device().is_cuda(), "x must be a CUDA tensor");
+    return kmeans_predict_impl(x, centers_, metric_, false);
+  }
+
+  torch::Tensor get_centers() { return centers_; }
+
+ private:
+  std::string metric_;
+  int max_iter_;
+  double tol_;
+  int64_t n_clusters_;
+  torch::Tensor centers_;
+};
+
+// ---- extensions (not in the reference; defined by the benchmark configurations) -------
+
+torch::Tensor affine_params_checked(torch::Tensor params, int64_t feat_dim) {
+  params = dev_contig(params, "params");
+  TORCH_CHECK(params.scalar_type() == torch::kFloat32 && params.dim() == 2 && params.size(0) == 2 &&
+                  params.size(1) >= feat_dim,
+              "affine params must be float32 [2, >= feat_dim] = (min, scale)");
+  return params;
+}
+
+torch::Tensor sq_affine_decompress(torch::Tensor compress_data, torch::Tensor params, int64_t target_bits,
+                                   int64_t feat_dim) {
+  compress_data = dev_contig(compress_data, "compress_data");
+  TORCH_CHECK(compress_data.dim() == 2 && (compress_data.scalar_type() == torch::kUInt8 ||
+                                           compress_data.scalar_type() == torch::kInt8),
+              "compress_data must be uint8 [rows, src_dim]");
+  params = affine_params_checked(params, feat_dim);
+  c10::DeviceGuard guard(compress_data.device());
+  auto out = empty_f32({compress_data.size(0), feat_dim}, compress_data);
+  check_rc(f2cgt_sq_affine_decompress(static_cast<const uint8_t*>(compress_data.data_ptr()),
+                                      out.data_ptr<float>(), params.data_ptr<float>(), params.size(1),
+                                      compress_data.size(0), compress_data.size(1), feat_dim,
+                                      (int)target_bits, current_stream()),
+           "sq_affine_decompress");
+  return out;
+}
+
+torch::Tensor sq_affine_decompress_spmm_csr(torch::Tensor compress_feat, torch::Tensor params,
+                                            torch::Tensor indptr, torch::Tensor indices,
+                                            int64_t target_bit, int64_t feat_dim) {
+  compress_feat = dev_contig(compress_feat, "compress_feat");
+  TORCH_CHECK(compress_feat.dim() == 2 && (compress_feat.scalar_type() == torch::kUInt8 ||
+                                           compress_feat.scalar_type() == torch::kInt8),
+              "compress_feat must be uint8 [rows, src_dim]");
+  params = affine_params_checked(params, feat_dim);
+  Graph g = graph_of(indptr, indices);
+  c10::DeviceGuard guard(compress_feat.device());
+  auto out = empty_f32({g.rows, feat_dim}, compress_feat);
+  check_rc(f2cgt_sq_affine_decompress_spmm_csr(
+               static_cast<const uint8_t*>(compress_feat.data_ptr()), params.data_ptr<float>(),
+               params.size(1), g.indptr.data_ptr(), g.indices.data_ptr(), g.tag, out.data_ptr<float>(),
+               g.rows, g.edges, compress_feat.size(0), compress_feat.size(1), feat_dim, (int)target_bit,
+               current_stream()),
+           "sq_affine_decompress_spmm_csr");
+  return out;
+}
+
+torch::Tensor hybrid_decompress_spmm_csr(torch::Tensor row_map, torch::Tensor sq_codes,
+                                         torch::Tensor sq_params, torch::Tensor vq_codes,
+                                         torch::Tensor vq_codebooks, torch::Tensor indptr,
+                                         torch::Tensor indices, int64_t feat_dim) {
+  row_map = dev_contig(row_map, "row_map");
+  sq_codes = dev_contig(sq_codes, "sq_codes");
+  vq_codes = dev_contig(vq_codes, "vq_codes");
+  vq_codebooks = dev_contig(vq_codebooks, "vq_codebooks");
+  TORCH_CHECK(row_map.dim() == 1 && row_map.scalar_type() == torch::kInt32, "row_map must be int32 [n]");
+  TORCH_CHECK(sq_codes.dim() == 2 && sq_codes.scalar_type() == torch::kUInt8 && sq_codes.size(1) == feat_dim,
+              "sq_codes must be uint8 [n_sq, feat_dim]");
+  TORCH_CHECK(vq_codes.dim() == 2 && vq_codes.scalar_type() == torch::kUInt8, "vq_codes must be uint8 [n_vq, n_codebooks]");
+  TORCH_CHECK(vq_codebooks.dim() == 3 && vq_codebooks.scalar_type() == torch::kFloat32 &&
+                  vq_codebooks.size(0) == vq_codes.size(1),
+              "vq_codebooks must be float32 [n_codebooks, K, width]");
+  sq_params = affine_params_checked(sq_params, feat_dim);
+  Graph g = graph_of(indptr, indices);
+  c10::DeviceGuard guard(row_map.device());
+  auto out = empty_f32({g.rows, feat_dim}, row_map);
+  check_rc(f2cgt_hybrid_decompress_spmm_csr(
+               row_map.data_ptr<int32_t>(), static_cast<const uint8_t*>(sq_codes.data_ptr()),
+               sq_params.data_ptr<float>(), sq_params.size(1),
+               static_cast<const uint8_t*>(vq_codes.data_ptr()), vq_codebooks.data_ptr<float>(),
+               g.indptr.data_ptr(), g.indices.data_ptr(), g.tag, out.data_ptr<float>(), g.rows, g.edges,
+               row_map.numel(), sq_codes.size(0), vq_codes.size(0), feat_dim, vq_codebooks.size(0),
+               vq_codebooks.size(1), vq_codebooks.size(2), current_stream()),
+           "hybrid_decompress_spmm_csr");
+  return out;
+}
+
+torch::Tensor kmeans_predict(torch::Tensor x, torch::Tensor centers, std::string metric) {
+  return kmeans_predict_impl(x, centers, metric, false);
+}
+
+torch::Tensor vq_encode(torch::Tensor x, torch::Tensor centers, std::string metric) {
+  return kmeans_predict_impl(x, centers, metric, true);
+}
+
+}  // namespace
+
+PYBIND11_MODULE(F2CGTLib, m) {
+  m.doc() = "MI355X-native drop-in for F2CGT's F2CGTLib operator module";
+  m.def("packbits", &packbits, py::arg("unpack"), py::arg("target_bits"))
+      .def("unpackbits", &unpackbits, py::arg("pack"), py::arg("target_bits"), py::arg("unpack_dim"))
+      .def("sq_compress", &sq_compress, py::arg("src"), py::arg("codebooks"), py::arg("target_bits"),
+           py::arg("column_slice"))
+      .def("sq_decompress", &sq_decompress, py::arg("compress_data"), py::arg("codebooks"),
+           py::arg("target_bits"), py::arg("column_slice"), py::arg("feat_dim"))
+      .def("vq_decompress", &vq_decompress, py::arg("index_tensor"), py::arg("codebooks"),
+           py::arg("feat_dim"))
+      .def("pairwise_distance", &pairwise_distance, py::arg("x"), py::arg("y"), py::arg("metric"))
+      .def("spmm_csr", &spmm_csr, py::arg("feat"), py::arg("indptr"), py::arg("indices"))
+      .def("vq_decompress_spmm_csr", &vq_decompress_spmm_csr, py::arg("compress_feat"),
+           py::arg("codebooks"), py::arg("indptr"), py::arg("indices"), py::arg("feat_dim"))
+      .def("sq_decompress_spmm_csr", &sq_decompress_spmm_csr, py::arg("compress_feat"),
+           py::arg("codebooks"), py::arg("indptr"), py::arg("indices"), py::arg("target_bit"),
+           py::arg("column_slice"), py::arg("feat_dim"));
+  // extensions
+  m.def("sq_affine_decompress", &sq_affine_decompress, py::arg("compress_data"), py::arg("params"),
+        py::arg("target_bits"), py::arg("feat_dim"))
+      .def("sq_affine_decompress_spmm_csr", &sq_affine_decompress_spmm_csr, py::arg("compress_feat"),
+           py::arg("params"), py::arg("indptr"), py::arg("indices"), py::arg("target_bit"),
+           py::arg("feat_dim"))
+      .def("hybrid_decompress_spmm_csr", &hybrid_decompress_spmm_csr, py::arg("row_map"),
+           py::arg("sq_codes"), py::arg("sq_params"), py::arg("vq_codes"), py::arg("vq_codebooks"),
+           py::arg("indptr"), py::arg("indices"), py::arg("feat_dim"))
+      .def("kmeans_predict", &kmeans_predict, py::arg("x"), py::arg("centers"), py::arg("metric"))
+      .def("vq_encode", &vq_encode, py::arg("x"), py::arg("centers"), py::arg("metric"));
+  py::class_<KMeans>(m, "KMeans")
+      .def(py::init<int64_t, int64_t, std::string, int, double, int, double, int, int, bool>(),
+           py::arg("n_cluster"), py::arg("feat_dim"), py::arg("metric"), py::arg("max_iter") = 300,
+           py::arg("tol") = 1e-4, py::arg("n_init") = 1, py::arg("oversampling_factor") = 2.0,
+           py::arg("batch_samples") = 1 << 15, py::arg("batch_centroids") = 0,
+           py::arg("inertia_check") = false)
+      .def(py::init<torch::Tensor, std::string, int, double, int, double, int, int, bool>(),
+           py::arg("centers"), py::arg("metric"), py::arg("max_iter") = 300, py::arg("tol") = 1e-4,
+           py::arg("n_init") = 1, py::arg("oversampling_factor") = 2.0,
+           py::arg("batch_samples") = 1 << 15, py::arg("batch_centroids") = 0,
+           py::arg("inertia_check") = false)
+      .def("fit", &KMeans::fit, py::arg("data"))
+      .def("predict", &KMeans::predict, py::arg("data"), py::arg("normalize_weights") = true)
+      .def("get_centers", &KMeans::get_centers);
+}

@@ -1,0 +1,179 @@
+/*
+ * f2cgt.h — C ABI of libf2cgt_hip.so: hand-written gfx950 (MI355X) kernels for the
+ * fused feature-decompression + neighbour-aggregation path of F2CGT.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer to a dense row-major buffer unless stated;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); every call
+ *     only enqueues work on that stream: no device-wide synchronisation, no host
+ *     read-back, no allocation (outputs are caller-allocated);
+ *   - return value 0 = success, < 0 = rejected arguments (F2CGT_E_*), > 0 = hipError_t
+ *     of a failed launch; f2cgt_last_error() gives the message of the calling thread's
+ *     last failure;
+ *   - dtype arguments take the F2CGT_DT_* tags below;
+ *   - CSC = indptr[num_rows + 1], indices[num_edges], both of `idx_dtype`
+ *     (F2CGT_DT_I32 or F2CGT_DT_I64).  Source ids are clamped to [0, num_src_rows) and
+ *     edge offsets to [0, num_edges], so malformed graphs give wrong sums, not faults.
+ *
+ * Each entry point names the reference interface (file:line under the reference
+ * checkout) whose device work it replaces.
+ */
+#ifndef F2CGT_H_
+#define F2CGT_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  F2CGT_DT_U8 = 0,
+  F2CGT_DT_I8 = 1,
+  F2CGT_DT_I16 = 2,
+  F2CGT_DT_I32 = 3,
+  F2CGT_DT_I64 = 4,
+  F2CGT_DT_F16 = 5,
+  F2CGT_DT_F32 = 6,
+  F2CGT_DT_F64 = 7
+};
+
+enum {
+  F2CGT_OK = 0,
+  F2CGT_E_INVALID = -1,     /* bad size / null pointer / misaligned buffer */
+  F2CGT_E_UNSUPPORTED = -2, /* dtype, target_bits or shape the kernels do not cover */
+  F2CGT_E_DEVICE = -3       /* no usable gfx950 device */
+};
+
+enum { F2CGT_METRIC_L2 = 0, F2CGT_METRIC_COSINE = 1 };
+
+/* Library version (major * 100 + minor). */
+int f2cgt_version(void);
+
+/* Message of the calling thread's most recent failure ("" if none). */
+const char* f2cgt_last_error(void);
+
+/* Number of compute units of the current device (the kernels size their grids by it). */
+int f2cgt_num_cus(void);
+
+/* ---- bit packing ------------------------------------------------------------- */
+
+/* Replaces packbits(), src/packbits.cu:44-64 (kernel :6-42).
+ * unpack uint8 [rows, unpack_dim] -> pack uint8 [rows, ceil(unpack_dim / (8/bits))];
+ * element i of a group goes to bits [bits*i, bits*(i+1)); target_bits in {1,2,4}. */
+int f2cgt_packbits(const uint8_t* unpack, uint8_t* pack, int64_t rows, int64_t unpack_dim,
+                   int target_bits, void* stream);
+
+/* Replaces unpackbits(), src/packbits.cu:96-114 (kernel :66-94).
+ * pack uint8 [rows, pack_dim] -> unpack uint8 [rows, unpack_dim]. */
+int f2cgt_unpackbits(const uint8_t* pack, uint8_t* unpack, int64_t rows, int64_t pack_dim,
+                     int64_t unpack_dim, int target_bits, void* stream);
+
+/* ---- scalar quantisation (log domain, the reference's SQ) ---------------------- */
+
+/* Replaces sq_compress(), src/sq_quantization.cu:65-83 (kernel :5-63).
+ * src fp32 [rows, feat_dim] -> dst fp32 [rows, feat_dim] of integer-valued codes;
+ * codebooks fp32 [num_codebooks, 5] = fmin,fmax,emin,emax,mean; column j uses
+ * codebook j / column_slice; target_bits in {1,2,4,8,16}. */
+int f2cgt_sq_compress(const float* src, float* dst, const float* codebooks, int64_t rows,
+                      int64_t feat_dim, int64_t num_codebooks, int target_bits,
+                      int64_t column_slice, void* stream);
+
+/* Replaces sq_decompress(), src/sq_quantization.cu:158-182 (kernel :85-156).
+ * codes [rows, src_dim] of code_dtype (U8/I8 packed bytes for bits < 8, I8/U8 for 8,
+ * I16 for 16) -> out fp32 [rows, feat_dim].  Codebook per OUTPUT column. */
+int f2cgt_sq_decompress(const void* codes, int code_dtype, float* out, const float* codebooks,
+                        int64_t rows, int64_t src_dim, int64_t feat_dim,
+                        int64_t num_codebooks, int target_bits, int64_t column_slice,
+                        void* stream);
+
+/* Per-column affine SQ decode (no counterpart in the reference; defined by the
+ * benchmark configurations): out[r][c] = params[c] + code * params[feat_dim_stride + c]
+ * with params fp32 [2, param_stride] (row 0 = min, row 1 = scale), unsigned codes,
+ * sub-byte codes packed low bits first; target_bits in {1,2,4,8}. */
+int f2cgt_sq_affine_decompress(const uint8_t* codes, float* out, const float* params,
+                               int64_t param_stride, int64_t rows, int64_t src_dim,
+                               int64_t feat_dim, int target_bits, void* stream);
+
+/* ---- vector quantisation decode ---------------------------------------------- */
+
+/* Replaces vq_decompress(), src/vq_quantization.cu:35-60 (kernel :5-33).
+ * codes [rows, num_codebooks] (U8/I8/I16), codebooks [num_codebooks, K, width]
+ * (F32 or F16) -> out fp32 [rows, feat_dim], feat_dim <= num_codebooks * width. */
+int f2cgt_vq_decompress(const void* codes, int code_dtype, const void* codebooks, int cb_dtype,
+                        float* out, int64_t rows, int64_t feat_dim, int64_t num_codebooks,
+                        int64_t K, int64_t width, void* stream);
+
+/* ---- CSC mean aggregation ---------------------------------------------------- */
+
+/* Replaces SpMMCsr(), src/fusion_spmm.cu:45-70 (kernel :13-43).
+ * feat [num_src_rows, feat_dim] of feat_dtype (F32/F16/F64) -> out same dtype
+ * [num_rows, feat_dim]; out[r] = sum(feat[indices[e]]) / max(deg, 1). */
+int f2cgt_spmm_csr(const void* feat, int feat_dtype, void* out, const void* indptr,
+                   const void* indices, int idx_dtype, int64_t num_rows, int64_t num_edges,
+                   int64_t num_src_rows, int64_t feat_dim, void* stream);
+
+/* Replaces VqDecompressSpMMFusionCsr(), src/fusion_spmm.cu:107-141 (kernel :72-105,
+ * decode src/cuda_utils.cuh:48-58).  fp32 codebooks; out fp32 [num_rows, feat_dim]. */
+int f2cgt_vq_decompress_spmm_csr(const void* codes, int code_dtype, const float* codebooks,
+                                 const void* indptr, const void* indices, int idx_dtype,
+                                 float* out, int64_t num_rows, int64_t num_edges,
+                                 int64_t num_src_rows, int64_t feat_dim,
+                                 int64_t num_codebooks, int64_t K, int64_t width,
+                                 void* stream);
+
+/* Replaces SqDecompressSpMMFusionCsr(), src/fusion_spmm.cu:240-272 (kernel :143-238).
+ * Codebook per PACKED BYTE (:180): requires column_slice % (8/bits) == 0. */
+int f2cgt_sq_decompress_spmm_csr(const void* codes, int code_dtype, const float* codebooks,
+                                 const void* indptr, const void* indices, int idx_dtype,
+                                 float* out, int64_t num_rows, int64_t num_edges,
+                                 int64_t num_src_rows, int64_t src_dim, int64_t feat_dim,
+                                 int64_t num_codebooks, int target_bits, int64_t column_slice,
+                                 void* stream);
+
+/* Fused per-column affine SQ decode + mean aggregation (benchmark-defined extension;
+ * argument order follows f2cgt_sq_decompress_spmm_csr). */
+int f2cgt_sq_affine_decompress_spmm_csr(const uint8_t* codes, const float* params,
+                                        int64_t param_stride, const void* indptr,
+                                        const void* indices, int idx_dtype, float* out,
+                                        int64_t num_rows, int64_t num_edges,
+                                        int64_t num_src_rows, int64_t src_dim,
+                                        int64_t feat_dim, int target_bits, void* stream);
+
+/* Two-table fused decode + mean aggregation (benchmark-defined extension; the reference's
+ * two-level mode, examples/compress.py:39-54,74-106, never mixes tables in one call).
+ * row_map int32 [num_src_rows]: m >= 0 -> row m of the 8-bit affine SQ table
+ * (sq_codes uint8 [num_sq_rows, feat_dim], sq_params fp32 [2, param_stride]);
+ * m < 0 -> row -m-1 of the VQ table (vq_codes uint8 [num_vq_rows, num_codebooks],
+ * vq_codebooks fp32 [num_codebooks, K, width]). */
+int f2cgt_hybrid_decompress_spmm_csr(const int32_t* row_map, const uint8_t* sq_codes,
+                                     const float* sq_params, int64_t param_stride,
+                                     const uint8_t* vq_codes, const float* vq_codebooks,
+                                     const void* indptr, const void* indices, int idx_dtype,
+                                     float* out, int64_t num_rows, int64_t num_edges,
+                                     int64_t num_src_rows, int64_t num_sq_rows,
+                                     int64_t num_vq_rows, int64_t feat_dim,
+                                     int64_t num_codebooks, int64_t K, int64_t width,
+                                     void* stream);
+
+/* ---- VQ encode ---------------------------------------------------------------- */
+
+/* Replaces pairwise_distance(), src/kmeans.cu:102-118 (raft L2Unexpanded /
+ * CosineExpanded).  x fp32 [m,k], y fp32 [n,k] -> dist fp32 [m,n]; metric L2 is the
+ * squared distance sum((x-y)^2). */
+int f2cgt_pairwise_distance(const float* x, const float* y, float* dist, int64_t m, int64_t n,
+                            int64_t k, int metric, void* stream);
+
+/* Replaces KMeans::predict(), src/kmeans.cu:77-98 (raft kmeans_predict) and the argmin
+ * the callers run on pairwise_distance (examples/my_kmeans.py:116-125).
+ * x fp32 [m,k], centers fp32 [n,k], n <= 65536.  Writes the index of the nearest centre
+ * (first minimum) to labels_i64 [m] and/or labels_u8 [m] (either may be NULL; labels_u8
+ * needs n <= 256).  The distance matrix is never materialised. */
+int f2cgt_kmeans_predict(const float* x, const float* centers, int64_t* labels_i64,
+                         uint8_t* labels_u8, int64_t m, int64_t n, int64_t k, int metric,
+                         void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* F2CGT_H_ */

@@ -1,0 +1,154 @@
+"""CPU-side checks of the product: the C-ABI library loads and exports every symbol that
+include/f2cgt.h declares, argument validation rejects bad calls before any device work,
+the pybind module exposes the reference's operator surface, and the synthetic workload
+generators have the stated statistics.  No kernel is launched here."""
+import ctypes
+import inspect
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import f2cgt_amd
+from f2cgt_amd import capi, synth
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "f2cgt.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(f2cgt_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert len(names) >= 16
+    handle = ctypes.CDLL(f2cgt_amd.capi_path())
+    for name in names:
+        assert hasattr(handle, name), name
+    assert set(names) == set(capi.SIGNATURES), "ctypes binding and header disagree"
+    assert capi.lib().f2cgt_version() >= 100
+
+
+def test_validation_rejects_before_device_work():
+    lib = capi.lib()
+    E_INVALID, E_UNSUPPORTED = -1, -2
+    assert lib.f2cgt_packbits(None, None, 4, 4, 3, None) == E_UNSUPPORTED
+    assert b"target_bits" in lib.f2cgt_last_error()
+    assert lib.f2cgt_packbits(None, None, -1, 4, 4, None) == E_INVALID
+    assert lib.f2cgt_packbits(None, None, 4, 4, 4, None) == E_INVALID  # null buffers
+    assert lib.f2cgt_packbits(None, None, 0, 4, 4, None) == 0          # empty: nothing to do
+    assert lib.f2cgt_unpackbits(None, None, 4, 2, 9, 2, None) == E_INVALID  # 9 > 2*4 codes
+    assert lib.f2cgt_sq_compress(None, None, None, 4, 100, 1, 4, 60, None) == E_INVALID  # codebooks do not cover
+    assert lib.f2cgt_sq_decompress(None, capi.DT_I16, None, None, 4, 50, 100, 1, 4, 100, None) == E_UNSUPPORTED
+    assert lib.f2cgt_sq_decompress(None, capi.DT_U8, None, None, 4, 40, 100, 1, 4, 100, None) == E_INVALID
+    assert lib.f2cgt_vq_decompress(None, capi.DT_U8, None, capi.DT_F64, None, 4, 8, 1, 256, 8, None) == E_UNSUPPORTED
+    assert lib.f2cgt_vq_decompress(None, capi.DT_U8, None, capi.DT_F32, None, 4, 9, 1, 256, 8, None) == E_INVALID
+    assert lib.f2cgt_spmm_csr(None, capi.DT_F32, None, None, None, capi.DT_I16, 1, 0, 1, 4, None) == E_UNSUPPORTED
+    # column_slice must be a multiple of the codes per byte in the fused SQ op
+    assert lib.f2cgt_sq_decompress_spmm_csr(None, capi.DT_U8, None, ctypes.c_void_p(8), None, capi.DT_I64,
+                                            ctypes.c_void_p(8),
+                                            1, 0, 1, 50, 100, 34, 4, 3, None) == E_INVALID
+    assert b"multiple" in lib.f2cgt_last_error()
+    assert lib.f2cgt_kmeans_predict(None, None, None, None, 5, 300, 8, 0, ctypes.c_void_p(0)) == E_INVALID
+    assert lib.f2cgt_pairwise_distance(None, None, None, 5, 3, 8, 7, None) == E_INVALID
+
+
+def test_extension_module_surface_matches_reference():
+    lib = f2cgt_amd.load()
+    import F2CGTLib  # registered under the reference's module name
+
+    assert F2CGTLib is lib
+    expected = {  # src/pybind.cu:8-28
+        "packbits": ["unpack", "target_bits"],
+        "unpackbits": ["pack", "target_bits", "unpack_dim"],
+        "sq_compress": ["src", "codebooks", "target_bits", "column_slice"],
+        "sq_decompress": ["compress_data", "codebooks", "target_bits", "column_slice", "feat_dim"],
+        "vq_decompress": ["index_tensor", "codebooks", "feat_dim"],
+        "pairwise_distance": ["x", "y", "metric"],
+        "spmm_csr": ["feat", "indptr", "indices"],
+        "vq_decompress_spmm_csr": ["compress_feat", "codebooks", "indptr", "indices", "feat_dim"],
+        "sq_decompress_spmm_csr": ["compress_feat", "codebooks", "indptr", "indices", "target_bit",
+                                   "column_slice", "feat_dim"],
+    }
+    for name, args in expected.items():
+        doc = getattr(lib, name).__doc__
+        sig = doc.split("\n")[0]
+        got = re.findall(r"(\w+): ", sig)
+        assert got == args, (name, sig)
+    km = lib.KMeans
+    for method in ("fit", "predict", "get_centers"):
+        assert hasattr(km, method)
+    assert "normalize_weights: bool = True" in km.predict.__doc__
+    init_doc = km.__init__.__doc__
+    kw = re.findall(r"(\w+): ", init_doc)
+    common = ["max_iter", "tol", "n_init", "oversampling_factor", "batch_samples", "batch_centroids",
+              "inertia_check"]
+    assert kw == ["self", "n_cluster", "feat_dim", "metric"] + common + ["self", "centers", "metric"] + common
+    for default in ("= 300", "= 0.0001", "= 1,", "= 2.0", "= 32768", "= 0,", "= False"):
+        assert init_doc.count(default) == 2, default
+
+
+def test_extension_rejects_cpu_tensors_and_bad_shapes():
+    lib = f2cgt_amd.load()
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        lib.packbits(torch.zeros(2, 4, dtype=torch.uint8), 4)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        lib.spmm_csr(torch.zeros(2, 4), torch.zeros(3, dtype=torch.int64), torch.zeros(0, dtype=torch.int64))
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        lib.KMeans(torch.zeros(4, 4), "l2")
+
+
+def test_no_cpu_fallback_in_product():
+    # the product must not import the oracle or carry a CPU path
+    for name in os.listdir(os.path.join(ROOT, "f2cgt_amd")):
+        if name.endswith(".py"):
+            text = open(os.path.join(ROOT, "f2cgt_amd", name)).read()
+            assert "oracle" not in text.replace("no CPU fallback", ""), name
+
+
+# ---- synthetic generators ------------------------------------------------------------------
+def test_powerlaw_degree_mean_and_cap():
+    g = torch.Generator().manual_seed(0)
+    deg = synth.powerlaw_degrees(400_000, 2.1, 12, g, "cpu")
+    assert deg.min() == 1 and deg.max() == 12
+    assert abs(deg.double().mean().item() - 2.2396) < 0.02
+    frac1 = (deg == 1).double().mean().item()
+    assert abs(frac1 - 1 / 1.5602) < 0.01  # P(1) = 1/zeta(2.1)
+
+
+def test_zipf_sampler_follows_power_law():
+    g = torch.Generator().manual_seed(1)
+    ids = synth.zipf_ids(1_000_000, (2_000_000,), 1.1, g, "cpu")
+    assert ids.min() == 0 and ids.max() < 1_000_000
+    counts = torch.bincount(ids, minlength=1_000_000).double()
+    # mass of [2^k - 1, 2^(k+1) - 1) under x^-s on [1, n+1): ratio of consecutive octaves = 2^(1-s)
+    oct_mass = [counts[2 ** k - 1:2 ** (k + 1) - 1].sum().item() for k in range(2, 12)]
+    ratios = np.array(oct_mass[1:]) / np.array(oct_mass[:-1])
+    assert np.allclose(ratios, 2 ** (1 - 1.1), rtol=0.03)
+
+
+def test_pack_low_first_matches_oracle_packing():
+    import f2cgt_oracle as oc
+    rng = np.random.default_rng(0)
+    for bits, d in ((4, 100), (4, 13), (2, 7), (1, 9)):
+        codes = rng.integers(0, 1 << bits, size=(11, d), dtype=np.uint8)
+        got = synth.pack_low_first(torch.from_numpy(codes), bits).numpy()
+        assert np.array_equal(got, oc.packbits(codes, bits))
+
+
+def test_small_workloads_are_consistent():
+    import f2cgt_oracle as oc
+    wl = synth.c2_sq4_affine(N=5000, R=700, chunk=2048)
+    assert wl["codes"].shape == (5000, 50) and wl["indices"].numel() == wl["E"]
+    assert int(wl["indptr"][-1]) == wl["E"] and wl["indices"].max() < 5000
+    dec = oc.sq_affine_decompress(wl["codes"].numpy(), wl["params"].numpy(), 4, 100)
+    assert np.isfinite(dec).all()
+    wl4 = synth.c4_hybrid(N=4000, R=300)
+    m = wl4["row_map"].numpy()
+    assert (m[:200] == np.arange(200)).all() and m[200] == -1 and m[-1] == -(4000 - 200)
+    assert wl4["sq_codes"].shape[0] == 200 and wl4["vq_codes"].shape[0] == 3800
+    assert 0 < wl4["hot_edges"] <= wl4["E"]

@@ -1,0 +1,456 @@
+"""Parity of the HIP library (through the C ABI, and through the F2CGTLib module) with
+the CPU oracle on seeded inputs.  Integer/byte results and decodes are bit-exact;
+aggregations use rtol 1e-5 (they are bit-exact too wherever the kernel keeps the
+sequential edge order, which is asserted where it holds)."""
+import numpy as np
+import pytest
+import torch
+
+import f2cgt_oracle as oc
+from f2cgt_amd import capi
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-5
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def random_graph(rng, rows, n_src, max_deg, idx=np.int64, empty_rows=True):
+    deg = rng.integers(0 if empty_rows else 1, max_deg + 1, size=rows)
+    indptr = np.zeros(rows + 1, dtype=idx)
+    indptr[1:] = np.cumsum(deg)
+    indices = rng.integers(0, n_src, size=int(indptr[-1])).astype(idx)
+    return indptr, indices
+
+
+def close(got, want, atol_scale=1.0):
+    scale = float(np.abs(want).max()) if want.size else 1.0
+    return np.allclose(got, want, rtol=RTOL, atol=RTOL * scale * atol_scale)
+
+
+# ---- golden fixtures ----------------------------------------------------------------------
+def test_golden_fixtures(golden):
+    g = golden
+    for bits in (1, 2, 4):
+        assert np.array_equal(host(capi.packbits(dev(g["pack%d_in" % bits]), bits)), g["pack%d_out" % bits])
+        assert np.array_equal(host(capi.unpackbits(dev(g["pack%d_out" % bits]), bits, 13)),
+                              g["unpack%d_out" % bits])
+    cbs = dev(g["sq_codebooks"])
+    ip, ix = dev(g["g_indptr"]), dev(g["g_indices"])
+    for bits in (1, 2, 4, 8, 16):
+        assert np.array_equal(host(capi.sq_compress(dev(g["sq_x"]), cbs, bits, 12)), g["sq%d_codes" % bits])
+        store = dev(g["sq%d_store" % bits])
+        assert np.array_equal(host(capi.sq_decompress(store, cbs, bits, 12, 24)), g["sq%d_decoded" % bits])
+        fused = host(capi.sq_decompress_spmm_csr(store[:3].contiguous(), cbs, ip, ix, bits, 12, 24))
+        assert np.array_equal(fused, g["g_sq%d_fused" % bits])
+    assert np.array_equal(host(capi.vq_decompress(dev(g["vq_idx"]), dev(g["vq_codebooks"]), 10)), g["vq_decoded"])
+    assert np.array_equal(host(capi.vq_decompress_spmm_csr(dev(g["vq_idx"]), dev(g["vq_codebooks"]), ip, ix, 10)),
+                          g["g_vq_fused"])
+    assert np.array_equal(host(capi.spmm_csr(dev(g["g_feat"]), ip, ix)), g["g_spmm"])
+    for bits in (4, 8):
+        store, params = dev(g["aff%d_store" % bits]), dev(g["aff%d_params" % bits])
+        assert np.array_equal(host(capi.sq_affine_decompress(store, params, bits, 10)), g["aff%d_decoded" % bits])
+        assert np.array_equal(host(capi.sq_affine_decompress_spmm_csr(store, params, ip, ix, bits, 10)),
+                              g["g_aff%d_fused" % bits])
+    hy = host(capi.hybrid_decompress_spmm_csr(dev(g["hy_map"]), dev(g["hy_sq"]), dev(g["hy_params"]),
+                                              dev(g["hy_vq"]), dev(g["hy_cb"]), dev(g["hy_indptr"]),
+                                              dev(g["hy_indices"]), 8))
+    assert np.array_equal(hy, g["hy_fused"])
+    for metric in ("l2", "cosine"):
+        d = host(capi.pairwise_distance(dev(g["enc_x"]), dev(g["enc_c"]), metric))
+        assert np.allclose(d, g["enc_dist_" + metric], rtol=1e-5, atol=1e-5)
+        assert np.array_equal(host(capi.kmeans_predict(dev(g["enc_x"]), dev(g["enc_c"]), metric)),
+                              g["enc_labels_" + metric])
+
+
+# ---- packbits / unpackbits -------------------------------------------------------------------
+@pytest.mark.parametrize("bits", [1, 2, 4])
+@pytest.mark.parametrize("shape", [(0, 8), (1, 1), (3, 13), (257, 100), (1000, 128), (5, 1031), (4099, 50)])
+def test_pack_unpack_bit_exact(bits, shape):
+    rng = np.random.default_rng(bits * 1000 + shape[0] + shape[1])
+    u = rng.integers(0, 256, size=shape, dtype=np.uint8)
+    want = oc.packbits(u, bits)
+    got = host(capi.packbits(dev(u), bits))
+    assert got.shape == want.shape and np.array_equal(got, want)
+    back = host(capi.unpackbits(dev(want), bits, shape[1]))
+    assert np.array_equal(back, oc.unpackbits(want, bits, shape[1]))
+    assert np.array_equal(back, u & ((1 << bits) - 1))
+
+
+def test_pack_large_roundtrip_property():
+    # C2 table shape: [2.4e6, 100] 4-bit codes -> [2.4e6, 50]
+    g = torch.Generator(device="cuda").manual_seed(0)
+    u = torch.randint(0, 16, (2_400_000, 100), generator=g, device="cuda", dtype=torch.uint8)
+    p = capi.packbits(u, 4)
+    assert p.shape == (2_400_000, 50)
+    assert torch.equal(capi.unpackbits(p, 4, 100), u)
+    assert torch.equal(p, (u[:, 0::2] | (u[:, 1::2] << 4)))
+
+
+# ---- SQ encode / decode ------------------------------------------------------------------------
+@pytest.mark.parametrize("bits", [1, 2, 4, 8, 16])
+def test_sq_compress_decompress_bit_exact(bits):
+    # shapes of tests/test_sq.py: 10000 x 200 single codebook; (60+50) two codebooks
+    rng = np.random.default_rng(bits)
+    x = rng.uniform(-1, 1, size=(10000, 200)).astype(np.float32)
+    x[0, :4] = [0.0, -0.0, 1e-9, 5.0]
+    cb = np.stack([oc.sq_codebook(x)])
+    codes = oc.sq_compress(x, cb, bits, 200)
+    got = host(capi.sq_compress(dev(x), dev(cb), bits, 200))
+    assert np.array_equal(got, codes)
+    store = oc.sq_codes_to_storage(codes, bits)
+    dec = host(capi.sq_decompress(dev(store), dev(cb), bits, 200, 200))
+    assert np.array_equal(dec, oc.sq_decompress(store, cb, bits, 200, 200))
+
+    a = rng.uniform(-1, 1, size=(3000, 60)).astype(np.float32)
+    b = (rng.uniform(-1, 1, size=(3000, 50)) + 10).astype(np.float32)
+    x2 = np.concatenate([a, b], axis=1)
+    cbs = np.stack([oc.sq_codebook(a), oc.sq_codebook(b)])
+    codes2 = oc.sq_compress(x2, cbs, bits, 60)
+    assert np.array_equal(host(capi.sq_compress(dev(x2), dev(cbs), bits, 60)), codes2)
+    store2 = oc.sq_codes_to_storage(codes2, bits)
+    dec2 = host(capi.sq_decompress(dev(store2), dev(cbs), bits, 60, 110))
+    assert np.array_equal(dec2, oc.sq_decompress(store2, cbs, bits, 60, 110))
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8, 16])
+def test_sq_decompress_every_code(bits):
+    n = 1 << bits
+    raw = np.arange(n, dtype=np.int64)
+    cbs = np.array([[0.01, 3.0, np.log2(0.01), np.log2(3.0) + 1e-5, 0.4],
+                    [1e-5, 900.0, np.log2(1e-5), np.log2(900.0), 0.2]], dtype=np.float32)
+    if bits < 8:
+        store = oc.packbits(np.concatenate([raw, raw]).astype(np.uint8)[None, :], bits)
+    elif bits == 8:
+        store = np.concatenate([raw, raw]).astype(np.uint8).view(np.int8)[None, :]
+    else:
+        store = np.concatenate([raw, raw]).astype(np.uint16).view(np.int16)[None, :]
+    want = oc.sq_decompress(store, cbs, bits, n, 2 * n)
+    got = host(capi.sq_decompress(dev(store), dev(cbs), bits, n, 2 * n))
+    assert np.array_equal(got, want)
+    assert np.array_equal(want[0, :n], oc.sq_lut(cbs, bits)[0])
+
+
+def test_sq_decompress_accepts_int8_storage():
+    rng = np.random.default_rng(9)
+    x = rng.uniform(-1, 1, size=(100, 64)).astype(np.float32)
+    cb = np.stack([oc.sq_codebook(x)])
+    store = oc.sq_codes_to_storage(oc.sq_compress(x, cb, 4, 64), 4)
+    a = host(capi.sq_decompress(dev(store), dev(cb), 4, 64, 64))
+    b = host(capi.sq_decompress(dev(store.view(np.int8)), dev(cb), 4, 64, 64))
+    assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("d", [10, 100, 128])
+def test_sq_affine_decompress_bit_exact(bits, d):
+    rng = np.random.default_rng(bits * 10 + d)
+    x = (rng.standard_normal((2000, d)) * rng.uniform(0.5, 2, size=d)).astype(np.float32)
+    params = oc.sq_affine_params(x, bits)
+    codes = oc.sq_affine_compress(x, params, bits)
+    store = oc.packbits(codes, bits) if bits < 8 else codes
+    got = host(capi.sq_affine_decompress(dev(store), dev(params), bits, d))
+    assert np.array_equal(got, oc.sq_affine_decompress(store, params, bits, d))
+
+
+# ---- VQ decode ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("cdt", [np.uint8, np.int8, np.int16])
+@pytest.mark.parametrize("cbdt", [np.float32, np.float16])
+def test_vq_decompress_dtypes(cdt, cbdt):
+    rng = np.random.default_rng(0)
+    K = 100 if cdt == np.int8 else (700 if cdt == np.int16 else 256)
+    cb = rng.standard_normal((4, K, 8)).astype(cbdt)
+    idx = rng.integers(0, K, size=(3000, 4)).astype(cdt)
+    for feat_dim in (32, 27):
+        got = host(capi.vq_decompress(dev(idx), dev(cb), feat_dim))
+        assert np.array_equal(got, oc.vq_decompress(idx, cb, feat_dim))
+
+
+def test_vq_decompress_reference_shapes():
+    # tests/test_vq.py: 1 codebook x 128 wide; (60 | 50 zero padded to 60) two codebooks
+    rng = np.random.default_rng(1)
+    cb = rng.uniform(-5, 5, size=(1, 256, 128)).astype(np.float32)
+    idx = rng.integers(0, 256, size=(100000, 1), dtype=np.uint8)
+    got = capi.vq_decompress(dev(idx), dev(cb), 128)
+    want = torch.index_select(dev(cb[0]), 0, dev(idx[:, 0]).long())
+    assert torch.equal(got, want)
+    cb2 = np.zeros((2, 256, 60), dtype=np.float32)
+    cb2[0] = rng.uniform(-5, 5, size=(256, 60))
+    cb2[1, :, :50] = rng.uniform(-10, 10, size=(256, 50))
+    idx2 = rng.integers(0, 256, size=(50000, 2), dtype=np.uint8)
+    got2 = host(capi.vq_decompress(dev(idx2), dev(cb2), 110))
+    assert np.array_equal(got2, oc.vq_decompress(idx2, cb2, 110))
+
+
+def test_vq_decompress_codebook_larger_than_lds():
+    rng = np.random.default_rng(2)
+    cb = rng.standard_normal((24, 256, 32)).astype(np.float32)  # 768 KB
+    idx = rng.integers(0, 256, size=(2000, 24), dtype=np.uint8)
+    got = host(capi.vq_decompress(dev(idx), dev(cb), 768))
+    assert np.array_equal(got, oc.vq_decompress(idx, cb, 768))
+
+
+# ---- plain CSC mean ---------------------------------------------------------------------------
+@pytest.mark.parametrize("idx", [np.int32, np.int64])
+@pytest.mark.parametrize("d", [1, 7, 100, 128, 300])
+def test_spmm_csr_f32(idx, d):
+    rng = np.random.default_rng(d)
+    feat = rng.standard_normal((1000, d)).astype(np.float32)
+    indptr, indices = random_graph(rng, 700, 1000, 17, idx)
+    got = host(capi.spmm_csr(dev(feat), dev(indptr), dev(indices)))
+    want = oc.spmm_csr(feat, indptr, indices)
+    assert np.array_equal(got, want)  # sequential edge order is kept
+
+
+def test_spmm_csr_f16_f64_and_empty():
+    rng = np.random.default_rng(3)
+    indptr, indices = random_graph(rng, 300, 500, 9)
+    f64 = rng.standard_normal((500, 33))
+    got = host(capi.spmm_csr(dev(f64), dev(indptr), dev(indices)))
+    assert np.array_equal(got, oc.spmm_csr(f64, indptr, indices))
+    f16 = rng.standard_normal((500, 33)).astype(np.float16)
+    got16 = host(capi.spmm_csr(dev(f16), dev(indptr), dev(indices))).astype(np.float32)
+    want16 = oc.spmm_csr(f16.astype(np.float32), indptr, indices)
+    assert np.allclose(got16, want16, rtol=2e-3, atol=2e-3)
+    # no rows, no edges
+    e = capi.spmm_csr(dev(f64.astype(np.float32)), dev(np.zeros(1, np.int64)), dev(np.zeros(0, np.int64)))
+    assert e.shape == (0, 33)
+    z = host(capi.spmm_csr(dev(f64.astype(np.float32)), dev(np.zeros(6, np.int64)), dev(np.zeros(0, np.int64))))
+    assert z.shape == (5, 33) and not z.any()
+
+
+# ---- fused VQ ---------------------------------------------------------------------------------
+def test_fused_vq_reference_literal_case():
+    # tests/test_fusion_decompress_spmm.py:19-33: fused == spmm_csr(vq_decompress(.)), bit for bit
+    rng = np.random.default_rng(4)
+    indptr = dev(np.array([0, 1, 3, 6], dtype=np.int64))
+    indices = dev(np.array([0, 1, 1, 2, 2, 0], dtype=np.int64))
+    cb = dev(rng.standard_normal((1, 256, 100)).astype(np.float32))
+    codes = dev(rng.integers(0, 256, size=(6, 1), dtype=np.uint8))
+    out1 = capi.spmm_csr(capi.vq_decompress(codes, cb, 100), indptr, indices)
+    out2 = capi.vq_decompress_spmm_csr(codes, cb, indptr, indices, 100)
+    assert torch.equal(out1, out2)
+
+
+@pytest.mark.parametrize("idx", [np.int32, np.int64])
+@pytest.mark.parametrize("shape", [(16, 256, 8, 128), (16, 256, 8, 100), (8, 256, 16, 128), (24, 256, 32, 768),
+                                   (3, 16, 4, 10), (1, 256, 100, 100), (5, 64, 6, 29)])
+def test_fused_vq_vs_oracle(idx, shape):
+    n_cb, K, w, feat_dim = shape
+    rng = np.random.default_rng(n_cb * 7 + w)
+    N, R = 5000, 1500
+    cb = rng.standard_normal((n_cb, K, w)).astype(np.float32)
+    codes = rng.integers(0, K, size=(N, n_cb), dtype=np.uint8)
+    indptr, indices = random_graph(rng, R, N, 20, idx)
+    got = host(capi.vq_decompress_spmm_csr(dev(codes), dev(cb), dev(indptr), dev(indices), feat_dim))
+    want = oc.vq_decompress_spmm_csr(codes, cb, indptr, indices, feat_dim)
+    assert close(got, want)
+    unfused = host(capi.spmm_csr(capi.vq_decompress(dev(codes), dev(cb), feat_dim), dev(indptr), dev(indices)))
+    assert close(got, unfused)
+
+
+def test_fused_vq_int16_codes_big_codebook():
+    rng = np.random.default_rng(5)
+    cb = rng.standard_normal((2, 5000, 8)).astype(np.float32)   # 160 KB per slice: global path
+    codes = rng.integers(0, 5000, size=(800, 2)).astype(np.int16)
+    indptr, indices = random_graph(rng, 300, 800, 6)
+    got = host(capi.vq_decompress_spmm_csr(dev(codes), dev(cb), dev(indptr), dev(indices), 16))
+    assert close(got, oc.vq_decompress_spmm_csr(codes, cb, indptr, indices, 16))
+
+
+# ---- fused SQ (log domain) --------------------------------------------------------------------------
+@pytest.mark.parametrize("bits", [1, 2, 4, 8, 16])
+def test_fused_sq_reference_literal_case(bits):
+    # tests/test_fusion_decompress_spmm.py:93-120
+    rng = np.random.default_rng(bits)
+    indptr = dev(np.array([0, 1, 3, 6], dtype=np.int64))
+    indices = dev(np.array([0, 1, 1, 2, 2, 0], dtype=np.int64))
+    x = rng.standard_normal((6, 100)).astype(np.float32)
+    cb = np.stack([oc.sq_codebook(x)])
+    codes = capi.sq_compress(dev(x), dev(cb), bits, 100)
+    if bits < 8:
+        exp = capi.packbits(codes.to(torch.uint8), bits)
+    elif bits == 8:
+        exp = codes.to(torch.int8)
+    else:
+        exp = codes.to(torch.int16)
+    out1 = capi.spmm_csr(capi.sq_decompress(exp, dev(cb), bits, 100, 100), indptr, indices)
+    out2 = capi.sq_decompress_spmm_csr(exp, dev(cb), indptr, indices, bits, 100, 100)
+    assert torch.equal(out1, out2)
+    want = oc.sq_decompress_spmm_csr(host(exp), cb, host(indptr), host(indices), bits, 100, 100)
+    assert np.array_equal(host(out2), want)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("d,cs", [(128, 128), (100, 100), (128, 32), (110, 56), (24, 8)])
+def test_fused_sq_vs_oracle(bits, d, cs):
+    rng = np.random.default_rng(bits * 100 + d)
+    N, R = 3000, 900
+    x = rng.uniform(-1, 1, size=(N, d)).astype(np.float32) * (1 + np.arange(d) // cs)
+    n_cb = (d + cs - 1) // cs
+    cbs = np.stack([oc.sq_codebook(x[:, i * cs:(i + 1) * cs]) for i in range(n_cb)])
+    store = oc.sq_codes_to_storage(oc.sq_compress(x, cbs, bits, cs), bits)
+    indptr, indices = random_graph(rng, R, N, 14, np.int64)
+    got = host(capi.sq_decompress_spmm_csr(dev(store), dev(cbs), dev(indptr), dev(indices), bits, cs, d))
+    want = oc.sq_decompress_spmm_csr(store, cbs, indptr, indices, bits, cs, d)
+    assert np.array_equal(got, want)
+
+
+# ---- fused affine SQ and hybrid ------------------------------------------------------------------------
+@pytest.mark.parametrize("bits,d", [(8, 128), (4, 100), (4, 128), (2, 64), (1, 40), (4, 7), (8, 30)])
+@pytest.mark.parametrize("idx", [np.int32, np.int64])
+def test_fused_affine_vs_oracle(bits, d, idx):
+    rng = np.random.default_rng(bits * 10 + d)
+    N, R = 4000, 1200
+    x = (rng.standard_normal((N, d)) * rng.uniform(0.5, 2, size=d)).astype(np.float32)
+    params = oc.sq_affine_params(x, bits)
+    codes = oc.sq_affine_compress(x, params, bits)
+    store = oc.packbits(codes, bits) if bits < 8 else codes
+    indptr, indices = random_graph(rng, R, N, 12, idx)
+    got = host(capi.sq_affine_decompress_spmm_csr(dev(store), dev(params), dev(indptr), dev(indices), bits, d))
+    want = oc.sq_affine_decompress_spmm_csr(store, params, indptr, indices, bits, d)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("shape", [(8, 256, 16), (16, 256, 8), (4, 64, 5), (3, 64, 100)])
+def test_hybrid_vs_oracle(shape):
+    n_cb, K, w = shape
+    D = n_cb * w
+    rng = np.random.default_rng(n_cb)
+    N, n_hot, R = 6000, 300, 1500
+    row_map = np.empty(N, dtype=np.int32)
+    perm = rng.permutation(N)
+    row_map[perm[:n_hot]] = np.arange(n_hot)
+    row_map[perm[n_hot:]] = -np.arange(N - n_hot) - 1
+    sq = rng.integers(0, 256, size=(n_hot, D), dtype=np.uint8)
+    params = np.stack([rng.standard_normal(D), rng.uniform(0.01, 0.05, D)]).astype(np.float32)
+    vq = rng.integers(0, K, size=(N - n_hot, n_cb), dtype=np.uint8)
+    cb = rng.standard_normal((n_cb, K, w)).astype(np.float32)
+    indptr, indices = random_graph(rng, R, N, 12)
+    hot_ids = perm[:n_hot]
+    # make ~60 % of the edges hit the hot table
+    mask = rng.random(indices.shape[0]) < 0.6
+    indices[mask] = rng.choice(hot_ids, size=int(mask.sum()))
+    got = host(capi.hybrid_decompress_spmm_csr(dev(row_map), dev(sq), dev(params), dev(vq), dev(cb), dev(indptr),
+                                               dev(indices), D))
+    want = oc.hybrid_decompress_spmm_csr(row_map, sq, params, vq, cb, indptr, indices, D)
+    assert np.array_equal(got, want)
+
+
+# ---- encode -------------------------------------------------------------------------------------
+@pytest.mark.parametrize("metric", ["l2", "cosine"])
+@pytest.mark.parametrize("m,n,k", [(1000, 256, 32), (333, 17, 5), (64, 64, 64), (129, 300, 100)])
+def test_pairwise_distance(metric, m, n, k):
+    rng = np.random.default_rng(m + n + k)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    y = rng.standard_normal((n, k)).astype(np.float32)
+    got = host(capi.pairwise_distance(dev(x), dev(y), metric))
+    want = oc.pairwise_distance(x, y, metric, dtype=np.float64)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("metric", ["l2", "cosine"])
+@pytest.mark.parametrize("m,n,k", [(20000, 256, 32), (5000, 256, 8), (3001, 100, 16), (777, 37, 5),
+                                   (4000, 256, 64), (500, 1000, 24), (300, 50, 200)])
+def test_kmeans_predict_vs_oracle(metric, m, n, k):
+    rng = np.random.default_rng(m + n + k)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    c = rng.standard_normal((n, k)).astype(np.float32)
+    want, near = oc.kmeans_predict(x, c, metric)
+    got = host(capi.kmeans_predict(dev(x), dev(c), metric))
+    assert np.array_equal(got[~near], want[~near])
+    assert near.mean() < 0.01
+    if n <= 256:
+        got8 = host(capi.kmeans_predict(dev(x), dev(c), metric, u8=True))
+        assert np.array_equal(got8.astype(np.int64), got)
+
+
+def test_kmeans_predict_exact_ties_pick_first():
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((4000, 32)).astype(np.float32)
+    c = rng.standard_normal((256, 32)).astype(np.float32)
+    c[200] = c[7]
+    c[255] = c[100]
+    got = host(capi.kmeans_predict(dev(x), dev(c), "l2"))
+    want, _ = oc.kmeans_predict(x, c, "l2")
+    assert np.array_equal(got, want)  # fp64 refinement resolves the duplicates to the first index
+    assert not np.isin(got, [200, 255]).any()
+    # data points that ARE centres
+    got_c = host(capi.kmeans_predict(dev(c), dev(c), "l2"))
+    assert np.array_equal(got_c, oc.kmeans_predict(c, c, "l2")[0])
+
+
+# ---- the F2CGTLib module (same kernels through the pybind shim) ------------------------------------
+def test_module_surface_end_to_end():
+    import f2cgt_amd
+
+    lib = f2cgt_amd.load()
+    rng = np.random.default_rng(12)
+    x = rng.uniform(-1, 1, size=(500, 100)).astype(np.float32)
+    cb = np.stack([oc.sq_codebook(x)])
+    indptr, indices = random_graph(rng, 200, 500, 10)
+    ip, ix = dev(indptr), dev(indices)
+    for bits in (1, 2, 4, 8, 16):
+        codes = lib.sq_compress(dev(x), dev(cb), bits, 100)
+        if bits < 8:
+            exp = lib.packbits(codes.to(torch.uint8), bits)
+            assert torch.equal(lib.unpackbits(exp, bits, 100), codes.to(torch.uint8))
+            exp = exp.to(torch.int8)  # packed tables are stored as int8 (examples/process_compress.py:109-141)
+        elif bits == 8:
+            exp = codes.to(torch.int8)
+        else:
+            exp = codes.to(torch.int16)
+        out1 = lib.spmm_csr(lib.sq_decompress(exp, dev(cb), bits, 100, 100), ip, ix)
+        out2 = lib.sq_decompress_spmm_csr(exp, dev(cb), ip, ix, bits, 100, 100)
+        assert torch.equal(out1, out2)
+    # int16 index tensors are accepted like the reference's dispatch
+    out3 = lib.spmm_csr(dev(x), ip.to(torch.int16), ix.to(torch.int16))
+    assert torch.equal(out3, lib.spmm_csr(dev(x), ip, ix))
+    # VQ through KMeans: fit, predict, decode, fused aggregate
+    data = dev(rng.standard_normal((3000, 16)).astype(np.float32))
+    km = lib.KMeans(64, 16, "l2")
+    km.fit(data)
+    centers = km.get_centers()
+    assert centers.shape == (64, 16) and centers.data_ptr() == km.get_centers().data_ptr()
+    labels = km.predict(data)
+    assert labels.dtype == torch.int64 and labels.shape == (3000,)
+    want, near = oc.kmeans_predict(host(data), host(centers), "l2")
+    assert np.array_equal(host(labels)[~near], want[~near])
+    km2 = lib.KMeans(centers, "cosine")
+    lc = km2.predict(data, normalize_weights=False)
+    wc, nearc = oc.kmeans_predict(host(data), host(centers), "cosine")
+    assert np.array_equal(host(lc)[~nearc], wc[~nearc])
+    dist = lib.pairwise_distance(data[:100], centers, "euclidean")
+    assert torch.equal(dist.argmin(dim=1), labels[:100]) or near[:100].any()
+    codes8 = labels.to(torch.uint8).reshape(-1, 1)
+    cbk = centers.reshape(1, 64, 16)
+    ipv, ixv = random_graph(rng, 400, 3000, 15)
+    o1 = lib.spmm_csr(lib.vq_decompress(codes8, cbk, 16), dev(ipv), dev(ixv))
+    o2 = lib.vq_decompress_spmm_csr(codes8, cbk, dev(ipv), dev(ixv), 16)
+    assert torch.equal(o1, o2)
+    with pytest.raises(RuntimeError, match="column_slice"):
+        lib.sq_decompress_spmm_csr(exp, dev(cb), ip, ix, 4, 3, 100)
+    with pytest.raises(RuntimeError):
+        lib.packbits(dev(np.zeros((2, 4), np.uint8)), 3)
+
+
+def test_ops_run_on_the_current_stream():
+    rng = np.random.default_rng(13)
+    cb = dev(rng.standard_normal((16, 256, 8)).astype(np.float32))
+    codes = dev(rng.integers(0, 256, size=(20000, 16), dtype=np.uint8))
+    indptr, indices = random_graph(rng, 5000, 20000, 15)
+    ip, ix = dev(indptr), dev(indices)
+    ref = capi.vq_decompress_spmm_csr(codes, cb, ip, ix, 128)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        out = capi.vq_decompress_spmm_csr(codes, cb, ip, ix, 128)
+    side.synchronize()
+    assert torch.equal(out, ref)
