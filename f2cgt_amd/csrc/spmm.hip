@@ -665,9 +665,6 @@ extern "C" int f2cgt_sq_decompress_spmm_csr(const void* codes, int code_dtype, c
                     target_bits == 16,
                 F2CGT_E_UNSUPPORTED, "%s: target_bit must be 1,2,4,8 or 16 (got %d)", what, target_bits);
   const int per = target_bits < 8 ? 8 / target_bits : 1;
-  F2CGT_REQUIRE(column_slice % per == 0, F2CGT_E_INVALID,
-                "%s: column_slice %lld must be a multiple of %d codes per byte", what,
-                (long long)column_slice, per);
   F2CGT_REQUIRE(num_codebooks * column_slice >= feat_dim, F2CGT_E_INVALID,
                 "%s: %lld codebooks of %lld columns do not cover feat_dim %lld", what,
                 (long long)num_codebooks, (long long)column_slice, (long long)feat_dim);

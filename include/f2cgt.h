@@ -123,7 +123,8 @@ int f2cgt_vq_decompress_spmm_csr(const void* codes, int code_dtype, const float*
                                  void* stream);
 
 /* Replaces SqDecompressSpMMFusionCsr(), src/fusion_spmm.cu:240-272 (kernel :143-238).
- * Codebook per PACKED BYTE (:180): requires column_slice % (8/bits) == 0. */
+ * Codebook per PACKED BYTE (:180): byte j uses codebook j*(8/bits) / column_slice, which
+ * equals the per-column choice of f2cgt_sq_decompress iff column_slice % (8/bits) == 0. */
 int f2cgt_sq_decompress_spmm_csr(const void* codes, int code_dtype, const float* codebooks,
                                  const void* indptr, const void* indices, int idx_dtype,
                                  float* out, int64_t num_rows, int64_t num_edges,

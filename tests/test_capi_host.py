@@ -48,11 +48,11 @@ def test_validation_rejects_before_device_work():
     assert lib.f2cgt_vq_decompress(None, capi.DT_U8, None, capi.DT_F64, None, 4, 8, 1, 256, 8, None) == E_UNSUPPORTED
     assert lib.f2cgt_vq_decompress(None, capi.DT_U8, None, capi.DT_F32, None, 4, 9, 1, 256, 8, None) == E_INVALID
     assert lib.f2cgt_spmm_csr(None, capi.DT_F32, None, None, None, capi.DT_I16, 1, 0, 1, 4, None) == E_UNSUPPORTED
-    # column_slice must be a multiple of the codes per byte in the fused SQ op
+    # column_slice must be positive in the fused SQ op
     assert lib.f2cgt_sq_decompress_spmm_csr(None, capi.DT_U8, None, ctypes.c_void_p(8), None, capi.DT_I64,
                                             ctypes.c_void_p(8),
-                                            1, 0, 1, 50, 100, 34, 4, 3, None) == E_INVALID
-    assert b"multiple" in lib.f2cgt_last_error()
+                                            1, 0, 1, 50, 100, 34, 4, 0, None) == E_INVALID
+    assert b"column_slice" in lib.f2cgt_last_error()
     assert lib.f2cgt_kmeans_predict(None, None, None, None, 5, 300, 8, 0, ctypes.c_void_p(0)) == E_INVALID
     assert lib.f2cgt_pairwise_distance(None, None, None, 5, 3, 8, 7, None) == E_INVALID
 

@@ -436,7 +436,7 @@ def test_module_surface_end_to_end():
     o2 = lib.vq_decompress_spmm_csr(codes8, cbk, dev(ipv), dev(ixv), 16)
     assert torch.equal(o1, o2)
     with pytest.raises(RuntimeError, match="column_slice"):
-        lib.sq_decompress_spmm_csr(exp, dev(cb), ip, ix, 4, 3, 100)
+        lib.sq_decompress_spmm_csr(exp, dev(cb), ip, ix, 4, 0, 100)
     with pytest.raises(RuntimeError):
         lib.packbits(dev(np.zeros((2, 4), np.uint8)), 3)
 
