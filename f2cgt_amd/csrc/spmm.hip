@@ -12,6 +12,7 @@
 // log-domain SQ evaluated directly (16-bit codes), per-column affine SQ, VQ with the
 // codebook window staged in LDS, and the two-table hybrid.
 #include "common.hpp"
+#include "spmm_fast.hpp"
 
 #include <type_traits>
 
@@ -681,6 +682,9 @@ extern "C" int f2cgt_sq_decompress_spmm_csr(const void* codes, int code_dtype, c
   const uint8_t* c8 = static_cast<const uint8_t*>(codes);
   if (target_bits == 16)
     return run_sq_direct<16, uint16_t>(codes, codebooks, indptr, indices, idx_dtype, out, num_rows, num_edges, num_src_rows, src_dim, D, n_cb, column_slice, st);
+  if (sq_block_eligible(codes, out, num_src_rows, src_dim, D, target_bits, (int64_t)n_cb << target_bits))
+    return sq_block_run(false, c8, codebooks, 0, column_slice, n_cb, indptr, indices, idx_dtype, out,
+                        num_rows, num_edges, num_src_rows, src_dim, D, target_bits, st, what);
   const bool lut_fits = (int64_t)n_cb * (1 << target_bits) * 4 <= 32 * 1024;
 #define F2CGT_CASE(B)                                                                                   \
   case B:                                                                                               \
@@ -712,6 +716,12 @@ extern "C" int f2cgt_sq_affine_decompress_spmm_csr(const uint8_t* codes, const f
   F2CGT_REQUIRE(params && (num_edges == 0 || codes), F2CGT_E_INVALID, "%s: null buffer", what);
   hipStream_t st = as_stream(stream);
   const int D = (int)feat_dim;
+  if (sq_affine_acc_eligible(codes, out, num_src_rows, src_dim, D, target_bits))
+    return sq_affine_acc_run(codes, params, param_stride, indptr, indices, idx_dtype, out, num_rows,
+                              num_edges, num_src_rows, src_dim, D, target_bits, st, what);
+  if (sq_block_eligible(codes, out, num_src_rows, src_dim, D, target_bits, 0))
+    return sq_block_run(true, codes, params, param_stride, 1, 1, indptr, indices, idx_dtype, out, num_rows,
+                        num_edges, num_src_rows, src_dim, D, target_bits, st, what);
   switch (target_bits) {
     case 1: return run_sq_affine<1>(codes, params, param_stride, indptr, indices, idx_dtype, out, num_rows, num_edges, num_src_rows, src_dim, D, st);
     case 2: return run_sq_affine<2>(codes, params, param_stride, indptr, indices, idx_dtype, out, num_rows, num_edges, num_src_rows, src_dim, D, st);

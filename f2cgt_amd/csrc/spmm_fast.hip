@@ -1,0 +1,544 @@
+// Row-block kernels for the fused decompress + mean aggregation.
+//
+// The per-row skeleton in spmm.hip walks indptr -> indices -> code row -> store as a
+// chain of dependent HBM round trips per destination row; with 2-15 edges per row that
+// chain, not bandwidth, sets the run time.  Here a workgroup owns a block of consecutive
+// destination rows and turns the chain into three wide phases, each one coalesced burst
+// of independent loads:
+//   1. indptr[row0 .. row0+RB]            -> LDS
+//   2. indices[e0 .. e1)  (contiguous)    -> LDS (clamped source ids)
+//   3. the packed code rows of all edges  -> LDS staging (each lane LB bytes)
+//   4. decode + sum in edge order per (row, column chunk) from LDS, IEEE divide by the
+//      degree, one non-temporal float4/float4x2 store; the block's output is one
+//      contiguous span, written in address order.
+// Several workgroups share a CU, so one block's phase 4 overlaps the loads of others.
+// Blocks whose edge count exceeds the LDS staging capacity fall back to a direct
+// per-row loop inside the same kernel.
+#include "spmm_fast.hpp"
+
+namespace f2cgt {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kStageBytes = 18 * 1024;  // LDS staging per workgroup -> 7-8 workgroups per CU
+constexpr int kGatherUnroll = 8;
+
+template <int LB> struct word_of;
+template <> struct word_of<1> { using type = uint8_t; };
+template <> struct word_of<2> { using type = uint16_t; };
+template <> struct word_of<4> { using type = uint32_t; };
+
+struct SqBlockArgs {
+  const uint8_t* codes;
+  const float* table;    // affine: params [2, param_stride]; log domain: codebooks [n_cb, 5]
+  int64_t param_stride;  // affine only
+  int64_t column_slice;  // log domain only
+  int num_codebooks;     // log domain only
+  int64_t R, E, N;
+  int src_dim, feat_dim;
+  int rows_per_block;    // RB
+  int edge_cap;          // staging capacity in edges
+  int pitch;             // staged bytes per edge (multiple of 4)
+  int cp2;               // lanes per row = pow2 >= chunks per row
+};
+
+// Per-lane decode state for its fixed column chunk.
+template <int BITS, int LB, bool AFFINE>
+struct ChunkDecoder {
+  static constexpr int PER = 8 / BITS;
+  static constexpr int NOUT = LB * PER;
+  static constexpr int NCODE = 1 << BITS;
+  float mn[AFFINE ? NOUT : 1];
+  float sc[AFFINE ? NOUT : 1];
+  int lut_base[AFFINE ? 1 : LB];
+  const float* lut;
+
+  __device__ void init(const SqBlockArgs& a, int chunk, bool active, const float* lds_lut) {
+    lut = lds_lut;
+    if (AFFINE) {
+#pragma unroll
+      for (int i = 0; i < NOUT; ++i) {
+        mn[i] = active ? a.table[chunk * NOUT + i] : 0.f;
+        sc[i] = active ? a.table[a.param_stride + chunk * NOUT + i] : 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int b = 0; b < LB; ++b) {
+        int64_t cb = ((int64_t)(chunk * LB + b) * PER) / a.column_slice;
+        cb = cb < a.num_codebooks ? cb : a.num_codebooks - 1;
+        lut_base[b] = (int)cb * NCODE;
+      }
+    }
+  }
+  __device__ __forceinline__ void add(uint32_t w, float (&acc)[NOUT]) const {
+    if (AFFINE) {
+#pragma unroll
+      for (int i = 0; i < NOUT; ++i) {
+        const float code = (float)((w >> (BITS * i)) & (NCODE - 1));
+        acc[i] += __fadd_rn(mn[i], __fmul_rn(code, sc[i]));
+      }
+    } else {
+#pragma unroll
+      for (int b = 0; b < LB; ++b) {
+        const uint32_t byte = (w >> (8 * b)) & 0xffu;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) acc[b * PER + k] += lut[lut_base[b] + ((byte >> (BITS * k)) & (NCODE - 1))];
+      }
+    }
+  }
+};
+
+template <int NOUT>
+__device__ __forceinline__ void store_chunk(float* o, const float (&acc)[NOUT], float deg) {
+#pragma unroll
+  for (int i = 0; i < NOUT; i += 4)
+    store_nt4(o + i, acc[i] / deg, acc[i + 1] / deg, acc[i + 2] / deg, acc[i + 3] / deg);
+}
+
+template <int BITS, int LB, bool AFFINE, typename Idx>
+__global__ __launch_bounds__(kBlock) void sq_block_kernel(SqBlockArgs a, const Idx* __restrict__ indptr,
+                                                          const Idx* __restrict__ indices,
+                                                          float* __restrict__ out) {
+  using W = typename word_of<LB>::type;
+  using Dec = ChunkDecoder<BITS, LB, AFFINE>;
+  constexpr int NOUT = Dec::NOUT;
+  extern __shared__ __align__(16) unsigned char smem[];
+  // layout: [lut floats][RB+1 edge offsets int64][edge_cap ids uint32][edge_cap * pitch bytes]
+  float* s_lut = reinterpret_cast<float*>(smem);
+  const int lut_floats = AFFINE ? 0 : ((a.num_codebooks * Dec::NCODE + 3) & ~3);
+  int64_t* s_ptr = reinterpret_cast<int64_t*>(s_lut + lut_floats);
+  uint32_t* s_ids = reinterpret_cast<uint32_t*>(s_ptr + a.rows_per_block + 2);
+  unsigned char* s_codes = reinterpret_cast<unsigned char*>(s_ids + a.edge_cap);
+
+  const int t = threadIdx.x;
+  const int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block;
+  const int nrows = (int)((a.R - row0) < a.rows_per_block ? (a.R - row0) : a.rows_per_block);
+
+  // phase 1: row offsets (and the LUT of the log-domain decoder)
+  for (int i = t; i <= nrows; i += kBlock) {
+    int64_t v = (int64_t)indptr[row0 + i];
+    s_ptr[i] = v < 0 ? 0 : (v > a.E ? a.E : v);
+  }
+  if (!AFFINE) {
+    for (int i = t; i < a.num_codebooks * Dec::NCODE; i += kBlock) {
+      const float* cb = a.table + (int64_t)(i >> BITS) * 5;
+      const uint32_t raw = (uint32_t)(i & (Dec::NCODE - 1));
+      float v;
+      if (BITS == 1) {
+        v = ((float)raw - 0.5f) * (2.f * cb[4]);
+      } else {
+        const float drange = (float)(1 << (BITS - 1));
+        const float k = __fdiv_rn(__fsub_rn(cb[3], cb[2]), drange);
+        v = sq_log_decode(BITS < 8 ? (float)raw - drange : (float)(int8_t)raw, k, cb[2]);
+      }
+      s_lut[i] = v;
+    }
+  }
+  const int chunks = a.feat_dim / NOUT;
+  const int chunk = t & (a.cp2 - 1);
+  const int slot = t / a.cp2;
+  const int nslots = kBlock / a.cp2;
+  const bool active = chunk < chunks;
+  Dec dec;
+  dec.init(a, chunk, active, s_lut);
+  __syncthreads();
+
+  const int64_t e0 = s_ptr[0];
+  int64_t e1 = s_ptr[nrows];
+  e1 = e1 < e0 ? e0 : e1;
+  const int64_t ne64 = e1 - e0;
+
+  if (ne64 <= a.edge_cap) {
+    const int ne = (int)ne64;
+    // phase 2: source ids
+    for (int i = t; i < ne; i += kBlock) s_ids[i] = (uint32_t)clamp_idx(indices[e0 + i], a.N);
+    __syncthreads();
+    // phase 3: gather the packed rows
+    if (active) {
+      const uint8_t* base = a.codes + chunk * LB;
+      for (int e = slot; e < ne; e += nslots * kGatherUnroll) {
+        W w[kGatherUnroll];
+#pragma unroll
+        for (int u = 0; u < kGatherUnroll; ++u) {
+          const int ee = e + u * nslots;
+          if (ee < ne) w[u] = *reinterpret_cast<const W*>(base + (int64_t)s_ids[ee] * a.src_dim);
+        }
+#pragma unroll
+        for (int u = 0; u < kGatherUnroll; ++u) {
+          const int ee = e + u * nslots;
+          if (ee < ne) *reinterpret_cast<W*>(s_codes + ee * a.pitch + chunk * LB) = w[u];
+        }
+      }
+    }
+    __syncthreads();
+    // phase 4: decode + mean, rows in address order
+    if (active) {
+      for (int r = slot; r < nrows; r += nslots) {
+        int b = (int)(s_ptr[r] - e0);
+        int e = (int)(s_ptr[r + 1] - e0);
+        b = b < 0 ? 0 : (b > ne ? ne : b);
+        e = e < b ? b : (e > ne ? ne : e);
+        float acc[NOUT];
+#pragma unroll
+        for (int i = 0; i < NOUT; ++i) acc[i] = 0.f;
+        for (int k = b; k < e; ++k)
+          dec.add((uint32_t)*reinterpret_cast<const W*>(s_codes + k * a.pitch + chunk * LB), acc);
+        const float deg = (float)(e - b == 0 ? 1 : e - b);
+        store_chunk<NOUT>(out + (row0 + r) * (int64_t)a.feat_dim + chunk * NOUT, acc, deg);
+      }
+    }
+  } else if (active) {
+    // over-capacity block: direct per-row loop
+    const uint8_t* base = a.codes + chunk * LB;
+    for (int r = slot; r < nrows; r += nslots) {
+      int64_t b = s_ptr[r], e = s_ptr[r + 1];
+      e = e < b ? b : e;
+      float acc[NOUT];
+#pragma unroll
+      for (int i = 0; i < NOUT; ++i) acc[i] = 0.f;
+      for (int64_t k = b; k < e; ++k) {
+        const int64_t s = clamp_idx(indices[k], a.N);
+        dec.add((uint32_t)*reinterpret_cast<const W*>(base + s * a.src_dim), acc);
+      }
+      const float deg = (float)(e - b == 0 ? 1 : e - b);
+      store_chunk<NOUT>(out + (row0 + r) * (int64_t)a.feat_dim + chunk * NOUT, acc, deg);
+    }
+  }
+}
+
+template <int BITS, int LB, bool AFFINE>
+int launch_sq_block(SqBlockArgs a, const void* indptr, const void* indices, int idx_dtype, float* out,
+                    hipStream_t st, const char* what) {
+  constexpr int NOUT = LB * (8 / BITS);
+  const int chunks = a.feat_dim / NOUT;
+  a.cp2 = pow2_ceil(chunks);
+  a.pitch = (chunks * LB + 3) & ~3;
+  const int lut_bytes = AFFINE ? 0 : (((a.num_codebooks << BITS) + 3) & ~3) * 4;
+  a.edge_cap = kStageBytes / (a.pitch + 4);
+  if (a.edge_cap > 1024) a.edge_cap = 1024;
+  const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 1.0;
+  int rb = (int)(0.7 * a.edge_cap / (avg_deg > 0.5 ? avg_deg : 0.5));
+  int rb2 = 4;
+  while (rb2 * 2 <= rb && rb2 < 64) rb2 *= 2;
+  const int min_rows = kBlock / a.cp2;  // at least one row per lane group
+  a.rows_per_block = rb2 < min_rows ? min_rows : rb2;
+  const size_t lds = (size_t)lut_bytes + (size_t)(a.rows_per_block + 2) * 8 + (size_t)a.edge_cap * 4 +
+                     (size_t)a.edge_cap * a.pitch;
+  const int64_t grid = ceil_div(a.R, a.rows_per_block);
+  if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
+  if (idx_dtype == F2CGT_DT_I32)
+    sq_block_kernel<BITS, LB, AFFINE, int32_t><<<(unsigned)grid, kBlock, lds, st>>>(
+        a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
+  else
+    sq_block_kernel<BITS, LB, AFFINE, int64_t><<<(unsigned)grid, kBlock, lds, st>>>(
+        a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
+  return launch_status(what);
+}
+
+
+// ---- affine SQ, 4- and 8-bit codes: integer accumulation in LDS ----------------------------
+// sum_e (min + c_e * scale) / deg == min + scale * (sum_e c_e) / deg, and the code sum is an
+// exact integer.  The block keeps per (row, 4 packed bytes) integer accumulators in LDS with the
+// codes widened to 16-bit fields (nibble k of each half-word -> accumulator k at 4 bits; even /
+// odd bytes -> accumulator 0 / 1 at 8 bits).  The gather is edge-parallel: one lane per aligned
+// dword of each edge's code row, realigned in registers (rows are only byte aligned in general:
+// src_dim = 50 at 4 bits x 100 columns), split into fields and added with LDS atomics, so there
+// is no per-row loop and no divergence.  The float work (convert, * 1/deg, * scale, + min) runs
+// once per output, one float4 of the block's contiguous output span per lane.  The result
+// differs from "decode, then sum in fp32" by a few ulp of the summands (it is the closer of the
+// two to the exact mean) and is identical to the decode for rows with one neighbour.
+//
+// Field capacity bounds the in-degree a row may have on this path (4369 at 4 bits, 257 at 8);
+// a block containing a larger row takes the direct per-output loop below instead.
+struct AccArgs {
+  const uint8_t* codes;
+  const float* params;
+  int64_t param_stride;
+  int64_t R, E, N;
+  int64_t table_bytes;
+  int src_dim, feat_dim;
+  int rows_per_block;
+  int edge_batch;
+  int dwords;        // aligned dwords that cover any row
+  int dw2;           // gather lanes per edge = pow2 >= dwords
+  int chunks;        // 4-byte column chunks per row that hold output columns
+  int f4_per_row;    // feat_dim / 4
+  uint32_t magic;    // ceil(2^32 / f4_per_row)
+  uint32_t last_full_dword;
+};
+
+template <int BITS>
+__device__ __forceinline__ void acc_direct_block(const AccArgs& a, const int* s_ptr, int64_t e0, int64_t row0,
+                                              int nrows, const int64_t* idx64, const int32_t* idx32,
+                                              float* __restrict__ out) {
+  constexpr int PER = 8 / BITS;
+  const int items = nrows * a.feat_dim;
+  for (int it = threadIdx.x; it < items; it += kBlock) {
+    const int r = it / a.feat_dim, col = it - r * a.feat_dim;
+    const int64_t b = e0 + s_ptr[r], e = e0 + s_ptr[r + 1];
+    uint64_t tot = 0;
+    for (int64_t k = b; k < e; ++k) {
+      const int64_t id = idx64 ? clamp_idx(idx64[k], a.N) : clamp_idx(idx32[k], a.N);
+      const uint32_t byte = a.codes[id * a.src_dim + col / PER];
+      tot += (byte >> (BITS * (col % PER))) & ((1u << BITS) - 1u);
+    }
+    const int64_t deg = e - b;
+    const float rdeg = __builtin_amdgcn_rcpf((float)(deg > 1 ? deg : 1));
+    const float v = __fadd_rn(a.params[col], __fmul_rn((float)tot * rdeg, a.params[a.param_stride + col]));
+    out[(row0 + r) * (int64_t)a.feat_dim + col] = deg == 0 ? 0.f : v;
+  }
+}
+
+template <int BITS, typename Idx>
+__global__ __launch_bounds__(kBlock) void sq_affine_acc_kernel(AccArgs a, const Idx* __restrict__ indptr,
+                                                               const Idx* __restrict__ indices,
+                                                               float* __restrict__ out) {
+  constexpr int NACC = BITS == 4 ? 4 : 2;             // accumulator words per chunk
+  constexpr int LIMIT = BITS == 4 ? 4369 : 257;       // edges per row before a 16-bit field can wrap
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint32_t* s_acc = reinterpret_cast<uint32_t*>(smem);                              // [RB][chunks][NACC]
+  float* s_par = reinterpret_cast<float*>(s_acc + (size_t)a.rows_per_block * a.chunks * NACC);  // [f4][8]
+  int* s_ptr = reinterpret_cast<int*>(s_par + (size_t)a.f4_per_row * 8);            // [RB + 1] (+ flag, tail)
+  uint32_t* s_row = reinterpret_cast<uint32_t*>(s_ptr + a.rows_per_block + 4);      // [edge_batch]
+  uint16_t* s_erow = reinterpret_cast<uint16_t*>(s_row + a.edge_batch);             // [edge_batch]
+  int* s_flag = s_ptr + a.rows_per_block + 1;
+  uint32_t* s_tail = reinterpret_cast<uint32_t*>(s_ptr + a.rows_per_block + 2);
+
+  const int t = threadIdx.x;
+  const int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block;
+  const int nrows = (int)((a.R - row0) < a.rows_per_block ? (a.R - row0) : a.rows_per_block);
+  int64_t e0 = (int64_t)indptr[row0];
+  e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
+  if (t == 0) {
+    *s_flag = 0;
+    uint32_t tail = 0;  // the bytes of the last, partial dword of the table (if any)
+    for (int64_t b = (int64_t)(a.last_full_dword + 1) * 4, i = 0; b < a.table_bytes && i < 4; ++b, ++i)
+      tail |= (uint32_t)a.codes[b] << (8 * i);
+    *s_tail = tail;
+  }
+  for (int i = t; i <= nrows; i += kBlock) {
+    int64_t v = (int64_t)indptr[row0 + i];
+    v = v < e0 ? e0 : (v > a.E ? a.E : v);
+    s_ptr[i] = (int)(v - e0 > 0x7fffffff ? 0x7fffffff : v - e0);
+  }
+  for (int i = t; i < nrows * a.chunks * NACC / 2; i += kBlock)
+    reinterpret_cast<uint2*>(s_acc)[i] = make_uint2(0u, 0u);
+  for (int i = t; i < a.f4_per_row * 4; i += kBlock) {
+    const int c4 = i >> 2, q = i & 3;
+    s_par[c4 * 8 + q] = a.params[i];
+    s_par[c4 * 8 + 4 + q] = a.params[a.param_stride + i];
+  }
+  __syncthreads();
+  if (s_ptr[nrows] > LIMIT) {  // only then can a single row exceed the field capacity
+    for (int r = t; r < nrows; r += kBlock)
+      if (s_ptr[r + 1] - s_ptr[r] > LIMIT) *s_flag = 1;
+    __syncthreads();
+    if (*s_flag) {
+      const bool is64 = sizeof(Idx) == 8;
+      acc_direct_block<BITS>(a, s_ptr, e0, row0, nrows,
+                             is64 ? reinterpret_cast<const int64_t*>(indices) : nullptr,
+                             is64 ? nullptr : reinterpret_cast<const int32_t*>(indices), out);
+      return;
+    }
+  }
+  const int ne = s_ptr[nrows];
+  const uint32_t tail_word = *s_tail;
+  const uint32_t* codes32 = reinterpret_cast<const uint32_t*>(a.codes);
+
+  for (int eb = 0; eb < ne; eb += a.edge_batch) {
+    const int nb = (ne - eb) < a.edge_batch ? (ne - eb) : a.edge_batch;
+    if (eb) __syncthreads();
+    for (int i = t; i < nb; i += kBlock) {
+      const uint64_t start = (uint64_t)clamp_idx(indices[e0 + eb + i], a.N) * (uint32_t)a.src_dim;
+      s_row[i] = (uint32_t)(start >> 2);
+      s_erow[i] = (uint16_t)((start & 3) << 14);
+    }
+    __syncthreads();
+    for (int r = t; r < nrows; r += kBlock) {  // tag every edge of the batch with its local row
+      int b = s_ptr[r] - eb, e = s_ptr[r + 1] - eb;
+      b = b < 0 ? 0 : b;
+      e = e > nb ? nb : e;
+      for (int k = b; k < e; ++k) s_erow[k] |= (uint16_t)r;
+    }
+    __syncthreads();
+    const int j = t & (a.dw2 - 1);
+    const int gslot = t / a.dw2;
+    const int gslots = kBlock / a.dw2;
+    constexpr int U = 4;
+    for (int e = gslot; e < nb; e += gslots * U) {
+      uint32_t w[U], er[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        int ee = e + u * gslots;
+        ee = ee < nb ? ee : nb - 1;
+        const uint32_t d = s_row[ee] + j;
+        er[u] = s_erow[ee];
+        const uint32_t v = codes32[d < a.last_full_dword ? d : a.last_full_dword];
+        w[u] = d > a.last_full_dword ? (d == a.last_full_dword + 1 ? tail_word : 0u) : v;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int ee = e + u * gslots;
+        const uint32_t hi = __shfl_down(w[u], 1);
+        const uint32_t al = __builtin_amdgcn_alignbyte(hi, w[u], er[u] >> 14);
+        if (ee < nb && j < a.chunks) {
+          uint32_t* acc = s_acc + ((er[u] & 0x3fffu) * a.chunks + j) * NACC;
+          if (BITS == 4) {
+            atomicAdd(acc + 0, al & 0x000f000fu);
+            atomicAdd(acc + 1, (al >> 4) & 0x000f000fu);
+            atomicAdd(acc + 2, (al >> 8) & 0x000f000fu);
+            atomicAdd(acc + 3, (al >> 12) & 0x000f000fu);
+          } else {
+            atomicAdd(acc + 0, al & 0x00ff00ffu);
+            atomicAdd(acc + 1, (al >> 8) & 0x00ff00ffu);
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // finalize: lane <-> one float4 of the block's contiguous output span
+  const int items = nrows * a.f4_per_row;
+  float* ob = out + row0 * (int64_t)a.feat_dim;
+  for (int it = t; it < items; it += kBlock) {
+    const int r = (int)__umulhi((uint32_t)it, a.magic);
+    const int c4 = it - r * a.f4_per_row;
+    float s0, s1, s2, s3;
+    if (BITS == 4) {
+      const uint4 q = *reinterpret_cast<const uint4*>(s_acc + (r * a.chunks + (c4 >> 1)) * 4);
+      const int sh = (c4 & 1) * 16;
+      s0 = (float)((q.x >> sh) & 0xffffu);
+      s1 = (float)((q.y >> sh) & 0xffffu);
+      s2 = (float)((q.z >> sh) & 0xffffu);
+      s3 = (float)((q.w >> sh) & 0xffffu);
+    } else {
+      const uint2 q = *reinterpret_cast<const uint2*>(s_acc + (r * a.chunks + c4) * 2);
+      s0 = (float)(q.x & 0xffffu);
+      s1 = (float)(q.y & 0xffffu);
+      s2 = (float)(q.x >> 16);
+      s3 = (float)(q.y >> 16);
+    }
+    const int deg = s_ptr[r + 1] - s_ptr[r];  // <= 0 for an empty (or malformed) row
+    const float rdeg = __builtin_amdgcn_rcpf((float)(deg > 1 ? deg : 1));  // rcp(1) == 1 exactly
+    const float4 mn = *reinterpret_cast<const float4*>(s_par + c4 * 8);
+    const float4 sc = *reinterpret_cast<const float4*>(s_par + c4 * 8 + 4);
+    float v0 = __fadd_rn(mn.x, __fmul_rn(s0 * rdeg, sc.x));
+    float v1 = __fadd_rn(mn.y, __fmul_rn(s1 * rdeg, sc.y));
+    float v2 = __fadd_rn(mn.z, __fmul_rn(s2 * rdeg, sc.z));
+    float v3 = __fadd_rn(mn.w, __fmul_rn(s3 * rdeg, sc.w));
+    if (deg <= 0) v0 = v1 = v2 = v3 = 0.f;
+    store_nt4(ob + (int64_t)it * 4, v0, v1, v2, v3);
+  }
+}
+
+template <int BITS>
+int launch_acc(AccArgs a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
+               const char* what) {
+  constexpr int NOUT = 32 / BITS;
+  constexpr int NACC = BITS == 4 ? 4 : 2;
+  a.chunks = (int)ceil_div(a.feat_dim, NOUT);
+  a.f4_per_row = a.feat_dim / 4;
+  a.magic = (uint32_t)((0x100000000ull + a.f4_per_row - 1) / a.f4_per_row);
+  const int maxshift = a.src_dim % 4 == 0 ? 0 : (a.src_dim % 2 == 0 ? 2 : 3);
+  a.dwords = (int)ceil_div(a.chunks * 4 + maxshift, 4);
+  a.dw2 = pow2_ceil(a.dwords);
+  a.last_full_dword = (uint32_t)((a.table_bytes - 4) >> 2);
+  a.edge_batch = 384;
+  const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 1.0;
+  const int want = (int)(160.0 / (avg_deg > 0.5 ? avg_deg : 0.5));
+  int rb = 8;
+  while (rb * 2 <= want && rb < 64) rb *= 2;
+  const size_t acc_row = (size_t)a.chunks * NACC * 4;
+  while (rb > 8 && rb * acc_row > 20 * 1024) rb /= 2;
+  a.rows_per_block = rb;
+  const size_t lds = rb * acc_row + (size_t)a.f4_per_row * 32 + (size_t)(rb + 4) * 4 +
+                     (size_t)a.edge_batch * 6 + 16;
+  const int64_t grid = ceil_div(a.R, rb);
+  if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
+  if (idx_dtype == F2CGT_DT_I32)
+    sq_affine_acc_kernel<BITS, int32_t><<<(unsigned)grid, kBlock, lds, st>>>(
+        a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
+  else
+    sq_affine_acc_kernel<BITS, int64_t><<<(unsigned)grid, kBlock, lds, st>>>(
+        a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
+  return launch_status(what);
+}
+
+}  // namespace
+
+bool sq_block_eligible(const void* codes, const float* out, int64_t N, int64_t src_dim, int feat_dim,
+                       int target_bits, int64_t lut_entries) {
+  int lb, nout;
+  switch (target_bits) {
+    case 8: lb = 4; nout = 4; break;
+    case 4: lb = 2; nout = 4; break;
+    case 2: lb = 1; nout = 4; break;
+    case 1: lb = 1; nout = 8; break;
+    default: return false;
+  }
+  if (feat_dim < nout || feat_dim % nout != 0) return false;
+  if (feat_dim / nout > kBlock) return false;
+  if (src_dim % lb != 0 || !aligned(codes, lb) || !aligned(out, 16)) return false;
+  if (src_dim * (8 / target_bits) < feat_dim) return false;
+  if (N >= (1ll << 32) || src_dim >= (1ll << 24)) return false;
+  if (lut_entries * 4 > 16 * 1024) return false;
+  return true;
+}
+
+int sq_block_run(bool affine, const uint8_t* codes, const float* table, int64_t param_stride,
+                 int64_t column_slice, int num_codebooks, const void* indptr, const void* indices,
+                 int idx_dtype, float* out, int64_t R, int64_t E, int64_t N, int64_t src_dim, int feat_dim,
+                 int target_bits, hipStream_t st, const char* what) {
+  SqBlockArgs a{};
+  a.codes = codes;
+  a.table = table;
+  a.param_stride = param_stride;
+  a.column_slice = column_slice;
+  a.num_codebooks = num_codebooks;
+  a.R = R; a.E = E; a.N = N;
+  a.src_dim = (int)src_dim;
+  a.feat_dim = feat_dim;
+#define F2CGT_GO(B, L)                                                                              \
+  return affine ? launch_sq_block<B, L, true>(a, indptr, indices, idx_dtype, out, st, what)        \
+                : launch_sq_block<B, L, false>(a, indptr, indices, idx_dtype, out, st, what)
+  switch (target_bits) {
+    case 8: F2CGT_GO(8, 4);
+    case 4: F2CGT_GO(4, 2);
+    case 2: F2CGT_GO(2, 1);
+    default: F2CGT_GO(1, 1);
+  }
+#undef F2CGT_GO
+}
+
+bool sq_affine_acc_eligible(const void* codes, const float* out, int64_t N, int64_t src_dim, int feat_dim,
+                            int target_bits) {
+  if (target_bits != 4 && target_bits != 8) return false;
+  if (!aligned(codes, 4) || !aligned(out, 16)) return false;
+  if (feat_dim < 4 || feat_dim % 4 != 0 || feat_dim > 4096) return false;
+  if (src_dim < 1 || src_dim >= (1ll << 20) || src_dim * (8 / target_bits) < feat_dim) return false;
+  const int64_t table_bytes = N * src_dim;
+  if (N >= (1ll << 32) || table_bytes < 8 || (table_bytes >> 2) >= (1ll << 32) - 4096) return false;
+  const int chunks = (int)ceil_div(feat_dim, 32 / target_bits);
+  if (pow2_ceil(chunks + 1) > kBlock) return false;
+  // the register realignment of byte-shifted rows exchanges dwords inside one wave
+  if (src_dim % 4 != 0 && pow2_ceil(chunks + 1) > kWave) return false;
+  if ((size_t)chunks * (target_bits == 4 ? 16 : 8) * 8 > 20 * 1024) return false;
+  return true;
+}
+
+int sq_affine_acc_run(const uint8_t* codes, const float* params, int64_t param_stride, const void* indptr,
+                      const void* indices, int idx_dtype, float* out, int64_t R, int64_t E, int64_t N,
+                      int64_t src_dim, int feat_dim, int target_bits, hipStream_t st, const char* what) {
+  AccArgs a{};
+  a.codes = codes;
+  a.params = params;
+  a.param_stride = param_stride;
+  a.R = R; a.E = E; a.N = N;
+  a.table_bytes = N * src_dim;
+  a.src_dim = (int)src_dim;
+  a.feat_dim = feat_dim;
+  return target_bits == 4 ? launch_acc<4>(a, indptr, indices, idx_dtype, out, st, what)
+                          : launch_acc<8>(a, indptr, indices, idx_dtype, out, st, what);
+}
+
+}  // namespace f2cgt

@@ -1,0 +1,24 @@
+// Row-block variants of the fused aggregation kernels (see spmm_fast.hip).
+#pragma once
+#include "common.hpp"
+
+namespace f2cgt {
+
+// True when the row-block SQ kernel covers this shape (otherwise use the per-row skeleton).
+bool sq_block_eligible(const void* codes, const float* out, int64_t N, int64_t src_dim, int feat_dim,
+                       int target_bits, int64_t lut_entries);
+
+// affine: table = params [2, param_stride]; log domain: table = codebooks [num_codebooks, 5].
+int sq_block_run(bool affine, const uint8_t* codes, const float* table, int64_t param_stride,
+                 int64_t column_slice, int num_codebooks, const void* indptr, const void* indices,
+                 int idx_dtype, float* out, int64_t R, int64_t E, int64_t N, int64_t src_dim, int feat_dim,
+                 int target_bits, hipStream_t st, const char* what);
+
+// Integer-accumulating row-block kernel for per-column affine codes of 4 or 8 bits.
+bool sq_affine_acc_eligible(const void* codes, const float* out, int64_t N, int64_t src_dim, int feat_dim,
+                            int target_bits);
+int sq_affine_acc_run(const uint8_t* codes, const float* params, int64_t param_stride, const void* indptr,
+                      const void* indices, int idx_dtype, float* out, int64_t R, int64_t E, int64_t N,
+                      int64_t src_dim, int feat_dim, int target_bits, hipStream_t st, const char* what);
+
+}  // namespace f2cgt
