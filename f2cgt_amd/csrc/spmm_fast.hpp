@@ -21,4 +21,11 @@ int sq_affine_acc_run(const uint8_t* codes, const float* params, int64_t param_s
                       const void* indices, int idx_dtype, float* out, int64_t R, int64_t E, int64_t N,
                       int64_t src_dim, int feat_dim, int target_bits, hipStream_t st, const char* what);
 
+// Persistent software-pipelined VQ kernel (uint8 codes, K <= 256, width 8/16/32), vq_fast.hip.
+bool vq_pipe_eligible(const void* codes, const float* codebooks, const float* out, int64_t R, int64_t N,
+                      int feat_dim, int n_cb, int K, int w);
+int vq_pipe_run(const uint8_t* codes, const float* codebooks, const void* indptr, const void* indices,
+                int idx_dtype, float* out, int64_t R, int64_t E, int64_t N, int feat_dim, int n_cb, int K, int w,
+                hipStream_t st, const char* what);
+
 }  // namespace f2cgt

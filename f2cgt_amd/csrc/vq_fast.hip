@@ -1,0 +1,307 @@
+// Persistent, software-pipelined kernel for the fused VQ decode + mean aggregation.
+//
+// One 1024-thread workgroup per CU keeps a 128-column tile of the codebook in LDS, laid out
+// [code][piece][8 floats] (a "piece" is 8 consecutive output columns), so the 32 B a lane reads
+// per edge land on bank groups fixed by its piece: measured ~110 B/clk/CU against 62 B/clk for
+// the natural [subspace][code][w] layout.  A lane owns one (destination row, piece) of a
+// 64-row block and walks the row's edges in order with register accumulators; the codebook
+// reads of the next group of edges are issued before the adds of the current group.
+//
+// Everything that comes from HBM is prefetched through registers two iterations ahead, one
+// element per lane and stage, and parked in LDS one barrier before it is needed:
+//     P  indptr of block b        issued at iteration b-6, in LDS (ring of 8) after b-5
+//     I  source id of edge t      issued at b-4 (needs P), stays in the lane's register
+//     C  code bytes of edge t     issued at b-2 (needs I), in LDS after b-1
+//     compute block b             iteration b
+// so the dependent chain indptr -> indices -> codes -> output never stalls a wave.
+// Workgroups are bound to a (column tile, row stripe); wide features (D = 768) use six tiles.
+#include "spmm_fast.hpp"
+
+namespace f2cgt {
+namespace {
+
+constexpr int kThreads = 1024;
+constexpr int kRows = 64;        // destination rows per block (kThreads / 16 pieces)
+constexpr int kEdgeCap = 1024;   // staged edges per block: one per lane
+constexpr int kRing = 8;
+constexpr int kGroup = 5;        // edges per register group of the inner loop
+
+struct VqArgs {
+  const uint8_t* codes;
+  const float* codebooks;
+  int64_t R, E, N;
+  int n_cb, K, w, feat_dim;
+  int n_tiles, n_stripes;
+};
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <int BT> struct code_word;
+template <> struct code_word<4> { using type = uint32_t; };
+template <> struct code_word<8> { using type = u32x2; };
+template <> struct code_word<16> { using type = u32x4; };
+
+__device__ __forceinline__ float dpp_swap_pair(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
+}
+
+// Correctly rounded a / d from r = RN-refined 1/d (two FMAs after the product).
+__device__ __forceinline__ float div_by(float a, float d, float r) {
+  const float q = a * r;
+  return __fmaf_rn(__fmaf_rn(-q, d, a), r, q);
+}
+
+template <int BT, typename Idx>
+struct VqPipe {
+  using CW = typename code_word<BT>::type;
+  // register state, two generations per stage
+  int64_t Pa, Pb, P0a, P0b;
+  uint32_t Ia, Ib;
+  CW Ca, Cb;
+  template <int G> __device__ __forceinline__ int64_t& Pr() { if constexpr (G == 0) return Pa; else return Pb; }
+  template <int G> __device__ __forceinline__ int64_t& P0r() { if constexpr (G == 0) return P0a; else return P0b; }
+  template <int G> __device__ __forceinline__ uint32_t& Ir() { if constexpr (G == 0) return Ia; else return Ib; }
+  template <int G> __device__ __forceinline__ CW& Cr() { if constexpr (G == 0) return Ca; else return Cb; }
+
+  const VqArgs& a;
+  const Idx* __restrict__ indptr;
+  const Idx* __restrict__ indices;
+  float* __restrict__ out;
+  float* s_cb;
+  unsigned char* s_codes;
+  int* s_ptr;       // [kRing][kRows + 2]: relative edge offsets, [kRows + 1] = edge count
+  int64_t* s_e0;    // [kRing]
+  int tile, stripe, t;
+  int64_t my_blocks;
+
+  __device__ VqPipe(const VqArgs& a_, const Idx* ip, const Idx* ix, float* o) : a(a_), indptr(ip), indices(ix), out(o) {}
+
+  __device__ __forceinline__ int64_t global_block(int64_t b) const { return stripe + b * a.n_stripes; }
+  __device__ __forceinline__ bool valid(int64_t b) const { return b >= 0 && b < my_blocks; }
+  __device__ __forceinline__ int rows_of(int64_t b) const {
+    const int64_t row0 = global_block(b) * kRows;
+    return (int)((a.R - row0) < kRows ? (a.R - row0) : kRows);
+  }
+
+  template <int PAR>
+  __device__ __forceinline__ void iteration(int64_t it) {
+    // ---- issue the three prefetch stages ---------------------------------------------------
+    {
+      const int64_t b = it + 2;  // C: code bytes, address from the id this lane fetched at b-4
+      if (valid(b)) {
+        const int ne = s_ptr[(b & (kRing - 1)) * (kRows + 2) + kRows + 1];
+        if (t < ne && ne <= kEdgeCap)
+          Cr<PAR>() = *reinterpret_cast<const CW*>(a.codes + (int64_t)Ir<PAR>() * a.n_cb + tile * BT);
+      }
+    }
+    {
+      const int64_t b = it + 4;  // I: source id of edge t
+      if (valid(b)) {
+        const int slot = (int)(b & (kRing - 1));
+        const int ne = s_ptr[slot * (kRows + 2) + kRows + 1];
+        if (t < ne && ne <= kEdgeCap) Ir<PAR>() = (uint32_t)clamp_idx(indices[s_e0[slot] + t], a.N);
+      }
+    }
+    {
+      const int64_t b = it + 6;  // P: row offsets
+      if (valid(b)) {
+        const int64_t row0 = global_block(b) * kRows;
+        const int nr = rows_of(b);
+        P0r<PAR>() = (int64_t)indptr[row0];
+        if (t <= nr) Pr<PAR>() = (int64_t)indptr[row0 + t];
+      }
+    }
+    // ---- compute block `it` ------------------------------------------------------------------
+    if (valid(it)) compute(it);
+    __syncthreads();
+    // ---- park what was issued one iteration ago ------------------------------------------------
+    {
+      const int64_t b = it + 1;  // C issued at it-1 lives in C[PAR ^ 1]
+      if (valid(b)) {
+        const int ne = s_ptr[(b & (kRing - 1)) * (kRows + 2) + kRows + 1];
+        if (t < ne && ne <= kEdgeCap) *reinterpret_cast<CW*>(s_codes + t * BT) = Cr<PAR ^ 1>();
+      }
+    }
+    {
+      const int64_t b = it + 5;  // P issued at it-1 lives in P[PAR ^ 1]
+      if (valid(b)) {
+        const int slot = (int)(b & (kRing - 1));
+        const int nr = rows_of(b);
+        int64_t e0 = P0r<PAR ^ 1>();
+        e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
+        if (t <= nr) {
+          int64_t v = Pr<PAR ^ 1>();
+          v = v < e0 ? e0 : (v > a.E ? a.E : v);
+          const int64_t rel = v - e0;
+          const int r32 = rel > 0x3fffffff ? 0x3fffffff : (int)rel;
+          s_ptr[slot * (kRows + 2) + t] = r32;
+          if (t == nr) s_ptr[slot * (kRows + 2) + kRows + 1] = r32;
+        }
+        if (t == 0) s_e0[slot] = e0;
+      }
+    }
+    __syncthreads();
+  }
+
+  // A lane owns one float4 of a destination row (32 lanes per row: the conflict-free LDS
+  // pattern) and takes two rows of the block, 32 apart.
+  __device__ __forceinline__ void compute(int64_t b) {
+    const int c4 = t & 31;
+    const int rs = t >> 5;
+    const int slot = (int)(b & (kRing - 1));
+    const int* sp = s_ptr + slot * (kRows + 2);
+    const int nr = rows_of(b);
+    const int tile_cols = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
+    if (c4 * 4 >= tile_cols) return;
+    const int ne = sp[kRows + 1];
+    const int byte_idx = (c4 * 4) / a.w;
+    const float* cbp = s_cb + c4 * 4;
+    const bool staged = ne <= kEdgeCap;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+      const int row = rs + pass * 32;
+      if (row >= nr) continue;
+      int eb = sp[row], ee = sp[row + 1];
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+      int n;
+      if (staged) {
+        eb = eb > ne ? ne : eb;
+        ee = ee > ne ? ne : ee;
+        n = ee - eb;
+        const unsigned char* cp = s_codes + eb * BT + byte_idx;
+        int k = 0;
+        for (; k + kGroup <= n; k += kGroup) {
+          uint32_t code[kGroup];
+          float4 x[kGroup];
+#pragma unroll
+          for (int u = 0; u < kGroup; ++u) code[u] = cp[u * BT];
+          cp += kGroup * BT;
+#pragma unroll
+          for (int u = 0; u < kGroup; ++u) x[u] = *reinterpret_cast<const float4*>(cbp + code[u] * 128);
+#pragma unroll
+          for (int u = 0; u < kGroup; ++u) { a0 += x[u].x; a1 += x[u].y; a2 += x[u].z; a3 += x[u].w; }
+        }
+        for (; k < n; ++k) {
+          const uint32_t code = *cp;
+          cp += BT;
+          const float4 x = *reinterpret_cast<const float4*>(cbp + code * 128);
+          a0 += x.x; a1 += x.y; a2 += x.z; a3 += x.w;
+        }
+      } else {
+        // block with more edges than the staging holds: walk the row straight from HBM
+        n = ee - eb;
+        const int64_t e0 = s_e0[slot];
+        for (int k = 0; k < n; ++k) {
+          const int64_t id = clamp_idx(indices[e0 + eb + k], a.N);
+          const uint32_t code = a.codes[id * a.n_cb + tile * BT + byte_idx];
+          const float4 x = *reinterpret_cast<const float4*>(cbp + code * 128);
+          a0 += x.x; a1 += x.y; a2 += x.z; a3 += x.w;
+        }
+      }
+      if (n > 1) {
+        const float d = (float)n;
+        float r = __builtin_amdgcn_rcpf(d);
+        r = __fmaf_rn(__fmaf_rn(-d, r, 1.f), r, r);
+        a0 = div_by(a0, d, r); a1 = div_by(a1, d, r); a2 = div_by(a2, d, r); a3 = div_by(a3, d, r);
+      }
+      store_nt4(out + (global_block(b) * kRows + row) * (int64_t)a.feat_dim + tile * 128 + c4 * 4, a0, a1, a2, a3);
+    }
+  }
+};
+
+template <int BT, typename Idx>
+__global__ __launch_bounds__(kThreads) void vq_pipe_kernel(VqArgs a, const Idx* __restrict__ indptr,
+                                                           const Idx* __restrict__ indices,
+                                                           float* __restrict__ out) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  VqPipe<BT, Idx> pipe(a, indptr, indices, out);
+  pipe.s_cb = reinterpret_cast<float*>(smem);
+  pipe.s_codes = smem + (size_t)a.K * 128 * 4;
+  pipe.s_e0 = reinterpret_cast<int64_t*>(pipe.s_codes + kEdgeCap * BT);
+  pipe.s_ptr = reinterpret_cast<int*>(pipe.s_e0 + kRing);
+  pipe.t = threadIdx.x;
+  pipe.tile = blockIdx.x % a.n_tiles;
+  pipe.stripe = blockIdx.x / a.n_tiles;
+  const int64_t nblocks = ceil_div(a.R, kRows);
+  pipe.my_blocks = pipe.stripe < nblocks ? (nblocks - pipe.stripe + a.n_stripes - 1) / a.n_stripes : 0;
+  pipe.Pa = pipe.Pb = pipe.P0a = pipe.P0b = 0;
+  pipe.Ia = pipe.Ib = 0;
+
+  // codebook tile -> LDS as [code][piece][8]
+  const int tile_cols = (a.feat_dim - pipe.tile * 128) >= 128 ? 128 : (a.feat_dim - pipe.tile * 128);
+  for (int i = threadIdx.x; i < a.K * 128; i += kThreads) {
+    const int code = i >> 7, c = i & 127;
+    float v = 0.f;
+    if (c < tile_cols) {
+      const int col = pipe.tile * 128 + c;
+      const int sub = col / a.w;
+      v = a.codebooks[((int64_t)sub * a.K + code) * a.w + (col - sub * a.w)];
+    }
+    pipe.s_cb[i] = v;
+  }
+  for (int i = threadIdx.x; i < kRing * (kRows + 2); i += kThreads) pipe.s_ptr[i] = 0;
+  __syncthreads();
+
+  for (int64_t it = -6; it < pipe.my_blocks; it += 2) {
+    pipe.template iteration<0>(it);
+    pipe.template iteration<1>(it + 1);
+  }
+}
+
+template <int BT>
+int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
+              const char* what) {
+  const size_t lds = (size_t)a.K * 128 * 4 + (size_t)kEdgeCap * BT + kRing * 8 + kRing * (kRows + 2) * 4;
+  const int cus = num_cus();
+  a.n_tiles = (int)ceil_div(a.feat_dim, 128);
+  a.n_stripes = cus / a.n_tiles;
+  if (a.n_stripes < 1) a.n_stripes = 1;
+  const int64_t nblocks = ceil_div(a.R, kRows);
+  if (a.n_stripes > nblocks) a.n_stripes = (int)(nblocks > 0 ? nblocks : 1);
+  const unsigned grid = (unsigned)(a.n_stripes * a.n_tiles);
+  hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_pipe_kernel<BT, int32_t>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_pipe_kernel<BT, int64_t>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e1 != hipSuccess || e2 != hipSuccess)
+    return fail((int)(e1 != hipSuccess ? e1 : e2), "%s: cannot reserve %zu B of LDS", what, lds);
+  if (idx_dtype == F2CGT_DT_I32)
+    vq_pipe_kernel<BT, int32_t><<<grid, kThreads, lds, st>>>(a, static_cast<const int32_t*>(indptr),
+                                                            static_cast<const int32_t*>(indices), out);
+  else
+    vq_pipe_kernel<BT, int64_t><<<grid, kThreads, lds, st>>>(a, static_cast<const int64_t*>(indptr),
+                                                            static_cast<const int64_t*>(indices), out);
+  return launch_status(what);
+}
+
+}  // namespace
+
+bool vq_pipe_eligible(const void* codes, const float* codebooks, const float* out, int64_t R, int64_t N,
+                      int feat_dim, int n_cb, int K, int w) {
+  if (K < 1 || K > 256) return false;
+  if (w != 8 && w != 16 && w != 32) return false;
+  const int bt = 128 / w;
+  if (n_cb % bt != 0 || !aligned(codes, bt)) return false;
+  if (feat_dim < 16 || feat_dim % 4 != 0 || feat_dim > n_cb * w) return false;
+  if (!aligned(out, 16) || !aligned(codebooks, 4)) return false;
+  if (N >= (1ll << 32)) return false;
+  if (R < 4 * kRows) return false;  // tiny problems: the per-row skeleton has less start-up cost
+  return true;
+}
+
+int vq_pipe_run(const uint8_t* codes, const float* codebooks, const void* indptr, const void* indices,
+                int idx_dtype, float* out, int64_t R, int64_t E, int64_t N, int feat_dim, int n_cb, int K, int w,
+                hipStream_t st, const char* what) {
+  VqArgs a{};
+  a.codes = codes;
+  a.codebooks = codebooks;
+  a.R = R; a.E = E; a.N = N;
+  a.n_cb = n_cb; a.K = K; a.w = w; a.feat_dim = feat_dim;
+  switch (128 / w) {
+    case 16: return launch_vq<16>(a, indptr, indices, idx_dtype, out, st, what);
+    case 8: return launch_vq<8>(a, indptr, indices, idx_dtype, out, st, what);
+    default: return launch_vq<4>(a, indptr, indices, idx_dtype, out, st, what);
+  }
+}
+
+}  // namespace f2cgt
