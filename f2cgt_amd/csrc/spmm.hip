@@ -762,6 +762,10 @@ extern "C" int f2cgt_hybrid_decompress_spmm_csr(
                 "%s: both tables must hold at least one row", what);
   hipStream_t st = as_stream(stream);
   const int D = (int)feat_dim, n_cb = (int)num_codebooks, k = (int)K, w = (int)width;
+  if (hybrid_acc_eligible(sq_codes, vq_codebooks, out, num_src_rows, num_sq_rows, num_vq_rows, D, w))
+    return hybrid_acc_run(row_map, sq_codes, sq_params, param_stride, vq_codes, vq_codebooks, indptr, indices,
+                          idx_dtype, out, num_rows, num_edges, num_src_rows, num_sq_rows, num_vq_rows, D, n_cb, k, w,
+                          st, what);
   const bool a16 = aligned(out, 16) && aligned(vq_codebooks, 16);
   if (w % 4 == 0 && D >= 256 && aligned(sq_codes, 4) && a16) {
     HybridDec<4> d{row_map, sq_codes, sq_params, param_stride, vq_codes, vq_codebooks, num_sq_rows, num_vq_rows, D, n_cb, k, w, nullptr};

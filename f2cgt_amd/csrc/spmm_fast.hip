@@ -464,6 +464,176 @@ int launch_acc(AccArgs a, const void* indptr, const void* indices, int idx_dtype
   return launch_status(what);
 }
 
+
+// ---- two-table hybrid (8-bit affine SQ rows + VQ rows), row-block form ----------------------
+// Same structure as sq_affine_acc_kernel<8>: SQ edges are gathered edge-parallel (32-bit lanes
+// over the 4-byte chunks of the code row) into 16-bit integer field accumulators in LDS.  The
+// (rare, by construction of the two-level scheme) VQ edges are added per output in edge order by
+// the lane that owns the output, reading the code byte and the codebook entry through L2, so the
+// 128 KB codebook does not pin the kernel to one workgroup per CU.
+//   out = (n_sq * min + scale * sum_sq(code) + sum_vq(codebook entry)) / deg
+struct HybArgs {
+  const int32_t* row_map;
+  const uint8_t* sq_codes;
+  const float* sq_params;
+  int64_t param_stride;
+  const uint8_t* vq_codes;
+  const float* vq_codebooks;
+  int64_t R, E, N, n_sq, n_vq;
+  int feat_dim, n_cb, K, w;
+  int rows_per_block, edge_batch;
+  int chunks, ch2;   // 4-column chunks per row; gather lanes per edge = pow2 >= chunks
+  uint32_t magic;
+};
+
+constexpr uint32_t kVqFlag = 0x80000000u;
+
+template <typename Idx>
+__global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx* __restrict__ indptr,
+                                                            const Idx* __restrict__ indices,
+                                                            float* __restrict__ out) {
+  constexpr int LIMIT = 257;
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint32_t* s_acc = reinterpret_cast<uint32_t*>(smem);                       // [RB][chunks][2]
+  float* s_par = reinterpret_cast<float*>(s_acc + (size_t)a.rows_per_block * a.chunks * 2);  // [chunks][8]
+  int* s_ptr = reinterpret_cast<int*>(s_par + (size_t)a.chunks * 8);         // [RB + 1]
+  int* s_nvq = s_ptr + a.rows_per_block + 4;                                 // [RB] VQ edges per row
+  uint32_t* s_row = reinterpret_cast<uint32_t*>(s_nvq + a.rows_per_block);   // [edge_batch] table row | flag
+  uint16_t* s_erow = reinterpret_cast<uint16_t*>(s_row + a.edge_batch);      // [edge_batch] local row
+
+  const int t = threadIdx.x;
+  const int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block;
+  const int nrows = (int)((a.R - row0) < a.rows_per_block ? (a.R - row0) : a.rows_per_block);
+  int64_t e0 = (int64_t)indptr[row0];
+  e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
+  for (int i = t; i <= nrows; i += kBlock) {
+    int64_t v = (int64_t)indptr[row0 + i];
+    v = v < e0 ? e0 : (v > a.E ? a.E : v);
+    s_ptr[i] = (int)(v - e0 > 0x7fffffff ? 0x7fffffff : v - e0);
+  }
+  for (int i = t; i < nrows * a.chunks; i += kBlock) reinterpret_cast<uint2*>(s_acc)[i] = make_uint2(0u, 0u);
+  for (int i = t; i < nrows; i += kBlock) s_nvq[i] = 0;
+  for (int i = t; i < a.feat_dim; i += kBlock) {
+    const int c4 = i >> 2, q = i & 3;
+    s_par[c4 * 8 + q] = a.sq_params[i];
+    s_par[c4 * 8 + 4 + q] = a.sq_params[a.param_stride + i];
+  }
+  __syncthreads();
+  const int ne = s_ptr[nrows];
+  const uint32_t* codes32 = reinterpret_cast<const uint32_t*>(a.sq_codes);
+  const int dwords_per_row = a.feat_dim >> 2;
+
+  // rows longer than the field capacity are summed directly in the epilogue (flag: all edges "VQ-like")
+  for (int eb = 0; eb < ne; eb += a.edge_batch) {
+    const int nb = (ne - eb) < a.edge_batch ? (ne - eb) : a.edge_batch;
+    if (eb) __syncthreads();
+    for (int i = t; i < nb; i += kBlock) {
+      const int64_t id = clamp_idx(indices[e0 + eb + i], a.N);
+      const int64_t m = (int64_t)a.row_map[id];
+      uint32_t v;
+      if (m >= 0) {
+        v = (uint32_t)(m < a.n_sq ? m : a.n_sq - 1);
+      } else {
+        const int64_t r = -m - 1;
+        v = (uint32_t)(r < a.n_vq ? r : a.n_vq - 1) | kVqFlag;
+      }
+      s_row[i] = v;
+      s_erow[i] = 0;
+    }
+    __syncthreads();
+    for (int r = t; r < nrows; r += kBlock) {
+      int b = s_ptr[r] - eb, e = s_ptr[r + 1] - eb;
+      const bool direct = s_ptr[r + 1] - s_ptr[r] > LIMIT;
+      b = b < 0 ? 0 : b;
+      e = e > nb ? nb : e;
+      int nvq = 0;
+      for (int k = b; k < e; ++k) {
+        s_erow[k] = (uint16_t)r;
+        if (direct) s_row[k] |= 0x40000000u;  // keep out of the integer accumulators
+        nvq += (s_row[k] >> 30) != 0;
+      }
+      if (e > b) s_nvq[r] += nvq;
+    }
+    __syncthreads();
+    const int j = t & (a.ch2 - 1);
+    const int gslot = t / a.ch2;
+    const int gslots = kBlock / a.ch2;
+    constexpr int U = 4;
+    for (int e = gslot; e < nb; e += gslots * U) {
+      uint32_t w[U], row[U], er[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        int ee = e + u * gslots;
+        ee = ee < nb ? ee : nb - 1;
+        row[u] = s_row[ee];
+        er[u] = s_erow[ee];
+        w[u] = 0;
+        if (j < a.chunks && (row[u] >> 30) == 0) w[u] = codes32[(int64_t)row[u] * dwords_per_row + j];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int ee = e + u * gslots;
+        if (ee < nb && j < a.chunks && (row[u] >> 30) == 0) {
+          uint32_t* acc = s_acc + (er[u] * a.chunks + j) * 2;
+          atomicAdd(acc + 0, w[u] & 0x00ff00ffu);
+          atomicAdd(acc + 1, (w[u] >> 8) & 0x00ff00ffu);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // finalize: lane <-> one float4 of the block's contiguous output span
+  const int items = nrows * a.chunks;
+  float* ob = out + row0 * (int64_t)a.feat_dim;
+  for (int it = t; it < items; it += kBlock) {
+    const int r = (int)__umulhi((uint32_t)it, a.magic);
+    const int c4 = it - r * a.chunks;
+    const uint2 q = *reinterpret_cast<const uint2*>(s_acc + (r * a.chunks + c4) * 2);
+    const int b = s_ptr[r], e = s_ptr[r + 1];
+    const int deg = e - b;
+    const int nvq = s_nvq[r];
+    const float nsq = (float)(deg - nvq);
+    const float4 mn = *reinterpret_cast<const float4*>(s_par + c4 * 8);
+    const float4 sc = *reinterpret_cast<const float4*>(s_par + c4 * 8 + 4);
+    float v0 = __fadd_rn(__fmul_rn(nsq, mn.x), __fmul_rn((float)(q.x & 0xffffu), sc.x));
+    float v1 = __fadd_rn(__fmul_rn(nsq, mn.y), __fmul_rn((float)(q.y & 0xffffu), sc.y));
+    float v2 = __fadd_rn(__fmul_rn(nsq, mn.z), __fmul_rn((float)(q.x >> 16), sc.z));
+    float v3 = __fadd_rn(__fmul_rn(nsq, mn.w), __fmul_rn((float)(q.y >> 16), sc.w));
+    if (nvq > 0) {  // the row's remaining edges, in edge order, straight from the tables
+      const int col = c4 * 4;
+      const int sub = col / a.w;
+      const int off = col - sub * a.w;
+      for (int k = b; k < e; ++k) {
+        const int64_t id = clamp_idx(indices[e0 + k], a.N);
+        const int64_t m = (int64_t)a.row_map[id];
+        if (m >= 0) {
+          if (deg <= LIMIT) continue;  // already in the integer accumulators
+          const int64_t row = m < a.n_sq ? m : a.n_sq - 1;
+          const uint32_t wv = codes32[row * dwords_per_row + c4];
+          v0 += __fadd_rn(mn.x, __fmul_rn((float)(wv & 0xffu), sc.x));
+          v1 += __fadd_rn(mn.y, __fmul_rn((float)((wv >> 8) & 0xffu), sc.y));
+          v2 += __fadd_rn(mn.z, __fmul_rn((float)((wv >> 16) & 0xffu), sc.z));
+          v3 += __fadd_rn(mn.w, __fmul_rn((float)(wv >> 24), sc.w));
+        } else {
+          int64_t row = -m - 1;
+          row = row < a.n_vq ? row : a.n_vq - 1;
+          int code = a.vq_codes[row * a.n_cb + sub];
+          code = code < a.K ? code : a.K - 1;
+          const float4 x = *reinterpret_cast<const float4*>(a.vq_codebooks + ((int64_t)sub * a.K + code) * a.w + off);
+          v0 += x.x; v1 += x.y; v2 += x.z; v3 += x.w;
+        }
+      }
+    }
+    if (deg > 1) {
+      const float d = (float)deg;
+      const float rdeg = __builtin_amdgcn_rcpf(d);
+      v0 *= rdeg; v1 *= rdeg; v2 *= rdeg; v3 *= rdeg;
+    }
+    if (deg <= 0) v0 = v1 = v2 = v3 = 0.f;
+    store_nt4(ob + (int64_t)it * 4, v0, v1, v2, v3);
+  }
+}
+
 }  // namespace
 
 bool sq_block_eligible(const void* codes, const float* out, int64_t N, int64_t src_dim, int feat_dim,
@@ -539,6 +709,47 @@ int sq_affine_acc_run(const uint8_t* codes, const float* params, int64_t param_s
   a.feat_dim = feat_dim;
   return target_bits == 4 ? launch_acc<4>(a, indptr, indices, idx_dtype, out, st, what)
                           : launch_acc<8>(a, indptr, indices, idx_dtype, out, st, what);
+}
+
+bool hybrid_acc_eligible(const void* sq_codes, const float* vq_codebooks, const float* out, int64_t N,
+                         int64_t n_sq, int64_t n_vq, int feat_dim, int w) {
+  if (!aligned(sq_codes, 4) || !aligned(out, 16) || !aligned(vq_codebooks, 16)) return false;
+  if (feat_dim < 4 || feat_dim % 4 != 0 || feat_dim > 1024 || w % 4 != 0) return false;
+  if (N >= (1ll << 32) || n_sq >= (1ll << 30) || n_vq >= (1ll << 30)) return false;
+  return true;
+}
+
+int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float* sq_params, int64_t param_stride,
+                   const uint8_t* vq_codes, const float* vq_codebooks, const void* indptr, const void* indices,
+                   int idx_dtype, float* out, int64_t R, int64_t E, int64_t N, int64_t n_sq, int64_t n_vq,
+                   int feat_dim, int n_cb, int K, int w, hipStream_t st, const char* what) {
+  HybArgs a{};
+  a.row_map = row_map; a.sq_codes = sq_codes; a.sq_params = sq_params; a.param_stride = param_stride;
+  a.vq_codes = vq_codes; a.vq_codebooks = vq_codebooks;
+  a.R = R; a.E = E; a.N = N; a.n_sq = n_sq; a.n_vq = n_vq;
+  a.feat_dim = feat_dim; a.n_cb = n_cb; a.K = K; a.w = w;
+  a.chunks = feat_dim / 4;
+  a.ch2 = pow2_ceil(a.chunks);
+  a.magic = (uint32_t)((0x100000000ull + a.chunks - 1) / a.chunks);
+  a.edge_batch = 384;
+  const double avg_deg = R > 0 ? (double)E / (double)R : 1.0;
+  const int want = (int)(200.0 / (avg_deg > 0.5 ? avg_deg : 0.5));
+  int rb = 8;
+  while (rb * 2 <= want && rb < 64) rb *= 2;
+  const size_t acc_row = (size_t)a.chunks * 8;
+  while (rb > 8 && rb * acc_row > 16 * 1024) rb /= 2;
+  a.rows_per_block = rb;
+  const size_t lds = rb * acc_row + (size_t)a.chunks * 32 + (size_t)(rb + 4) * 4 + (size_t)rb * 4 +
+                     (size_t)a.edge_batch * 6 + 16;
+  const int64_t grid = ceil_div(R, rb);
+  if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
+  if (idx_dtype == F2CGT_DT_I32)
+    hybrid_acc_kernel<int32_t><<<(unsigned)grid, kBlock, lds, st>>>(
+        a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
+  else
+    hybrid_acc_kernel<int64_t><<<(unsigned)grid, kBlock, lds, st>>>(
+        a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
+  return launch_status(what);
 }
 
 }  // namespace f2cgt
