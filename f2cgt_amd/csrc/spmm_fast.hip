@@ -488,7 +488,7 @@ struct HybArgs {
 
 constexpr uint32_t kVqFlag = 0x80000000u;
 
-template <typename Idx>
+template <typename Idx, int VEC>
 __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx* __restrict__ indptr,
                                                             const Idx* __restrict__ indices,
                                                             float* __restrict__ out) {
@@ -555,6 +555,47 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
       if (e > b) s_nvq[r] += nvq;
     }
     __syncthreads();
+    if (VEC == 4) {
+      // a lane takes 16 bytes (4 chunks) of an edge's code row: chunks / 4 lanes per edge
+      const int lanes = a.ch2 >> 2;
+      const int j = t & (lanes - 1);
+      const int gslot = t / lanes;
+      const int gslots = kBlock / lanes;
+      constexpr int U = 4;
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      const u32x4* codes128 = reinterpret_cast<const u32x4*>(a.sq_codes);
+      const int q_per_row = a.feat_dim >> 4;
+      // a lane group walks a contiguous run of edges (mostly one destination row), so the lane
+      // groups of a wave add into different accumulator rows and the LDS atomics do not collide
+      const int per = (nb + gslots - 1) / gslots;
+      const int e_begin = gslot * per;
+      const int e_end = (e_begin + per) < nb ? (e_begin + per) : nb;
+      for (int e = e_begin; e < e_end; e += U) {
+        u32x4 w[U];
+        uint32_t row[U], er[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          int ee = e + u;
+          ee = ee < e_end ? ee : e_end - 1;
+          row[u] = s_row[ee];
+          er[u] = s_erow[ee];
+          w[u] = u32x4{0u, 0u, 0u, 0u};
+          if (j < q_per_row && (row[u] >> 30) == 0) w[u] = codes128[(int64_t)row[u] * q_per_row + j];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int ee = e + u;
+          if (ee < e_end && j < q_per_row && (row[u] >> 30) == 0) {
+            uint32_t* acc = s_acc + (er[u] * a.chunks + 4 * j) * 2;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+              atomicAdd(acc + 2 * c, w[u][c] & 0x00ff00ffu);
+              atomicAdd(acc + 2 * c + 1, (w[u][c] >> 8) & 0x00ff00ffu);
+            }
+          }
+        }
+      }
+    } else {
     const int j = t & (a.ch2 - 1);
     const int gslot = t / a.ch2;
     const int gslots = kBlock / a.ch2;
@@ -580,6 +621,7 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
         }
       }
     }
+    }
   }
   __syncthreads();
   // finalize: lane <-> one float4 of the block's contiguous output span
@@ -603,11 +645,19 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
       const int col = c4 * 4;
       const int sub = col / a.w;
       const int off = col - sub * a.w;
+      const bool in_lds = ne <= a.edge_batch;  // one batch: s_row still describes every edge of the block
       for (int k = b; k < e; ++k) {
-        const int64_t id = clamp_idx(indices[e0 + k], a.N);
-        const int64_t m = (int64_t)a.row_map[id];
+        int64_t m;
+        if (in_lds) {
+          const uint32_t v = s_row[k];
+          if ((v >> 30) == 0) continue;  // SQ edge already in the integer accumulators
+          m = (v & kVqFlag) ? -(int64_t)(v & 0x3fffffffu) - 1 : (int64_t)(v & 0x3fffffffu);
+        } else {
+          const int64_t id = clamp_idx(indices[e0 + k], a.N);
+          m = (int64_t)a.row_map[id];
+          if (m >= 0 && deg <= LIMIT) continue;
+        }
         if (m >= 0) {
-          if (deg <= LIMIT) continue;  // already in the integer accumulators
           const int64_t row = m < a.n_sq ? m : a.n_sq - 1;
           const uint32_t wv = codes32[row * dwords_per_row + c4];
           v0 += __fadd_rn(mn.x, __fmul_rn((float)(wv & 0xffu), sc.x));
@@ -731,9 +781,9 @@ int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float*
   a.chunks = feat_dim / 4;
   a.ch2 = pow2_ceil(a.chunks);
   a.magic = (uint32_t)((0x100000000ull + a.chunks - 1) / a.chunks);
-  a.edge_batch = 384;
+  a.edge_batch = 1024;
   const double avg_deg = R > 0 ? (double)E / (double)R : 1.0;
-  const int want = (int)(200.0 / (avg_deg > 0.5 ? avg_deg : 0.5));
+  const int want = (int)(400.0 / (avg_deg > 0.5 ? avg_deg : 0.5));
   int rb = 8;
   while (rb * 2 <= want && rb < 64) rb *= 2;
   const size_t acc_row = (size_t)a.chunks * 8;
@@ -743,12 +793,18 @@ int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float*
                      (size_t)a.edge_batch * 6 + 16;
   const int64_t grid = ceil_div(R, rb);
   if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
-  if (idx_dtype == F2CGT_DT_I32)
-    hybrid_acc_kernel<int32_t><<<(unsigned)grid, kBlock, lds, st>>>(
-        a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
-  else
-    hybrid_acc_kernel<int64_t><<<(unsigned)grid, kBlock, lds, st>>>(
-        a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
+  const bool vec4 = feat_dim % 16 == 0 && aligned(sq_codes, 16) && a.ch2 >= 4;
+  const int32_t* ip32 = static_cast<const int32_t*>(indptr);
+  const int32_t* ix32 = static_cast<const int32_t*>(indices);
+  const int64_t* ip64 = static_cast<const int64_t*>(indptr);
+  const int64_t* ix64 = static_cast<const int64_t*>(indices);
+  if (idx_dtype == F2CGT_DT_I32) {
+    if (vec4) hybrid_acc_kernel<int32_t, 4><<<(unsigned)grid, kBlock, lds, st>>>(a, ip32, ix32, out);
+    else hybrid_acc_kernel<int32_t, 1><<<(unsigned)grid, kBlock, lds, st>>>(a, ip32, ix32, out);
+  } else {
+    if (vec4) hybrid_acc_kernel<int64_t, 4><<<(unsigned)grid, kBlock, lds, st>>>(a, ip64, ix64, out);
+    else hybrid_acc_kernel<int64_t, 1><<<(unsigned)grid, kBlock, lds, st>>>(a, ip64, ix64, out);
+  }
   return launch_status(what);
 }
 
