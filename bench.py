@@ -9,6 +9,11 @@ synchronisations); `roofline.achieved` is algorithmic bytes per launch divided b
 average launch duration measured with HIP events on the launch stream; `cpu_baseline`
 is the reference's unfused CPU flow (torch dequantise + torch sparse mm) timed on this
 box's host cores on a bounded sample of the same workload.
+
+    python bench.py --all            adds the other workloads and the streaming/encode ops
+                                     under "others" (same JSON line)
+    python bench.py --calibrate-copy runs plain device copies of a known size (for scaling the
+                                     rocprofv3 FETCH_SIZE / WRITE_SIZE counters), no JSON
 """
 import argparse
 import json
@@ -20,20 +25,131 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_F32_PEAK_TFLOPS = 157.3
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by the
-# same counters on a plain copy kernel of known size); see profiles/.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE, each scaled by
+# what the same counter reads for a plain copy of known size; see profiles/).  Keyed by
+# (workload name, index dtype).  Missing = not measured.
+MEASURED_TRAFFIC_BYTES = {
+    ("c1_sq8_affine", "int64"): 18279493,
+    ("c2_sq4_affine", "int64"): 132288366,
+    ("c3_vq_16x8", "int64"): 487431606,
+    ("c4_hybrid", "int64"): 1003788187,
+    ("c5_vq_24x32", "int64"): 3306912153,
+}
+
+
+def _launcher(capi, wl, out):
+    """Returns a zero-argument callable that enqueues one fused launch (pre-bound C ABI call)."""
+    import torch
+
+    lib = capi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    tag = capi.DT_I64 if wl["indptr"].dtype == torch.int64 else capi.DT_I32
+    R, E = wl["R"], wl["E"]
+    if wl["kind"] == "sq_affine":
+        c, p = wl["codes"], wl["params"]
+        args = (c.data_ptr(), p.data_ptr(), p.shape[1], wl["indptr"].data_ptr(), wl["indices"].data_ptr(), tag,
+                out.data_ptr(), R, E, c.shape[0], c.shape[1], wl["feat_dim"], wl["bits"], stream)
+        fn = lib.f2cgt_sq_affine_decompress_spmm_csr
+    elif wl["kind"] == "vq":
+        c, cb = wl["codes"], wl["codebooks"]
+        args = (c.data_ptr(), capi.DT_U8, cb.data_ptr(), wl["indptr"].data_ptr(), wl["indices"].data_ptr(), tag,
+                out.data_ptr(), R, E, c.shape[0], wl["feat_dim"], cb.shape[0], cb.shape[1], cb.shape[2], stream)
+        fn = lib.f2cgt_vq_decompress_spmm_csr
+    else:
+        cb = wl["vq_codebooks"]
+        args = (wl["row_map"].data_ptr(), wl["sq_codes"].data_ptr(), wl["sq_params"].data_ptr(),
+                wl["sq_params"].shape[1], wl["vq_codes"].data_ptr(), cb.data_ptr(), wl["indptr"].data_ptr(),
+                wl["indices"].data_ptr(), tag, out.data_ptr(), R, E, wl["row_map"].numel(),
+                wl["sq_codes"].shape[0], wl["vq_codes"].shape[0], wl["feat_dim"], cb.shape[0], cb.shape[1],
+                cb.shape[2], stream)
+        fn = lib.f2cgt_hybrid_decompress_spmm_csr
+
+    def step():
+        rc = fn(*args)
+        if rc != 0:
+            raise RuntimeError("launch failed (%d): %s" % (rc, lib.f2cgt_last_error().decode()))
+    return step
+
+
+def _time_steps(step, steps, warmup):
+    """-> (wall ms per step, HIP-event ms per launch)."""
+    import torch
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()           # torch's current stream: the one the C ABI launches on
+    for _ in range(steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall * 1e3 / steps, ev0.elapsed_time(ev1) / steps
+
+
+def _run_workload(name, idx, steps, warmup):
+    import torch
+    from f2cgt_amd import capi, synth
+
+    idx_dtype = torch.int64 if idx == "int64" else torch.int32
+    wl = synth.WORKLOADS[name](device="cuda", idx_dtype=idx_dtype)
+    out = torch.empty((wl["R"], wl["feat_dim"]), dtype=torch.float32, device="cuda")
+    ms_step, ms_launch = _time_steps(_launcher(capi, wl, out), steps, warmup)
+    return wl, ms_step, ms_launch
+
+
+def _others(idx):
+    """Secondary measurements: the remaining workloads, the encode step and the streaming ops."""
+    import torch
+    from f2cgt_amd import capi, synth
+
+    res = {}
+    for name, steps in (("c1", 2000), ("c3", 300), ("c4", 100), ("c5", 60)):
+        wl, ms_step, ms_launch = _run_workload(name, idx, steps, max(5, steps // 10))
+        gbs = wl["algo_bytes"] / (ms_launch * 1e-3) / 1e9
+        res[wl["name"]] = {"launch_us": ms_launch * 1e3, "edges_per_s": wl["E"] / (ms_step * 1e-3),
+                           "algorithmic_GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS}
+        del wl
+        torch.cuda.empty_cache()
+    enc = synth.c5_encode(device="cuda")
+    labels = torch.empty((enc["m"],), dtype=torch.uint8, device="cuda")
+    _, ms = _time_steps(lambda: capi.kmeans_predict(enc["x"], enc["centers"], "l2", u8=True, out=labels), 50, 5)
+    tf = enc["flops"] / (ms * 1e-3) / 1e12
+    res["c5_encode_l2_argmin"] = {"launch_us": ms * 1e3, "TFLOPps": tf, "frac_mfma_f32_peak": tf / MFMA_F32_PEAK_TFLOPS,
+                                  "vectors_per_s": enc["m"] / (ms * 1e-3)}
+    # streaming ops at the C2 table shape
+    n, d = 2_400_000, 100
+    codes = torch.randint(0, 16, (n, d), dtype=torch.uint8, device="cuda")
+    _, ms = _time_steps(lambda: capi.packbits(codes, 4), 50, 5)
+    res["packbits_4bit_2.4Mx100"] = {"launch_us": ms * 1e3, "GBps": n * d * 1.5 / (ms * 1e-3) / 1e9}
+    packed = capi.packbits(codes, 4)
+    _, ms = _time_steps(lambda: capi.unpackbits(packed, 4, d), 50, 5)
+    res["unpackbits_4bit_2.4Mx100"] = {"launch_us": ms * 1e3, "GBps": n * d * 1.5 / (ms * 1e-3) / 1e9}
+    params = torch.rand((2, d), device="cuda")
+    _, ms = _time_steps(lambda: capi.sq_affine_decompress(packed, params, 4, d), 20, 3)
+    res["sq_affine_decompress_4bit_2.4Mx100"] = {"launch_us": ms * 1e3, "GBps": n * d * 4.5 / (ms * 1e-3) / 1e9}
+    cb = torch.randn((16, 256, 8), device="cuda")
+    vq = torch.randint(0, 256, (n, 16), dtype=torch.uint8, device="cuda")
+    _, ms = _time_steps(lambda: capi.vq_decompress(vq, cb, 128), 20, 3)
+    res["vq_decompress_16x8_2.4M"] = {"launch_us": ms * 1e3, "GBps": n * (16 + 512) / (ms * 1e-3) / 1e9}
+    return res
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--idx", default="int64", choices=["int64", "int32"])
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the cpu_baseline leg (0 = skip)")
+    ap.add_argument("--all", action="store_true", help="also measure the other workloads and ops")
+    ap.add_argument("--calibrate-copy", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
@@ -41,43 +157,21 @@ def main():
         sys.exit(2)
 
     import torch
-    from f2cgt_amd import capi, synth
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
-    idx_dtype = torch.int64 if args.idx == "int64" else torch.int32
-    wl = synth.WORKLOADS[args.workload](device="cuda", idx_dtype=idx_dtype)
-    out = torch.empty((wl["R"], wl["feat_dim"]), dtype=torch.float32, device="cuda")
 
-    if wl["kind"] == "sq_affine":
-        def step():
-            capi.sq_affine_decompress_spmm_csr(wl["codes"], wl["params"], wl["indptr"], wl["indices"],
-                                               wl["bits"], wl["feat_dim"], out=out)
-    elif wl["kind"] == "vq":
-        def step():
-            capi.vq_decompress_spmm_csr(wl["codes"], wl["codebooks"], wl["indptr"], wl["indices"],
-                                        wl["feat_dim"], out=out)
-    else:
-        def step():
-            capi.hybrid_decompress_spmm_csr(wl["row_map"], wl["sq_codes"], wl["sq_params"], wl["vq_codes"],
-                                            wl["vq_codebooks"], wl["indptr"], wl["indices"], wl["feat_dim"],
-                                            out=out)
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print("calibration: 5 device copies of %d bytes each (read %d, write %d per dispatch)"
+              % (src.numel(), src.numel(), src.numel()))
+        return
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    ev0 = torch.cuda.Event(enable_timing=True)
-    ev1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    ev0.record()           # same stream the C ABI launches on (torch's current stream)
-    for _ in range(args.steps):
-        step()
-    ev1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    launch_ms = ev0.elapsed_time(ev1) / args.steps
-    ms_per_step = wall * 1e3 / args.steps
-
+    wl, ms_per_step, launch_ms = _run_workload(args.workload, args.idx, args.steps, args.warmup)
     achieved = wl["algo_bytes"] / (launch_ms * 1e-3) / 1e9
     traffic = MEASURED_TRAFFIC_BYTES.get((wl["name"], args.idx))
     result = {
@@ -121,6 +215,10 @@ def main():
                       "median of %d; unique+relabel (%.3f s) timed separately and excluded"
                       % (rows, wl["R"], edges, reps, relabel_secs),
         }
+    if args.all:
+        del wl
+        torch.cuda.empty_cache()
+        result["others"] = _others(args.idx)
     print(json.dumps(result))
 
 
