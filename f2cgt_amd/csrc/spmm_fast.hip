@@ -494,8 +494,11 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
                                                             float* __restrict__ out) {
   constexpr int LIMIT = 257;
   extern __shared__ __align__(16) unsigned char smem[];
-  uint32_t* s_acc = reinterpret_cast<uint32_t*>(smem);                       // [RB][chunks][2]
-  float* s_par = reinterpret_cast<float*>(s_acc + (size_t)a.rows_per_block * a.chunks * 2);  // [chunks][8]
+  // integer accumulators: [RB][plane 0: bytes 0,2 | plane 1: bytes 1,3][chunk], rows 8 words apart
+  // in bank space so that the lane groups of a wave (different rows) spread over all 32 banks
+  const int acc_pitch = 2 * a.chunks + 8;
+  uint32_t* s_acc = reinterpret_cast<uint32_t*>(smem);
+  float* s_par = reinterpret_cast<float*>(s_acc + (size_t)a.rows_per_block * acc_pitch);  // [chunks][8]
   int* s_ptr = reinterpret_cast<int*>(s_par + (size_t)a.chunks * 8);         // [RB + 1]
   int* s_nvq = s_ptr + a.rows_per_block + 4;                                 // [RB] VQ edges per row
   uint32_t* s_row = reinterpret_cast<uint32_t*>(s_nvq + a.rows_per_block);   // [edge_batch] table row | flag
@@ -511,7 +514,7 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
     v = v < e0 ? e0 : (v > a.E ? a.E : v);
     s_ptr[i] = (int)(v - e0 > 0x7fffffff ? 0x7fffffff : v - e0);
   }
-  for (int i = t; i < nrows * a.chunks; i += kBlock) reinterpret_cast<uint2*>(s_acc)[i] = make_uint2(0u, 0u);
+  for (int i = t; i < nrows * acc_pitch; i += kBlock) s_acc[i] = 0u;
   for (int i = t; i < nrows; i += kBlock) s_nvq[i] = 0;
   for (int i = t; i < a.feat_dim; i += kBlock) {
     const int c4 = i >> 2, q = i & 3;
@@ -562,16 +565,15 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
       const int gslot = t / lanes;
       const int gslots = kBlock / lanes;
       constexpr int U = 4;
-      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-      const u32x4* codes128 = reinterpret_cast<const u32x4*>(a.sq_codes);
-      const int q_per_row = a.feat_dim >> 4;
-      // a lane group walks a contiguous run of edges (mostly one destination row), so the lane
-      // groups of a wave add into different accumulator rows and the LDS atomics do not collide
+      // lane j of the lanes that share an edge takes dwords j, j+q, j+2q, j+3q (q = chunks / 4):
+      // every load and every atomic instruction touches q consecutive words per edge
       const int per = (nb + gslots - 1) / gslots;
       const int e_begin = gslot * per;
       const int e_end = (e_begin + per) < nb ? (e_begin + per) : nb;
+      const int q = a.chunks >> 2;   // dwords per lane stride (chunks is a multiple of 4 here)
+      const bool lane_on = j < q;
       for (int e = e_begin; e < e_end; e += U) {
-        u32x4 w[U];
+        uint32_t w[U][4];
         uint32_t row[U], er[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -579,18 +581,20 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
           ee = ee < e_end ? ee : e_end - 1;
           row[u] = s_row[ee];
           er[u] = s_erow[ee];
-          w[u] = u32x4{0u, 0u, 0u, 0u};
-          if (j < q_per_row && (row[u] >> 30) == 0) w[u] = codes128[(int64_t)row[u] * q_per_row + j];
+          const bool on = lane_on && (row[u] >> 30) == 0;
+          const uint32_t* src = codes32 + (int64_t)row[u] * dwords_per_row + j;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) w[u][c] = on ? src[c * q] : 0u;
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const int ee = e + u;
-          if (ee < e_end && j < q_per_row && (row[u] >> 30) == 0) {
-            uint32_t* acc = s_acc + (er[u] * a.chunks + 4 * j) * 2;
+          if (ee < e_end && lane_on && (row[u] >> 30) == 0) {
+            uint32_t* acc = s_acc + er[u] * acc_pitch + j;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-              atomicAdd(acc + 2 * c, w[u][c] & 0x00ff00ffu);
-              atomicAdd(acc + 2 * c + 1, (w[u][c] >> 8) & 0x00ff00ffu);
+              atomicAdd(acc + c * q, w[u][c] & 0x00ff00ffu);
+              atomicAdd(acc + a.chunks + c * q, (w[u][c] >> 8) & 0x00ff00ffu);
             }
           }
         }
@@ -615,9 +619,9 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
       for (int u = 0; u < U; ++u) {
         const int ee = e + u * gslots;
         if (ee < nb && j < a.chunks && (row[u] >> 30) == 0) {
-          uint32_t* acc = s_acc + (er[u] * a.chunks + j) * 2;
-          atomicAdd(acc + 0, w[u] & 0x00ff00ffu);
-          atomicAdd(acc + 1, (w[u] >> 8) & 0x00ff00ffu);
+          uint32_t* acc = s_acc + er[u] * acc_pitch + j;
+          atomicAdd(acc, w[u] & 0x00ff00ffu);
+          atomicAdd(acc + a.chunks, (w[u] >> 8) & 0x00ff00ffu);
         }
       }
     }
@@ -630,7 +634,9 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
   for (int it = t; it < items; it += kBlock) {
     const int r = (int)__umulhi((uint32_t)it, a.magic);
     const int c4 = it - r * a.chunks;
-    const uint2 q = *reinterpret_cast<const uint2*>(s_acc + (r * a.chunks + c4) * 2);
+    uint2 q;
+    q.x = s_acc[r * acc_pitch + c4];
+    q.y = s_acc[r * acc_pitch + a.chunks + c4];
     const int b = s_ptr[r], e = s_ptr[r + 1];
     const int deg = e - b;
     const int nvq = s_nvq[r];
@@ -786,7 +792,7 @@ int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float*
   const int want = (int)(400.0 / (avg_deg > 0.5 ? avg_deg : 0.5));
   int rb = 8;
   while (rb * 2 <= want && rb < 64) rb *= 2;
-  const size_t acc_row = (size_t)a.chunks * 8;
+  const size_t acc_row = (size_t)(2 * a.chunks + 8) * 4;
   while (rb > 8 && rb * acc_row > 16 * 1024) rb /= 2;
   a.rows_per_block = rb;
   const size_t lds = rb * acc_row + (size_t)a.chunks * 32 + (size_t)(rb + 4) * 4 + (size_t)rb * 4 +
