@@ -350,15 +350,15 @@ __global__ __launch_bounds__(kBlock) void sq_affine_acc_kernel(AccArgs a, const 
     if (eb) __syncthreads();
     for (int i = t; i < nb; i += kBlock) {
       const uint64_t start = (uint64_t)clamp_idx(indices[e0 + eb + i], a.N) * (uint32_t)a.src_dim;
+      // local row of edge eb + i: the last r with s_ptr[r] <= eb + i (binary search, s_ptr is sorted)
+      const int pos = eb + i;
+      int lo = 0, hi = nrows;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (s_ptr[mid] <= pos) lo = mid; else hi = mid;
+      }
       s_row[i] = (uint32_t)(start >> 2);
-      s_erow[i] = (uint16_t)((start & 3) << 14);
-    }
-    __syncthreads();
-    for (int r = t; r < nrows; r += kBlock) {  // tag every edge of the batch with its local row
-      int b = s_ptr[r] - eb, e = s_ptr[r + 1] - eb;
-      b = b < 0 ? 0 : b;
-      e = e > nb ? nb : e;
-      for (int k = b; k < e; ++k) s_erow[k] |= (uint16_t)r;
+      s_erow[i] = (uint16_t)(((start & 3) << 14) | (uint32_t)lo);
     }
     __syncthreads();
     const int j = t & (a.dw2 - 1);
