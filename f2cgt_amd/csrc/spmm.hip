@@ -641,7 +641,7 @@ extern "C" int f2cgt_vq_decompress_spmm_csr(const void* codes, int code_dtype, c
   hipStream_t st = as_stream(stream);
   const int D = (int)feat_dim, n_cb = (int)num_codebooks, k = (int)K, w = (int)width;
   if (code_dtype == F2CGT_DT_U8 &&
-      vq_pipe_eligible(codes, codebooks, out, num_rows, num_src_rows, D, n_cb, k, w))
+      vq_pipe_eligible(codes, codebooks, out, num_rows, num_edges, num_src_rows, D, n_cb, k, w))
     return vq_pipe_run(static_cast<const uint8_t*>(codes), codebooks, indptr, indices, idx_dtype, out, num_rows,
                        num_edges, num_src_rows, D, n_cb, k, w, st, what);
   switch (code_dtype) {

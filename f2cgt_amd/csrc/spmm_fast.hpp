@@ -30,8 +30,8 @@ int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float*
                    int feat_dim, int n_cb, int K, int w, hipStream_t st, const char* what);
 
 // Persistent software-pipelined VQ kernel (uint8 codes, K <= 256, width 8/16/32), vq_fast.hip.
-bool vq_pipe_eligible(const void* codes, const float* codebooks, const float* out, int64_t R, int64_t N,
-                      int feat_dim, int n_cb, int K, int w);
+bool vq_pipe_eligible(const void* codes, const float* codebooks, const float* out, int64_t R, int64_t E,
+                      int64_t N, int feat_dim, int n_cb, int K, int w);
 int vq_pipe_run(const uint8_t* codes, const float* codebooks, const void* indptr, const void* indices,
                 int idx_dtype, float* out, int64_t R, int64_t E, int64_t N, int feat_dim, int n_cb, int K, int w,
                 hipStream_t st, const char* what);

@@ -56,11 +56,11 @@ struct VqPipe {
   using CW = typename code_word<BT>::type;
   // register state, two generations per stage
   int64_t Pa, Pb, P0a, P0b;
-  uint32_t Ia, Ib;
+  int64_t Ia, Ib;
   CW Ca, Cb;
   template <int G> __device__ __forceinline__ int64_t& Pr() { if constexpr (G == 0) return Pa; else return Pb; }
   template <int G> __device__ __forceinline__ int64_t& P0r() { if constexpr (G == 0) return P0a; else return P0b; }
-  template <int G> __device__ __forceinline__ uint32_t& Ir() { if constexpr (G == 0) return Ia; else return Ib; }
+  template <int G> __device__ __forceinline__ int64_t& Ir() { if constexpr (G == 0) return Ia; else return Ib; }
   template <int G> __device__ __forceinline__ CW& Cr() { if constexpr (G == 0) return Ca; else return Cb; }
 
   const VqArgs& a;
@@ -83,62 +83,69 @@ struct VqPipe {
     return (int)((a.R - row0) < kRows ? (a.R - row0) : kRows);
   }
 
+  // Block-uniform values read back from LDS are moved to scalar registers so that the stage
+  // bookkeeping runs on the scalar unit and only the per-lane load/store remains vector work.
+  __device__ __forceinline__ int uniform_ne(int64_t b) const {
+    return __builtin_amdgcn_readfirstlane(s_ptr[(int)(b & (kRing - 1)) * (kRows + 2) + kRows + 1]);
+  }
+  __device__ __forceinline__ int64_t uniform_e0(int64_t b) const {
+    const int64_t v = s_e0[b & (kRing - 1)];
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+  }
+
   template <int PAR>
   __device__ __forceinline__ void iteration(int64_t it) {
     // ---- issue the three prefetch stages ---------------------------------------------------
-    {
-      const int64_t b = it + 2;  // C: code bytes, address from the id this lane fetched at b-4
-      if (valid(b)) {
-        const int ne = s_ptr[(b & (kRing - 1)) * (kRows + 2) + kRows + 1];
-        if (t < ne && ne <= kEdgeCap)
-          Cr<PAR>() = *reinterpret_cast<const CW*>(a.codes + (int64_t)Ir<PAR>() * a.n_cb + tile * BT);
-      }
+    // Every wave issues exactly three loads per iteration (lanes without work read a harmless
+    // valid address), and nothing here consumes a loaded value at once, so the memory counter
+    // waits the compiler inserts are "all but the last few", never a full drain.
+    {  // C: code bytes of edge t of block it+2; the id was fetched at it-2 and is clamped only now
+      const int ne = valid(it + 2) ? uniform_ne(it + 2) : 0;
+      const bool on = ne <= kEdgeCap && t < ne;
+      const uint64_t raw = (uint64_t)Ir<PAR>();
+      const uint64_t id = raw < (uint64_t)a.N ? raw : (uint64_t)(a.N - 1);
+      const uint8_t* src = a.codes + (on ? id * (uint32_t)a.n_cb : 0) + tile * BT;
+      Cr<PAR>() = *reinterpret_cast<const CW*>(src);
     }
-    {
-      const int64_t b = it + 4;  // I: source id of edge t
-      if (valid(b)) {
-        const int slot = (int)(b & (kRing - 1));
-        const int ne = s_ptr[slot * (kRows + 2) + kRows + 1];
-        if (t < ne && ne <= kEdgeCap) Ir<PAR>() = (uint32_t)clamp_idx(indices[s_e0[slot] + t], a.N);
-      }
+    {  // I: source id of edge t of block it+4 (raw; ids outside [0, N) read row N-1)
+      const bool v = valid(it + 4);
+      const int ne = v ? uniform_ne(it + 4) : 0;
+      const bool on = ne <= kEdgeCap && t < ne;
+      const int64_t e0 = v ? uniform_e0(it + 4) : 0;
+      const Idx* src = on ? indices + e0 + t : indptr;
+      Ir<PAR>() = (int64_t)*src;
     }
-    {
-      const int64_t b = it + 6;  // P: row offsets
-      if (valid(b)) {
-        const int64_t row0 = global_block(b) * kRows;
-        const int nr = rows_of(b);
-        P0r<PAR>() = (int64_t)indptr[row0];
-        if (t <= nr) Pr<PAR>() = (int64_t)indptr[row0 + t];
-      }
+    {  // P: row offsets of block it+6
+      const bool v = valid(it + 6);
+      const int64_t row0 = v ? global_block(it + 6) * kRows : 0;
+      const int nr = v ? rows_of(it + 6) : 0;
+      P0r<PAR>() = (int64_t)indptr[row0];
+      Pr<PAR>() = (int64_t)indptr[row0 + (t <= nr ? t : 0)];
     }
     // ---- compute block `it` ------------------------------------------------------------------
     if (valid(it)) compute(it);
     __syncthreads();
     // ---- park what was issued one iteration ago ------------------------------------------------
-    {
-      const int64_t b = it + 1;  // C issued at it-1 lives in C[PAR ^ 1]
-      if (valid(b)) {
-        const int ne = s_ptr[(b & (kRing - 1)) * (kRows + 2) + kRows + 1];
-        if (t < ne && ne <= kEdgeCap) *reinterpret_cast<CW*>(s_codes + t * BT) = Cr<PAR ^ 1>();
-      }
+    if (valid(it + 1)) {  // C issued at it-1 lives in the other generation
+      const int ne = uniform_ne(it + 1);
+      if (ne <= kEdgeCap && t < ne) *reinterpret_cast<CW*>(s_codes + t * BT) = Cr<PAR ^ 1>();
     }
-    {
-      const int64_t b = it + 5;  // P issued at it-1 lives in P[PAR ^ 1]
-      if (valid(b)) {
-        const int slot = (int)(b & (kRing - 1));
-        const int nr = rows_of(b);
-        int64_t e0 = P0r<PAR ^ 1>();
-        e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
-        if (t <= nr) {
-          int64_t v = Pr<PAR ^ 1>();
-          v = v < e0 ? e0 : (v > a.E ? a.E : v);
-          const int64_t rel = v - e0;
-          const int r32 = rel > 0x3fffffff ? 0x3fffffff : (int)rel;
-          s_ptr[slot * (kRows + 2) + t] = r32;
-          if (t == nr) s_ptr[slot * (kRows + 2) + kRows + 1] = r32;
-        }
-        if (t == 0) s_e0[slot] = e0;
+    if (valid(it + 5)) {  // P issued at it-1
+      const int slot = (int)((it + 5) & (kRing - 1));
+      const int nr = rows_of(it + 5);
+      int64_t e0 = P0r<PAR ^ 1>();
+      e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
+      if (t <= nr) {
+        int64_t v = Pr<PAR ^ 1>();
+        v = v < e0 ? e0 : (v > a.E ? a.E : v);
+        const int64_t rel = v - e0;
+        const int r32 = rel > 0x3fffffff ? 0x3fffffff : (int)rel;
+        s_ptr[slot * (kRows + 2) + t] = r32;
+        if (t == nr) s_ptr[slot * (kRows + 2) + kRows + 1] = r32;
       }
+      if (t == 0) s_e0[slot] = e0;
     }
     __syncthreads();
   }
@@ -153,7 +160,7 @@ struct VqPipe {
     const int nr = rows_of(b);
     const int tile_cols = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
     if (c4 * 4 >= tile_cols) return;
-    const int ne = sp[kRows + 1];
+    const int ne = __builtin_amdgcn_readfirstlane(sp[kRows + 1]);
     const int byte_idx = (c4 * 4) / a.w;
     const float* cbp = s_cb + c4 * 4;
     const bool staged = ne <= kEdgeCap;
@@ -276,8 +283,9 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
 
 }  // namespace
 
-bool vq_pipe_eligible(const void* codes, const float* codebooks, const float* out, int64_t R, int64_t N,
-                      int feat_dim, int n_cb, int K, int w) {
+bool vq_pipe_eligible(const void* codes, const float* codebooks, const float* out, int64_t R, int64_t E,
+                      int64_t N, int feat_dim, int n_cb, int K, int w) {
+  if (E < 1 || N < 1 || codes == nullptr) return false;  // idle lanes read row 0 / indptr[0]
   if (K < 1 || K > 256) return false;
   if (w != 8 && w != 16 && w != 32) return false;
   const int bt = 128 / w;
