@@ -238,42 +238,46 @@ int launch_sq_block(SqBlockArgs a, const void* indptr, const void* indices, int 
 
 // ---- affine SQ, 4- and 8-bit codes: integer accumulation in LDS ----------------------------
 // sum_e (min + c_e * scale) / deg == min + scale * (sum_e c_e) / deg, and the code sum is an
-// exact integer.  The block keeps per (row, 4 packed bytes) integer accumulators in LDS with the
-// codes widened to 16-bit fields (nibble k of each half-word -> accumulator k at 4 bits; even /
-// odd bytes -> accumulator 0 / 1 at 8 bits).  The gather is edge-parallel: one lane per aligned
-// dword of each edge's code row, realigned in registers (rows are only byte aligned in general:
-// src_dim = 50 at 4 bits x 100 columns), split into fields and added with LDS atomics, so there
-// is no per-row loop and no divergence.  The float work (convert, * 1/deg, * scale, + min) runs
-// once per output, one float4 of the block's contiguous output span per lane.  The result
-// differs from "decode, then sum in fp32" by a few ulp of the summands (it is the closer of the
-// two to the exact mean) and is identical to the decode for rows with one neighbour.
-//
-// Field capacity bounds the in-degree a row may have on this path (4369 at 4 bits, 257 at 8);
-// a block containing a larger row takes the direct per-output loop below instead.
+// exact integer.  The block keeps integer accumulators in LDS with the codes of a dword spread
+// over fields wide enough that no field can carry into its neighbour:
+//     4-bit codes, every row of the block <= 17 edges : 8-bit fields, 2 words per code dword
+//     4-bit codes, <= 4369 edges per row              : 16-bit fields, 4 words per code dword
+//     8-bit codes, <= 257 edges per row               : 16-bit fields, 2 words per code dword
+// The gather is edge-parallel: a lane takes 8 bytes of an edge's code row with one (byte-granular,
+// the hardware handles unaligned global loads) 64-bit load, splits them into fields with a few
+// mask/shift operations and adds them with LDS atomics -- no per-row loop, no divergence, and
+// the instruction count per edge is what bounds this kernel, not HBM.  The float work (convert,
+// * 1/deg, * scale, + min) runs once per output with the column parameters held in registers.
+// The result differs from "decode, then sum in fp32" by a few ulp of the summands (it is the
+// closer of the two to the exact mean) and is identical to the decode for rows with one neighbour.
+// A block with a row above the widest field capacity takes the direct per-output loop instead.
 struct AccArgs {
   const uint8_t* codes;
   const float* params;
   int64_t param_stride;
   int64_t R, E, N;
-  int64_t table_bytes;
   int src_dim, feat_dim;
-  int rows_per_block;
+  int rows_per_block;  // destination rows per workgroup
+  int sub_rows;        // rows that go through the accumulators at a time
   int edge_batch;
-  int dwords;        // aligned dwords that cover any row
-  int dw2;           // gather lanes per edge = pow2 >= dwords
-  int chunks;        // 4-byte column chunks per row that hold output columns
+  int eff_bytes;     // leading bytes of a code row that hold output columns
+  int lanes;         // 8-byte gather lanes per edge
+  int lane_shift;    // log2 of the lane-group size (pow2 >= lanes)
+  int pitch_n;       // accumulator words per row with 2 words per code dword
+  int pitch_w;       // ... with 4 words per code dword (4-bit codes, 16-bit fields)
   int f4_per_row;    // feat_dim / 4
-  uint32_t magic;    // ceil(2^32 / f4_per_row)
-  uint32_t last_full_dword;
+  int fin_group;     // finalize: lanes per row (min(f4_per_row, block))
+  int fin_slots;     // finalize: rows per pass
+  uint32_t fin_magic;  // ceil(2^16 / fin_group)
 };
 
-template <int BITS>
+template <int TB, int BITS>
 __device__ __forceinline__ void acc_direct_block(const AccArgs& a, const int* s_ptr, int64_t e0, int64_t row0,
                                               int nrows, const int64_t* idx64, const int32_t* idx32,
                                               float* __restrict__ out) {
   constexpr int PER = 8 / BITS;
   const int items = nrows * a.feat_dim;
-  for (int it = threadIdx.x; it < items; it += kBlock) {
+  for (int it = threadIdx.x; it < items; it += TB) {
     const int r = it / a.feat_dim, col = it - r * a.feat_dim;
     const int64_t b = e0 + s_ptr[r], e = e0 + s_ptr[r + 1];
     uint64_t tot = 0;
@@ -285,183 +289,287 @@ __device__ __forceinline__ void acc_direct_block(const AccArgs& a, const int* s_
     const int64_t deg = e - b;
     const float rdeg = __builtin_amdgcn_rcpf((float)(deg > 1 ? deg : 1));
     const float v = __fadd_rn(a.params[col], __fmul_rn((float)tot * rdeg, a.params[a.param_stride + col]));
-    out[(row0 + r) * (int64_t)a.feat_dim + col] = deg == 0 ? 0.f : v;
+    out[(row0 + r) * (int64_t)a.feat_dim + col] = deg <= 0 ? 0.f : v;
   }
 }
 
-template <int BITS, typename Idx>
-__global__ __launch_bounds__(kBlock) void sq_affine_acc_kernel(AccArgs a, const Idx* __restrict__ indptr,
+// ---- building blocks of the integer-accumulating kernel ----
+// NW = accumulator words per code dword (see the table above).
+
+template <int TB>
+__device__ __forceinline__ void acc_zero(uint32_t* s_acc, int words) {
+  for (int i = threadIdx.x; i < words >> 2; i += TB)
+    reinterpret_cast<uint4*>(s_acc)[i] = make_uint4(0u, 0u, 0u, 0u);
+}
+
+// s_edge[i] = {source row id, local row} for the edges [eb, eb + nb) of the block (positions are
+// relative to the block's first edge).  The ids are written edge-parallel; the local row of an
+// edge is written by the thread of that row (rows [0, nr) whose range is ptr[r] .. ptr[r + 1]).
+template <int TB, typename Idx>
+__device__ __forceinline__ void acc_tag(const AccArgs& a, const int* ptr, int nr, int eb, int nb, int64_t e0,
+                                        const Idx* __restrict__ indices, uint2* s_edge) {
+  uint32_t* flat = reinterpret_cast<uint32_t*>(s_edge);
+  for (int i = threadIdx.x; i < nb; i += TB)
+    flat[2 * i] = (uint32_t)clamp_idx(indices[e0 + eb + i], a.N);
+  for (int r = threadIdx.x; r < nr; r += TB) {
+    int b = ptr[r] - eb, e = ptr[r + 1] - eb;
+    b = b < 0 ? 0 : b;
+    e = e > nb ? nb : e;
+    for (int k = b; k < e; ++k) flat[2 * k + 1] = (uint32_t)r;
+  }
+}
+
+// Adds the code fields of the tagged edges s_edge[i0 .. i1) to the accumulators; an edge of local
+// row y goes to accumulator row y - row_base.
+template <int TB, int BITS, int NW>
+__device__ __forceinline__ void acc_gather(const AccArgs& a, uint32_t* s_acc, const uint2* s_edge, int i0, int i1,
+                                           int row_base, int pitch) {
+  constexpr uint32_t M = NW == 4 ? 0x000f000fu : (BITS == 4 ? 0x0f0f0f0fu : 0x00ff00ffu);
+  constexpr int S = BITS == 4 ? 4 : 8;  // shift between the words of one code dword
+  const int t = threadIdx.x;
+  const int lanes = a.lanes;
+  // lane j of a group covers row bytes [8j, 8j+8); the last lane's load is moved back so that it
+  // ends with the row's useful bytes, and shifted so that everything past them reads as 0
+  const int j = t & ((1 << a.lane_shift) - 1);
+  const int gslot = t >> a.lane_shift;
+  const int gslots = TB >> a.lane_shift;
+  const bool lane_on = j < lanes;
+  const int want_off = lane_on ? 8 * j : 0;
+  const int off = want_off < a.eff_bytes - 8 ? want_off : a.eff_bytes - 8;
+  const int sh = (want_off - off) * 8;
+  uint32_t* accj = s_acc + j - row_base * pitch;
+  constexpr int U = 4;
+  if (!lane_on) return;
+  uint32_t keep = 0;
+  for (int e = i0 + gslot; e < i1; e += gslots * U) {
+    uint2 ed[U];
+    uint64_t w[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int ee = e + u * gslots;
+      ee = ee < i1 ? ee : i1 - 1;
+      ed[u] = s_edge[ee];
+      __builtin_memcpy(&w[u], a.codes + ((uint64_t)ed[u].x * (uint32_t)a.src_dim + (uint32_t)off), 8);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      // The unconditional use keeps every load up here, issued back to back; a load whose only
+      // use sits in the branch below is moved into it by the compiler and waited for on its own.
+      keep ^= (uint32_t)w[u];
+      if (u == 0 || e + u * gslots < i1) {
+        const uint64_t v = w[u] >> sh;
+        const uint32_t d0 = (uint32_t)v, d1 = (uint32_t)(v >> 32);
+        uint32_t* acc = accj + (int)ed[u].y * pitch;
+#pragma unroll
+        for (int k = 0; k < NW; ++k) {
+          atomicAdd(acc + k * lanes, (d0 >> (S * k)) & M);
+          atomicAdd(acc + (NW + k) * lanes, (d1 >> (S * k)) & M);
+        }
+      }
+    }
+  }
+  if (keep == 0x9e3779b9u && a.eff_bytes < 0) s_acc[0] = keep;  // never true; gives `keep` a use
+}
+
+// Means of the rows [rb, rb + nr) of the block from the accumulator rows [0, nr): a lane keeps
+// one float4 column group (its parameters in registers) and walks the rows.
+template <int TB, int BITS, int NW>
+__device__ __forceinline__ void acc_finalize(const AccArgs& a, const uint32_t* s_acc, const float* s_rdeg,
+                                             int64_t row0, int rb, int nr, int pitch, float* __restrict__ out) {
+  const int t = threadIdx.x;
+  const int lanes = a.lanes;
+  const int g = (int)(((uint32_t)t * a.fin_magic) >> 16);
+  const int l = t - g * a.fin_group;
+  if (g >= a.fin_slots) return;
+  for (int c4 = l; c4 < a.f4_per_row; c4 += a.fin_group) {
+    float mn[4], sc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      mn[i] = a.params[c4 * 4 + i];
+      sc[i] = a.params[a.param_stride + c4 * 4 + i];
+    }
+    const int d = BITS == 4 ? (c4 >> 1) : c4;     // code dword that holds these 4 columns
+    const int fsh = BITS == 4 ? (c4 & 1) * 16 : 0;
+    const uint32_t* accd = s_acc + ((d & 1) * NW) * lanes + (d >> 1);
+    float* o = out + ((row0 + rb) * (int64_t)a.feat_dim + c4 * 4);
+    for (int r = g; r < nr; r += a.fin_slots) {
+      const uint32_t* ar = accd + r * pitch;
+      float s0, s1, s2, s3;
+      if (NW == 4) {
+        s0 = (float)((ar[0] >> fsh) & 0xffffu);
+        s1 = (float)((ar[lanes] >> fsh) & 0xffffu);
+        s2 = (float)((ar[2 * lanes] >> fsh) & 0xffffu);
+        s3 = (float)((ar[3 * lanes] >> fsh) & 0xffffu);
+      } else if (BITS == 4) {
+        const uint32_t w0 = ar[0] >> fsh, w1 = ar[lanes] >> fsh;
+        s0 = (float)(w0 & 0xffu);
+        s1 = (float)(w1 & 0xffu);
+        s2 = (float)((w0 >> 8) & 0xffu);
+        s3 = (float)((w1 >> 8) & 0xffu);
+      } else {
+        const uint32_t w0 = ar[0], w1 = ar[lanes];
+        s0 = (float)(w0 & 0xffffu);
+        s1 = (float)(w1 & 0xffffu);
+        s2 = (float)(w0 >> 16);
+        s3 = (float)(w1 >> 16);
+      }
+      const float rdeg = s_rdeg[rb + r];  // 0 marks an empty row, rcp(1) == 1 exactly
+      float v0 = __fadd_rn(mn[0], __fmul_rn(s0 * rdeg, sc[0]));
+      float v1 = __fadd_rn(mn[1], __fmul_rn(s1 * rdeg, sc[1]));
+      float v2 = __fadd_rn(mn[2], __fmul_rn(s2 * rdeg, sc[2]));
+      float v3 = __fadd_rn(mn[3], __fmul_rn(s3 * rdeg, sc[3]));
+      if (rdeg == 0.f) v0 = v1 = v2 = v3 = 0.f;
+      // plain stores: rows are not cache-line multiples in general, and the L2 merges the partial
+      // lines that neighbouring waves write before they go to HBM
+      *reinterpret_cast<float4*>(o + (int64_t)r * a.feat_dim) = make_float4(v0, v1, v2, v3);
+    }
+  }
+}
+
+// All rows of the block, `sub` rows at a time through the accumulators.
+template <int TB, int BITS, int NW, typename Idx>
+__device__ __forceinline__ void acc_block(const AccArgs& a, uint32_t* s_acc, const int* s_ptr, const float* s_rdeg,
+                                          uint2* s_edge, int64_t e0, int64_t row0, int nrows,
+                                          const Idx* __restrict__ indices, float* __restrict__ out) {
+  const int pitch = NW == 4 ? a.pitch_w : a.pitch_n;
+  const int sub = NW == 4 ? a.sub_rows >> 1 : a.sub_rows;
+  const int ne = s_ptr[nrows];
+  if (ne <= a.edge_batch) {
+    // common case: every edge of the block is tagged once, up front
+    acc_tag<TB>(a, s_ptr, nrows, 0, ne, e0, indices, s_edge);
+    acc_zero<TB>(s_acc, (nrows < sub ? nrows : sub) * pitch);
+    __syncthreads();
+    for (int sb = 0; sb < nrows; sb += sub) {
+      const int nr = (nrows - sb) < sub ? (nrows - sb) : sub;
+      acc_gather<TB, BITS, NW>(a, s_acc, s_edge, s_ptr[sb], s_ptr[sb + nr], sb, pitch);
+      __syncthreads();
+      acc_finalize<TB, BITS, NW>(a, s_acc, s_rdeg, row0, sb, nr, pitch, out);
+      if (sb + sub < nrows) {
+        __syncthreads();
+        acc_zero<TB>(s_acc, sub * pitch);
+        __syncthreads();
+      }
+    }
+  } else {
+    for (int sb = 0; sb < nrows; sb += sub) {
+      const int nr = (nrows - sb) < sub ? (nrows - sb) : sub;
+      const int* ptr = s_ptr + sb;
+      if (sb) __syncthreads();
+      acc_zero<TB>(s_acc, nr * pitch);
+      for (int eb = ptr[0]; eb < ptr[nr]; eb += a.edge_batch) {
+        const int nb = (ptr[nr] - eb) < a.edge_batch ? (ptr[nr] - eb) : a.edge_batch;
+        if (eb != ptr[0]) __syncthreads();
+        acc_tag<TB>(a, ptr, nr, eb, nb, e0, indices, s_edge);
+        __syncthreads();
+        acc_gather<TB, BITS, NW>(a, s_acc, s_edge, 0, nb, 0, pitch);
+      }
+      __syncthreads();
+      acc_finalize<TB, BITS, NW>(a, s_acc, s_rdeg, row0, sb, nr, pitch, out);
+    }
+  }
+}
+
+template <int TB, int BITS, typename Idx>
+__global__ __launch_bounds__(TB) void sq_affine_acc_kernel(AccArgs a, const Idx* __restrict__ indptr,
                                                                const Idx* __restrict__ indices,
                                                                float* __restrict__ out) {
-  constexpr int NACC = BITS == 4 ? 4 : 2;             // accumulator words per chunk
-  constexpr int LIMIT = BITS == 4 ? 4369 : 257;       // edges per row before a 16-bit field can wrap
+  constexpr int CAP_N = BITS == 4 ? 17 : 257;     // edges per row: 2 accumulator words per code dword
+  constexpr int CAP_W = BITS == 4 ? 4369 : 257;   // 4 words per code dword (4-bit codes only)
   extern __shared__ __align__(16) unsigned char smem[];
-  uint32_t* s_acc = reinterpret_cast<uint32_t*>(smem);                              // [RB][chunks][NACC]
-  float* s_par = reinterpret_cast<float*>(s_acc + (size_t)a.rows_per_block * a.chunks * NACC);  // [f4][8]
-  int* s_ptr = reinterpret_cast<int*>(s_par + (size_t)a.f4_per_row * 8);            // [RB + 1] (+ flag, tail)
-  uint32_t* s_row = reinterpret_cast<uint32_t*>(s_ptr + a.rows_per_block + 4);      // [edge_batch]
-  uint16_t* s_erow = reinterpret_cast<uint16_t*>(s_row + a.edge_batch);             // [edge_batch]
-  int* s_flag = s_ptr + a.rows_per_block + 1;
-  uint32_t* s_tail = reinterpret_cast<uint32_t*>(s_ptr + a.rows_per_block + 2);
+  uint32_t* s_acc = reinterpret_cast<uint32_t*>(smem);                         // [sub_rows][pitch_n]
+  int* s_ptr = reinterpret_cast<int*>(s_acc + (size_t)a.sub_rows * a.pitch_n);  // [RB + 1]
+  float* s_rdeg = reinterpret_cast<float*>(s_ptr + a.rows_per_block + 4);      // [RB]
+  uint32_t* s_wflag = reinterpret_cast<uint32_t*>(s_rdeg + a.rows_per_block);  // [waves]
+  uint2* s_edge = reinterpret_cast<uint2*>(s_wflag + 4);          // [edge_batch]
 
   const int t = threadIdx.x;
   const int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block;
   const int nrows = (int)((a.R - row0) < a.rows_per_block ? (a.R - row0) : a.rows_per_block);
   int64_t e0 = (int64_t)indptr[row0];
   e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
-  if (t == 0) {
-    *s_flag = 0;
-    uint32_t tail = 0;  // the bytes of the last, partial dword of the table (if any)
-    for (int64_t b = (int64_t)(a.last_full_dword + 1) * 4, i = 0; b < a.table_bytes && i < 4; ++b, ++i)
-      tail |= (uint32_t)a.codes[b] << (8 * i);
-    *s_tail = tail;
-  }
-  for (int i = t; i <= nrows; i += kBlock) {
+  uint32_t level = 0;
+  for (int i = t; i <= nrows; i += TB) {
     int64_t v = (int64_t)indptr[row0 + i];
     v = v < e0 ? e0 : (v > a.E ? a.E : v);
-    s_ptr[i] = (int)(v - e0 > 0x7fffffff ? 0x7fffffff : v - e0);
-  }
-  for (int i = t; i < nrows * a.chunks * NACC / 2; i += kBlock)
-    reinterpret_cast<uint2*>(s_acc)[i] = make_uint2(0u, 0u);
-  for (int i = t; i < a.f4_per_row * 4; i += kBlock) {
-    const int c4 = i >> 2, q = i & 3;
-    s_par[c4 * 8 + q] = a.params[i];
-    s_par[c4 * 8 + 4 + q] = a.params[a.param_stride + i];
-  }
-  __syncthreads();
-  if (s_ptr[nrows] > LIMIT) {  // only then can a single row exceed the field capacity
-    for (int r = t; r < nrows; r += kBlock)
-      if (s_ptr[r + 1] - s_ptr[r] > LIMIT) *s_flag = 1;
-    __syncthreads();
-    if (*s_flag) {
-      const bool is64 = sizeof(Idx) == 8;
-      acc_direct_block<BITS>(a, s_ptr, e0, row0, nrows,
-                             is64 ? reinterpret_cast<const int64_t*>(indices) : nullptr,
-                             is64 ? nullptr : reinterpret_cast<const int32_t*>(indices), out);
-      return;
+    const int p = (int)(v - e0 > 0x7fffffff ? 0x7fffffff : v - e0);
+    s_ptr[i] = p;
+    if (i < nrows) {
+      int64_t v2 = (int64_t)indptr[row0 + i + 1];
+      v2 = v2 < e0 ? e0 : (v2 > a.E ? a.E : v2);
+      const int deg = (int)(v2 - e0 > 0x7fffffff ? 0x7fffffff : v2 - e0) - p;
+      s_rdeg[i] = deg > 0 ? __builtin_amdgcn_rcpf((float)deg) : 0.f;
+      level |= (deg > CAP_N ? 1u : 0u) | (deg > CAP_W ? 2u : 0u);
     }
   }
-  const int ne = s_ptr[nrows];
-  const uint32_t tail_word = *s_tail;
-  const uint32_t* codes32 = reinterpret_cast<const uint32_t*>(a.codes);
+  {
+    const uint32_t wl = (__ballot(level & 1u) ? 1u : 0u) | (__ballot(level & 2u) ? 2u : 0u);
+    if ((t & (kWave - 1)) == 0) s_wflag[t / kWave] = wl;
+  }
+  __syncthreads();
+  uint32_t block_level = 0;
+#pragma unroll
+  for (int w = 0; w < TB / kWave; ++w) block_level |= s_wflag[w];
+  if (block_level & 2u) {
+    const bool is64 = sizeof(Idx) == 8;
+    acc_direct_block<TB, BITS>(a, s_ptr, e0, row0, nrows,
+                           is64 ? reinterpret_cast<const int64_t*>(indices) : nullptr,
+                           is64 ? nullptr : reinterpret_cast<const int32_t*>(indices), out);
+    return;
+  }
+  if (BITS == 4 && (block_level & 1u))
+    acc_block<TB, BITS, 4, Idx>(a, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
+  else
+    acc_block<TB, BITS, 2, Idx>(a, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
+}
 
-  for (int eb = 0; eb < ne; eb += a.edge_batch) {
-    const int nb = (ne - eb) < a.edge_batch ? (ne - eb) : a.edge_batch;
-    if (eb) __syncthreads();
-    for (int i = t; i < nb; i += kBlock) {
-      const uint64_t start = (uint64_t)clamp_idx(indices[e0 + eb + i], a.N) * (uint32_t)a.src_dim;
-      // local row of edge eb + i: the last r with s_ptr[r] <= eb + i (binary search, s_ptr is sorted)
-      const int pos = eb + i;
-      int lo = 0, hi = nrows;
-      while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (s_ptr[mid] <= pos) lo = mid; else hi = mid;
-      }
-      s_row[i] = (uint32_t)(start >> 2);
-      s_erow[i] = (uint16_t)(((start & 3) << 14) | (uint32_t)lo);
-    }
-    __syncthreads();
-    const int j = t & (a.dw2 - 1);
-    const int gslot = t / a.dw2;
-    const int gslots = kBlock / a.dw2;
-    constexpr int U = 4;
-    for (int e = gslot; e < nb; e += gslots * U) {
-      uint32_t w[U], er[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        int ee = e + u * gslots;
-        ee = ee < nb ? ee : nb - 1;
-        const uint32_t d = s_row[ee] + j;
-        er[u] = s_erow[ee];
-        const uint32_t v = codes32[d < a.last_full_dword ? d : a.last_full_dword];
-        w[u] = d > a.last_full_dword ? (d == a.last_full_dword + 1 ? tail_word : 0u) : v;
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int ee = e + u * gslots;
-        const uint32_t hi = __shfl_down(w[u], 1);
-        const uint32_t al = __builtin_amdgcn_alignbyte(hi, w[u], er[u] >> 14);
-        if (ee < nb && j < a.chunks) {
-          uint32_t* acc = s_acc + ((er[u] & 0x3fffu) * a.chunks + j) * NACC;
-          if (BITS == 4) {
-            atomicAdd(acc + 0, al & 0x000f000fu);
-            atomicAdd(acc + 1, (al >> 4) & 0x000f000fu);
-            atomicAdd(acc + 2, (al >> 8) & 0x000f000fu);
-            atomicAdd(acc + 3, (al >> 12) & 0x000f000fu);
-          } else {
-            atomicAdd(acc + 0, al & 0x00ff00ffu);
-            atomicAdd(acc + 1, (al >> 8) & 0x00ff00ffu);
-          }
-        }
-      }
-    }
-  }
-  __syncthreads();
-  // finalize: lane <-> one float4 of the block's contiguous output span
-  const int items = nrows * a.f4_per_row;
-  float* ob = out + row0 * (int64_t)a.feat_dim;
-  for (int it = t; it < items; it += kBlock) {
-    const int r = (int)__umulhi((uint32_t)it, a.magic);
-    const int c4 = it - r * a.f4_per_row;
-    float s0, s1, s2, s3;
-    if (BITS == 4) {
-      const uint4 q = *reinterpret_cast<const uint4*>(s_acc + (r * a.chunks + (c4 >> 1)) * 4);
-      const int sh = (c4 & 1) * 16;
-      s0 = (float)((q.x >> sh) & 0xffffu);
-      s1 = (float)((q.y >> sh) & 0xffffu);
-      s2 = (float)((q.z >> sh) & 0xffffu);
-      s3 = (float)((q.w >> sh) & 0xffffu);
-    } else {
-      const uint2 q = *reinterpret_cast<const uint2*>(s_acc + (r * a.chunks + c4) * 2);
-      s0 = (float)(q.x & 0xffffu);
-      s1 = (float)(q.y & 0xffffu);
-      s2 = (float)(q.x >> 16);
-      s3 = (float)(q.y >> 16);
-    }
-    const int deg = s_ptr[r + 1] - s_ptr[r];  // <= 0 for an empty (or malformed) row
-    const float rdeg = __builtin_amdgcn_rcpf((float)(deg > 1 ? deg : 1));  // rcp(1) == 1 exactly
-    const float4 mn = *reinterpret_cast<const float4*>(s_par + c4 * 8);
-    const float4 sc = *reinterpret_cast<const float4*>(s_par + c4 * 8 + 4);
-    float v0 = __fadd_rn(mn.x, __fmul_rn(s0 * rdeg, sc.x));
-    float v1 = __fadd_rn(mn.y, __fmul_rn(s1 * rdeg, sc.y));
-    float v2 = __fadd_rn(mn.z, __fmul_rn(s2 * rdeg, sc.z));
-    float v3 = __fadd_rn(mn.w, __fmul_rn(s3 * rdeg, sc.w));
-    if (deg <= 0) v0 = v1 = v2 = v3 = 0.f;
-    store_nt4(ob + (int64_t)it * 4, v0, v1, v2, v3);
-  }
+template <int TB, int BITS>
+int launch_acc_tb(AccArgs a, size_t lds, int64_t grid, const void* indptr, const void* indices, int idx_dtype,
+                  float* out, hipStream_t st, const char* what) {
+  a.fin_group = a.f4_per_row < TB ? a.f4_per_row : TB;
+  a.fin_slots = TB / a.fin_group;
+  a.fin_magic = (uint32_t)((65536 + a.fin_group - 1) / a.fin_group);
+  if (idx_dtype == F2CGT_DT_I32)
+    sq_affine_acc_kernel<TB, BITS, int32_t><<<(unsigned)grid, TB, lds, st>>>(
+        a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
+  else
+    sq_affine_acc_kernel<TB, BITS, int64_t><<<(unsigned)grid, TB, lds, st>>>(
+        a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
+  return launch_status(what);
 }
 
 template <int BITS>
 int launch_acc(AccArgs a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
                const char* what) {
-  constexpr int NOUT = 32 / BITS;
-  constexpr int NACC = BITS == 4 ? 4 : 2;
-  a.chunks = (int)ceil_div(a.feat_dim, NOUT);
+  a.eff_bytes = (int)ceil_div(a.feat_dim, 8 / BITS);
+  a.lanes = (int)ceil_div(a.eff_bytes, 8);
+  const int lanes2 = pow2_ceil(a.lanes);
+  a.lane_shift = 0;
+  while ((1 << a.lane_shift) < lanes2) ++a.lane_shift;
+  // rows of the accumulator array start lanes2 banks apart so that the lane groups of a wave,
+  // which mostly work on neighbouring rows, spread over all 32 banks
+  const int skew = lanes2 % 32;
+  a.pitch_n = ((4 * a.lanes + 31) / 32 * 32 + skew + 3) & ~3;
+  a.pitch_w = ((8 * a.lanes + 31) / 32 * 32 + skew + 3) & ~3;
   a.f4_per_row = a.feat_dim / 4;
-  a.magic = (uint32_t)((0x100000000ull + a.f4_per_row - 1) / a.f4_per_row);
-  const int maxshift = a.src_dim % 4 == 0 ? 0 : (a.src_dim % 2 == 0 ? 2 : 3);
-  a.dwords = (int)ceil_div(a.chunks * 4 + maxshift, 4);
-  a.dw2 = pow2_ceil(a.dwords);
-  a.last_full_dword = (uint32_t)((a.table_bytes - 4) >> 2);
-  a.edge_batch = 384;
   const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 1.0;
-  const int want = (int)(160.0 / (avg_deg > 0.5 ? avg_deg : 0.5));
-  int rb = 8;
-  while (rb * 2 <= want && rb < 64) rb *= 2;
-  const size_t acc_row = (size_t)a.chunks * NACC * 4;
-  while (rb > 8 && rb * acc_row > 20 * 1024) rb /= 2;
+  const double dg = avg_deg > 0.5 ? avg_deg : 0.5;
+  // the wide layout runs on half the rows at a time, so it must fit twice into the narrow one
+  const size_t acc_row = (size_t)(a.pitch_n * 2 > a.pitch_w ? a.pitch_n : (a.pitch_w + 1) / 2) * 4;
+  // 128-thread workgroups: more, smaller blocks in flight per CU overlap the dependent
+  // indptr -> indices -> code-row loads of one block with the output stores of others
+  constexpr int TB = 128;
+  a.edge_batch = 2 * TB;
+  int sub = ((int)(TB / dg) + 4) / 8 * 8;  // ~one edge per thread and sub-block, multiple of 8 rows
+  sub = sub < 8 ? 8 : (sub > 64 ? 64 : sub);
+  while (sub > 8 && sub * acc_row > 24 * 1024) sub -= 8;
+  int rb = sub * (int)(0.6 * a.edge_batch / (dg * sub));
+  rb = rb < sub ? sub : (rb > 256 ? 256 / sub * sub : rb);
   a.rows_per_block = rb;
-  const size_t lds = rb * acc_row + (size_t)a.f4_per_row * 32 + (size_t)(rb + 4) * 4 +
-                     (size_t)a.edge_batch * 6 + 16;
+  a.sub_rows = sub;
+  const size_t lds = sub * acc_row + (size_t)(rb + 4) * 4 + (size_t)rb * 4 + 16 + (size_t)a.edge_batch * 8 + 16;
   const int64_t grid = ceil_div(a.R, rb);
   if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
-  if (idx_dtype == F2CGT_DT_I32)
-    sq_affine_acc_kernel<BITS, int32_t><<<(unsigned)grid, kBlock, lds, st>>>(
-        a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
-  else
-    sq_affine_acc_kernel<BITS, int64_t><<<(unsigned)grid, kBlock, lds, st>>>(
-        a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
-  return launch_status(what);
+  return launch_acc_tb<TB, BITS>(a, lds, grid, indptr, indices, idx_dtype, out, st, what);
 }
 
 
@@ -739,16 +847,14 @@ int sq_block_run(bool affine, const uint8_t* codes, const float* table, int64_t 
 bool sq_affine_acc_eligible(const void* codes, const float* out, int64_t N, int64_t src_dim, int feat_dim,
                             int target_bits) {
   if (target_bits != 4 && target_bits != 8) return false;
-  if (!aligned(codes, 4) || !aligned(out, 16)) return false;
-  if (feat_dim < 4 || feat_dim % 4 != 0 || feat_dim > 4096) return false;
-  if (src_dim < 1 || src_dim >= (1ll << 20) || src_dim * (8 / target_bits) < feat_dim) return false;
-  const int64_t table_bytes = N * src_dim;
-  if (N >= (1ll << 32) || table_bytes < 8 || (table_bytes >> 2) >= (1ll << 32) - 4096) return false;
-  const int chunks = (int)ceil_div(feat_dim, 32 / target_bits);
-  if (pow2_ceil(chunks + 1) > kBlock) return false;
-  // the register realignment of byte-shifted rows exchanges dwords inside one wave
-  if (src_dim % 4 != 0 && pow2_ceil(chunks + 1) > kWave) return false;
-  if ((size_t)chunks * (target_bits == 4 ? 16 : 8) * 8 > 20 * 1024) return false;
+  if (codes == nullptr || !aligned(out, 16)) return false;
+  if (feat_dim % 4 != 0 || feat_dim > 4096) return false;
+  if (feat_dim * target_bits < 64) return false;  // a gather lane loads 8 bytes of the row
+  if (src_dim < 8 || src_dim >= (1ll << 20) || src_dim * (8 / target_bits) < feat_dim) return false;
+  if (N < 1 || N >= (1ll << 32)) return false;
+  const int lanes = (int)ceil_div(ceil_div(feat_dim, 8 / target_bits), 8);
+  if (pow2_ceil(lanes) > 128) return false;
+  if ((size_t)(8 * lanes + 64) * 4 * 4 > 24 * 1024) return false;  // 8 rows of the wide layout
   return true;
 }
 
@@ -760,7 +866,6 @@ int sq_affine_acc_run(const uint8_t* codes, const float* params, int64_t param_s
   a.params = params;
   a.param_stride = param_stride;
   a.R = R; a.E = E; a.N = N;
-  a.table_bytes = N * src_dim;
   a.src_dim = (int)src_dim;
   a.feat_dim = feat_dim;
   return target_bits == 4 ? launch_acc<4>(a, indptr, indices, idx_dtype, out, st, what)
