@@ -1,11 +1,12 @@
 // Persistent, software-pipelined kernel for the fused VQ decode + mean aggregation.
 //
 // One 1024-thread workgroup per CU keeps a 128-column tile of the codebook in LDS, laid out
-// [code][piece][8 floats] (a "piece" is 8 consecutive output columns), so the 32 B a lane reads
-// per edge land on bank groups fixed by its piece: measured ~110 B/clk/CU against 62 B/clk for
-// the natural [subspace][code][w] layout.  A lane owns one (destination row, piece) of a
-// 64-row block and walks the row's edges in order with register accumulators; the codebook
-// reads of the next group of edges are issued before the adds of the current group.
+// [code][128 columns], so the 16 B a lane reads per edge sit at bank offset 4 * (lane % 32):
+// the 32 lanes of a row read 512 contiguous bytes of one code's row only when codes agree, and
+// otherwise spread over all banks.  A lane owns one float4 of a destination row (32 lanes per
+// row) and two rows of a 64-row block, walks the row's edges in order with register
+// accumulators, and issues the codebook reads of the next group of edges before the adds of
+// the current group.
 //
 // Everything that comes from HBM is prefetched through registers two iterations ahead, one
 // element per lane and stage, and parked in LDS one barrier before it is needed:
@@ -25,6 +26,7 @@ constexpr int kRows = 64;        // destination rows per block (kThreads / 16 pi
 constexpr int kEdgeCap = 1024;   // staged edges per block: one per lane
 constexpr int kRing = 8;
 constexpr int kGroup = 5;        // edges per register group of the inner loop
+constexpr int kXcds = 8;         // accelerator dies (one L2 each) of the MI355X
 
 struct VqArgs {
   const uint8_t* codes;
@@ -32,6 +34,7 @@ struct VqArgs {
   int64_t R, E, N;
   int n_cb, K, w, feat_dim;
   int n_tiles, n_stripes;
+  int stripes_per_xcd;  // > 0: the column tiles of a stripe share one XCD (see the kernel)
 };
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -227,8 +230,18 @@ __global__ __launch_bounds__(kThreads) void vq_pipe_kernel(VqArgs a, const Idx* 
   pipe.s_e0 = reinterpret_cast<int64_t*>(pipe.s_codes + kEdgeCap * BT);
   pipe.s_ptr = reinterpret_cast<int*>(pipe.s_e0 + kRing);
   pipe.t = threadIdx.x;
-  pipe.tile = blockIdx.x % a.n_tiles;
-  pipe.stripe = blockIdx.x / a.n_tiles;
+  if (a.stripes_per_xcd > 0) {
+    // Workgroup ids are dealt round-robin to the XCDs.  The column tiles of a stripe read the same
+    // indptr, indices and code rows, so they are placed on one XCD and share its L2: the rows come
+    // from HBM once per stripe instead of once per tile.
+    const int xcd = blockIdx.x % kXcds, k = blockIdx.x / kXcds;
+    if (k >= a.stripes_per_xcd * a.n_tiles) return;
+    pipe.tile = k % a.n_tiles;
+    pipe.stripe = xcd * a.stripes_per_xcd + k / a.n_tiles;
+  } else {
+    pipe.tile = blockIdx.x % a.n_tiles;
+    pipe.stripe = blockIdx.x / a.n_tiles;
+  }
   const int64_t nblocks = ceil_div(a.R, kRows);
   pipe.my_blocks = pipe.stripe < nblocks ? (nblocks - pipe.stripe + a.n_stripes - 1) / a.n_stripes : 0;
   pipe.Pa = pipe.Pb = pipe.P0a = pipe.P0b = 0;
@@ -265,7 +278,14 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
   if (a.n_stripes < 1) a.n_stripes = 1;
   const int64_t nblocks = ceil_div(a.R, kRows);
   if (a.n_stripes > nblocks) a.n_stripes = (int)(nblocks > 0 ? nblocks : 1);
-  const unsigned grid = (unsigned)(a.n_stripes * a.n_tiles);
+  unsigned grid = (unsigned)(a.n_stripes * a.n_tiles);
+  a.stripes_per_xcd = 0;
+  if (a.n_tiles > 1 && cus % kXcds == 0 && (cus / kXcds) / a.n_tiles >= 1 &&
+      (int64_t)kXcds * ((cus / kXcds) / a.n_tiles) <= nblocks) {
+    a.stripes_per_xcd = (cus / kXcds) / a.n_tiles;
+    a.n_stripes = kXcds * a.stripes_per_xcd;
+    grid = (unsigned)cus;
+  }
   hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_pipe_kernel<BT, int32_t>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_pipe_kernel<BT, int64_t>),
