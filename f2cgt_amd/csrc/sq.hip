@@ -149,10 +149,130 @@ __global__ __launch_bounds__(kBlock) void sq_affine_decompress_kernel(
   }
 }
 
+// ---- float4-per-lane streaming decoders ------------------------------------------------
+// Both decoders above walk the packed side (one lane per byte, scalar stores).  When rows are
+// whole float4 groups the output side can drive instead: one lane per output float4, eight
+// float4 per lane, a workgroup writes one dense 32 KB span with non-temporal stores, and the
+// (row, column group) of an item comes from a 32-bit multiply-high instead of a 64-bit divide.
+// The lane loads exactly the code bits of its four columns (1-4 bytes, byte granular).
+constexpr int kF4Items = 8;
+
+struct F4Args {
+  const uint8_t* codes;
+  float* out;
+  const float* table;     // affine: params [2, param_stride]; log domain: codebooks [n_cb, 5]
+  int64_t param_stride;
+  int64_t column_slice;
+  int n_cb;
+  int64_t src_dim;
+  int64_t total_f4;
+  uint32_t f4_per_row;
+  uint32_t magic;         // ceil(2^32 / f4_per_row)
+};
+
+template <int BITS, bool AFFINE>
+__global__ __launch_bounds__(kBlock) void sq_decode_f4_kernel(F4Args a) {
+  constexpr int NCODE = 1 << BITS;
+  constexpr uint32_t MASK = NCODE - 1;
+  extern __shared__ __align__(16) float s_tab[];
+  // affine: [f4][mn x4, scale x4]; log domain: LUT [n_cb][NCODE], then the codebook of each column
+  const int feat_dim = (int)a.f4_per_row * 4;
+  int* s_cbi = reinterpret_cast<int*>(s_tab + ((a.n_cb * NCODE + 3) & ~3));
+  if (AFFINE) {
+    for (int i = threadIdx.x; i < feat_dim; i += kBlock) {
+      s_tab[(i >> 2) * 8 + (i & 3)] = a.table[i];
+      s_tab[(i >> 2) * 8 + 4 + (i & 3)] = a.table[a.param_stride + i];
+    }
+  } else {
+    for (int i = threadIdx.x; i < a.n_cb * NCODE; i += kBlock)
+      s_tab[i] = sq_log_value<BITS>((uint32_t)(i & MASK), a.table + (int64_t)(i >> BITS) * 5);
+    for (int i = threadIdx.x; i < feat_dim; i += kBlock) {
+      int64_t cb = i / a.column_slice;
+      cb = cb < a.n_cb ? cb : a.n_cb - 1;
+      s_cbi[i] = (int)cb * NCODE;
+    }
+  }
+  __syncthreads();
+
+  const int64_t base = (int64_t)blockIdx.x * (kF4Items * kBlock);
+  // first row of the span: floor(base / f4_per_row), from the fp64 quotient and a fix-up
+  int64_t rb = (int64_t)((double)base / (double)a.f4_per_row);
+  if (rb * a.f4_per_row > base) --rb;
+  if ((rb + 1) * (int64_t)a.f4_per_row <= base) ++rb;
+  const uint32_t cb0 = (uint32_t)(base - rb * a.f4_per_row);
+
+  uint32_t word[kF4Items], c4s[kF4Items];
+#pragma unroll
+  for (int k = 0; k < kF4Items; ++k) {
+    const uint32_t li = cb0 + threadIdx.x + k * kBlock;
+    const uint32_t rl = __umulhi(li, a.magic);
+    const uint32_t c4 = li - rl * a.f4_per_row;
+    const bool on = base + threadIdx.x + k * kBlock < a.total_f4;
+    const uint8_t* src = a.codes + (on ? (rb + rl) * a.src_dim : 0);
+    c4s[k] = c4;
+    if (BITS == 8) {
+      uint32_t w; __builtin_memcpy(&w, src + (on ? 4 * c4 : 0), 4); word[k] = w;
+    } else if (BITS == 4) {
+      uint16_t w; __builtin_memcpy(&w, src + (on ? 2 * c4 : 0), 2); word[k] = w;
+    } else if (BITS == 2) {
+      word[k] = src[on ? c4 : 0];
+    } else {
+      word[k] = (src[on ? (c4 >> 1) : 0] >> ((c4 & 1) * 4)) & 0xfu;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kF4Items; ++k) {
+    const int64_t i = base + threadIdx.x + k * kBlock;
+    if (i >= a.total_f4) break;
+    const uint32_t c4 = c4s[k];
+    float v[4];
+    if (AFFINE) {
+      const float4 mn = *reinterpret_cast<const float4*>(s_tab + c4 * 8);
+      const float4 sc = *reinterpret_cast<const float4*>(s_tab + c4 * 8 + 4);
+      v[0] = __fadd_rn(mn.x, __fmul_rn((float)(word[k] & MASK), sc.x));
+      v[1] = __fadd_rn(mn.y, __fmul_rn((float)((word[k] >> BITS) & MASK), sc.y));
+      v[2] = __fadd_rn(mn.z, __fmul_rn((float)((word[k] >> (2 * BITS)) & MASK), sc.z));
+      v[3] = __fadd_rn(mn.w, __fmul_rn((float)((word[k] >> (3 * BITS)) & MASK), sc.w));
+    } else {
+      const int4 cbi = *reinterpret_cast<const int4*>(s_cbi + c4 * 4);
+      v[0] = s_tab[cbi.x + (word[k] & MASK)];
+      v[1] = s_tab[cbi.y + ((word[k] >> BITS) & MASK)];
+      v[2] = s_tab[cbi.z + ((word[k] >> (2 * BITS)) & MASK)];
+      v[3] = s_tab[cbi.w + ((word[k] >> (3 * BITS)) & MASK)];
+    }
+    store_nt4(a.out + i * 4, v[0], v[1], v[2], v[3]);
+  }
+}
+
+// Launches the float4 decoder when the shape allows it; returns -1 when it does not.
+template <int BITS, bool AFFINE>
+int decode_f4_launch(const uint8_t* codes, float* out, const float* table, int64_t param_stride,
+                     int64_t column_slice, int n_cb, int64_t rows, int64_t src_dim, int64_t feat_dim,
+                     hipStream_t st, const char* what) {
+  if (feat_dim % 4 != 0 || feat_dim > 8192 || !aligned(out, 16)) return -1;
+  const size_t lds = AFFINE ? (size_t)feat_dim * 8
+                            : ((((size_t)n_cb << BITS) + 3) / 4 * 4 + (size_t)feat_dim) * 4;
+  if (lds > (size_t)kMaxLutBytes) return -1;
+  F4Args a{};
+  a.codes = codes; a.out = out; a.table = table;
+  a.param_stride = param_stride; a.column_slice = column_slice; a.n_cb = AFFINE ? 0 : n_cb;
+  a.src_dim = src_dim;
+  a.f4_per_row = (uint32_t)(feat_dim / 4);
+  a.total_f4 = rows * (feat_dim / 4);
+  a.magic = (uint32_t)((0x100000000ull + a.f4_per_row - 1) / a.f4_per_row);
+  const int64_t grid = ceil_div(a.total_f4, kF4Items * kBlock);
+  if (grid > 0x7fffffffll) return -1;
+  sq_decode_f4_kernel<BITS, AFFINE><<<(unsigned)grid, kBlock, lds, st>>>(a);
+  return launch_status(what);
+}
+
 template <int BITS>
 int decompress_lut_launch(const uint8_t* codes, float* out, const float* codebooks, int64_t rows,
                           int64_t src_dim, int64_t feat_dim, int64_t column_slice, int n_cb,
                           hipStream_t st) {
+  const int rc = decode_f4_launch<BITS, false>(codes, out, codebooks, 0, column_slice, n_cb, rows, src_dim,
+                                               feat_dim, st, "sq_decompress");
+  if (rc >= 0) return rc;
   const int64_t items = rows * ceil_div(feat_dim, 8 / BITS);
   const size_t lds = (size_t)n_cb * (1 << BITS) * sizeof(float);
   sq_decompress_lut_kernel<BITS><<<grid_for(items, 8), kBlock, lds, st>>>(
@@ -274,6 +394,16 @@ extern "C" int f2cgt_sq_affine_decompress(const uint8_t* codes, float* out, cons
   if (rows * feat_dim == 0) return 0;
   F2CGT_REQUIRE(codes && out && params, F2CGT_E_INVALID, "sq_affine_decompress: null buffer");
   hipStream_t st = as_stream(stream);
+  {
+    int rc = -1;
+    switch (target_bits) {
+      case 1: rc = decode_f4_launch<1, true>(codes, out, params, param_stride, 1, 0, rows, src_dim, feat_dim, st, "sq_affine_decompress"); break;
+      case 2: rc = decode_f4_launch<2, true>(codes, out, params, param_stride, 1, 0, rows, src_dim, feat_dim, st, "sq_affine_decompress"); break;
+      case 4: rc = decode_f4_launch<4, true>(codes, out, params, param_stride, 1, 0, rows, src_dim, feat_dim, st, "sq_affine_decompress"); break;
+      default: rc = decode_f4_launch<8, true>(codes, out, params, param_stride, 1, 0, rows, src_dim, feat_dim, st, "sq_affine_decompress"); break;
+    }
+    if (rc >= 0) return rc;
+  }
   const int grid = grid_for(rows * ceil_div(feat_dim, 8 / target_bits), 16);
 #define F2CGT_CASE(B)                                                                          \
   case B:                                                                                      \

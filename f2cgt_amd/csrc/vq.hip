@@ -48,6 +48,104 @@ __global__ __launch_bounds__(kBlock) void vq_decompress_kernel(
   }
 }
 
+// ---- uint8 codes, fp32 codebooks, K <= 256, width dividing 128 ---------------------------
+// One persistent 1024-thread workgroup per CU keeps a 128-column tile of the codebooks in LDS as
+// [code][128 columns]: lane (t % 32) reads the 16 bytes at code * 512 + 16 * (t % 32), so the
+// eight lanes that the LDS serves per clock always cover all 32 banks.  A lane owns one float4
+// column group and takes eight rows (32 apart) per step: eight code-byte loads in flight, eight
+// LDS reads, eight non-temporal float4 stores; the code bytes of the next step are loaded
+// before the stores of the current one are issued.  Full steps run without predicates so the
+// prefetch never has to wait for the stores behind it.
+constexpr int kTileThreads = 1024;
+constexpr int kTileRows = 256;   // rows per step: 32 lane groups x 8
+
+struct VqTileArgs {
+  const uint8_t* codes;
+  const float* codebooks;
+  float* out;
+  int64_t rows;
+  int feat_dim, n_cb, K, w;
+  int n_tiles, n_stripes;
+};
+
+__global__ __launch_bounds__(kTileThreads) void vq_decompress_tile_kernel(VqTileArgs a) {
+  extern __shared__ __align__(16) float s_cb[];
+  const int tile = blockIdx.x % a.n_tiles;
+  const int stripe = blockIdx.x / a.n_tiles;
+  const int tile_cols = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
+  for (int i = threadIdx.x; i < a.K * 128; i += kTileThreads) {
+    const int code = i >> 7, c = i & 127;
+    float v = 0.f;
+    if (c < tile_cols) {
+      const int col = tile * 128 + c;
+      const int sub = col / a.w;
+      v = a.codebooks[((int64_t)sub * a.K + code) * a.w + (col - sub * a.w)];
+    }
+    s_cb[i] = v;
+  }
+  __syncthreads();
+  const int c4 = threadIdx.x & 31;
+  const int rs = threadIdx.x >> 5;
+  if (c4 * 4 >= tile_cols) return;
+  const int col0 = tile * 128 + c4 * 4;
+  const uint8_t* cp = a.codes + col0 / a.w;
+  const float* cbp = s_cb + c4 * 4;
+  float* op = a.out + col0;
+  const int64_t steps = a.rows / kTileRows;   // full steps
+  const uint32_t kmax = (uint32_t)a.K - 1u;
+
+  uint32_t code[8];
+  int64_t s = stripe;
+  if (s < steps) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) code[u] = cp[(s * kTileRows + rs + 32 * u) * a.n_cb];
+  }
+  for (; s < steps; s += a.n_stripes) {
+    const int64_t sn = s + a.n_stripes < steps ? s + a.n_stripes : s;  // last step reloads itself
+    uint32_t next[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) next[u] = cp[(sn * kTileRows + rs + 32 * u) * a.n_cb];
+    float4 x[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const uint32_t c = code[u] < kmax ? code[u] : kmax;
+      x[u] = *reinterpret_cast<const float4*>(cbp + c * 128);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      store_nt4(op + (s * kTileRows + rs + 32 * u) * (int64_t)a.feat_dim, x[u].x, x[u].y, x[u].z, x[u].w);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) code[u] = next[u];
+  }
+  // the rows after the last full step, one stripe
+  if (stripe == (int)(steps % a.n_stripes)) {
+    for (int64_t r = steps * kTileRows + rs; r < a.rows; r += 32) {
+      uint32_t c = cp[r * a.n_cb];
+      c = c < kmax ? c : kmax;
+      const float4 x = *reinterpret_cast<const float4*>(cbp + c * 128);
+      store_nt4(op + r * (int64_t)a.feat_dim, x.x, x.y, x.z, x.w);
+    }
+  }
+}
+
+// Returns -1 when the shape is not covered.
+int launch_tile(const uint8_t* codes, const float* codebooks, float* out, int64_t rows, int64_t feat_dim,
+                int n_cb, int K, int w, hipStream_t st) {
+  if (K > 256 || w < 4 || 128 % w != 0 || feat_dim % 4 != 0 || feat_dim < 64) return -1;
+  if (!aligned(out, 16) || rows < 4 * kTileRows) return -1;
+  VqTileArgs a{codes, codebooks, out, rows, (int)feat_dim, n_cb, K, w, 0, 0};
+  a.n_tiles = (int)ceil_div(feat_dim, 128);
+  const int cus = num_cus();
+  if (a.n_tiles > cus) return -1;
+  a.n_stripes = cus / a.n_tiles;
+  const size_t lds = (size_t)K * 128 * 4;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_decompress_tile_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return fail((int)e, "vq_decompress: cannot reserve %zu B of LDS", lds);
+  vq_decompress_tile_kernel<<<(unsigned)(a.n_stripes * a.n_tiles), kTileThreads, lds, st>>>(a);
+  return launch_status("vq_decompress");
+}
+
 template <typename CT, typename CBT>
 int launch(const void* codes, const void* codebooks, float* out, int64_t rows, int64_t feat_dim,
            int n_cb, int K, int w, hipStream_t st) {
@@ -104,6 +202,11 @@ extern "C" int f2cgt_vq_decompress(const void* codes, int code_dtype, const void
   hipStream_t st = as_stream(stream);
   const int n_cb = (int)num_codebooks, k = (int)K, w = (int)width;
   const bool f32 = cb_dtype == F2CGT_DT_F32;
+  if (code_dtype == F2CGT_DT_U8 && f32) {
+    const int rc = launch_tile(static_cast<const uint8_t*>(codes), static_cast<const float*>(codebooks), out, rows,
+                               feat_dim, n_cb, k, w, st);
+    if (rc >= 0) return rc;
+  }
   switch (code_dtype) {
     case F2CGT_DT_U8:
       return f32 ? launch<uint8_t, float>(codes, codebooks, out, rows, feat_dim, n_cb, k, w, st)

@@ -199,6 +199,35 @@ def test_vq_decompress_codebook_larger_than_lds():
     assert np.array_equal(got, oc.vq_decompress(idx, cb, 768))
 
 
+@pytest.mark.parametrize("shape", [(16, 256, 8, 128, 5077), (8, 64, 16, 100, 3001), (25, 256, 4, 100, 1024),
+                                   (24, 200, 32, 768, 2049), (2, 256, 64, 128, 4096), (16, 256, 8, 64, 1500)])
+def test_vq_decompress_tile_path(shape):
+    # uint8 codes + fp32 codebooks of a width dividing 128: the persistent LDS-tile kernel, with
+    # row counts that leave a remainder after the last full 256-row step
+    n_cb, K, w, feat_dim, rows = shape
+    rng = np.random.default_rng(rows)
+    cb = rng.standard_normal((n_cb, K, w)).astype(np.float32)
+    idx = rng.integers(0, K, size=(rows, n_cb), dtype=np.uint8)
+    idx[::97, 0] = 255   # codes >= K read entry K - 1, as in the generic kernel
+    got = host(capi.vq_decompress(dev(idx), dev(cb), feat_dim))
+    want = oc.vq_decompress(np.minimum(idx, K - 1), cb, feat_dim)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+def test_sq_affine_decompress_padded_storage(bits):
+    # storage rows wider than the decoded columns need (odd byte pitch: rows are not word aligned)
+    rng = np.random.default_rng(bits)
+    d = 72
+    x = rng.standard_normal((3000, d)).astype(np.float32)
+    params = oc.sq_affine_params(x, bits)
+    codes = oc.sq_affine_compress(x, params, bits)
+    store = oc.packbits(codes, bits) if bits < 8 else codes
+    wide = np.concatenate([store, rng.integers(0, 256, size=(3000, 5), dtype=np.uint8)], axis=1)
+    got = host(capi.sq_affine_decompress(dev(wide), dev(params), bits, d))
+    assert np.array_equal(got, oc.sq_affine_decompress(store, params, bits, d))
+
+
 # ---- plain CSC mean ---------------------------------------------------------------------------
 @pytest.mark.parametrize("idx", [np.int32, np.int64])
 @pytest.mark.parametrize("d", [1, 7, 100, 128, 300])
