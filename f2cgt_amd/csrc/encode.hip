@@ -5,12 +5,15 @@
 // numbers carry no cancellation error.
 //
 // kmeans_predict never writes the matrix.  A wave owns 32 rows of x and walks the
-// centres 32 at a time with fp32 MFMA (v_mfma_f32_32x32x2_f32): A = centre tile,
-// B = x tile, so every lane holds 16 centre scores of ONE x row and the running
+// centres 64 at a time with fp32 MFMA (v_mfma_f32_32x32x2_f32): A = centre tile,
+// B = x tile, so every lane holds 16 centre scores of ONE x row per tile and the running
 // arg-min stays in registers.  Scores use the expanded form (|c|^2 - 2 x.c, the row
 // constant |x|^2 dropped); rows whose two best scores are closer than the rounding
 // bound of that form are re-evaluated exactly in fp64 by the whole wave, so the label
-// is the true first minimum.
+// is the true first minimum.  On this chip vector instructions do not run in the shadow of
+// matrix instructions of the same SIMD (measured: a 128-instruction update per 34 MFMAs costs
+// its full issue time with one to three waves per SIMD), so the update is kept to four
+// instructions per score and everything else is folded into the MFMA operands.
 #include "common.hpp"
 
 #include <cfloat>
@@ -59,6 +62,30 @@ __device__ int exact_argmin_row(const float* __restrict__ xrow, const float* __r
   return besti;
 }
 
+// Same for the L2 metric with the centres already staged in LDS, transposed as
+// cT[(half * KH + t) * n_pad + centre] (dimension = half * khalf + t): lanes read consecutive words.
+__device__ int exact_argmin_row_l2_lds(const float* __restrict__ xrow, const float* cT, int n, int n_pad, int KH,
+                                       int khalf, int k, int lane) {
+  double bestv = DBL_MAX;
+  int besti = INT_MAX;
+  for (int c = lane; c < n; c += kWave) {
+    double d = 0.0;
+    for (int dim = 0; dim < k; ++dim) {
+      const int hh = dim >= khalf ? 1 : 0;
+      const double df = (double)xrow[dim] - (double)cT[(hh * KH + dim - hh * khalf) * n_pad + c];
+      d += df * df;
+    }
+    if (d < bestv) { bestv = d; besti = c; }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const double ov = __shfl_xor(bestv, off);
+    const int oi = __shfl_xor(besti, off);
+    if (ov < bestv || (ov == bestv && oi < besti)) { bestv = ov; besti = oi; }
+  }
+  return besti;
+}
+
 // ---- general fallback: one wave per row, exact -------------------------------------------
 __global__ __launch_bounds__(256) void predict_exact_kernel(const float* __restrict__ x,
                                                             const float* __restrict__ centers,
@@ -80,6 +107,25 @@ __global__ __launch_bounds__(256) void predict_exact_kernel(const float* __restr
 // ---- MFMA path ----------------------------------------------------------------------------
 // KH = per-half register depth: the k dimensions are split in two halves of
 // khalf = ceil(k/2); lanes 0-31 feed half 0, lanes 32-63 half 1 (zero padded to KH).
+// The whole score comes out of the matrix core: x is pre-scaled (-2 x for L2, -x for cosine;
+// cosine centres are staged divided by their norm) and one extra k step multiplies the centre's
+// bias (|c|^2, or +inf for the padding centres) by 1, so the epilogue is only the running
+// (best, second, arg) update: compare, select, v_med3, v_min per score.  Two centre tiles are
+// accumulated at a time, so one tile's MFMA chain runs under the other's epilogue.
+__device__ __forceinline__ void argmin_update(const floatx16& acc, int ct, float& best, float& second, int& bv,
+                                              int& bct) {
+  const float before = best;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const float s = acc[v];
+    const bool lt = s < best;
+    second = __builtin_amdgcn_fmed3f(best, second, s);
+    bv = lt ? v : bv;
+    best = lt ? s : best;
+  }
+  bct = best < before ? ct : bct;
+}
+
 template <int KH>
 __global__ __launch_bounds__(256) void predict_mfma_kernel(const float* __restrict__ x,
                                                            const float* __restrict__ centers,
@@ -88,36 +134,38 @@ __global__ __launch_bounds__(256) void predict_mfma_kernel(const float* __restri
                                                            int n, int k, int metric, int n_pad) {
   extern __shared__ float smem[];
   float* cT = smem;                   // [2*KH][n_pad]  centre coordinates, transposed
-  float* bias = cT + 2 * KH * n_pad;  // [n_pad]  score = bias + mul * dot
-  float* mul = bias + n_pad;          // [n_pad]
-  int* cmax_bits = reinterpret_cast<int*>(mul + n_pad);  // max |c|^2 as ordered int bits
+  float* cB = cT + 2 * KH * n_pad;    // [2][n_pad]  bias row (half 0) and a zero row (half 1)
+  int* cmax_bits = reinterpret_cast<int*>(cB + 2 * n_pad);  // max |c|^2 as ordered int bits
 
   const int khalf = (k + 1) / 2;
+  const bool cosine = metric == F2CGT_METRIC_COSINE;
   if (threadIdx.x == 0) *cmax_bits = 0;
   __syncthreads();
-  for (int j = threadIdx.x; j < n_pad; j += blockDim.x) {
+  // stage the centres transposed: coalesced reads of the [n, k] array, scattered LDS writes
+  for (int i = threadIdx.x; i < 2 * KH * n_pad; i += blockDim.x) cT[i] = 0.f;
+  __syncthreads();
+#pragma unroll 8
+  for (int i = threadIdx.x; i < n * k; i += blockDim.x) {
+    const int jj = i / k, dim = i - jj * k;
+    const int hh = dim >= khalf ? 1 : 0;
+    cT[(hh * KH + dim - hh * khalf) * n_pad + jj] = centers[i];
+  }
+  __syncthreads();
+  for (int jj = threadIdx.x; jj < n_pad; jj += blockDim.x) {
     float cn = 0.f;
 #pragma unroll 4
     for (int kk = 0; kk < 2 * KH; ++kk) {
-      const int h = kk / KH, t = kk - h * KH;
-      const int dim = h * khalf + t;
-      const bool ok = j < n && t < khalf && dim < k;
-      const float v = ok ? centers[(int64_t)j * k + dim] : 0.f;
-      cT[kk * n_pad + j] = v;
+      const float v = cT[kk * n_pad + jj];
       cn += v * v;
     }
-    if (j >= n) {
-      bias[j] = INFINITY;
-      mul[j] = 0.f;
-    } else if (metric == F2CGT_METRIC_COSINE) {
+    if (cosine) {
       const float nr = sqrtf(cn);
-      bias[j] = 0.f;
-      mul[j] = -1.f / (nr > 1e-30f ? nr : 1e-30f);
-    } else {
-      bias[j] = cn;
-      mul[j] = -2.f;
-      atomicMax(cmax_bits, __float_as_int(cn));
+      const float scale = 1.f / (nr > 1e-30f ? nr : 1e-30f);
+      for (int kk = 0; kk < 2 * KH; ++kk) cT[kk * n_pad + jj] *= scale;
     }
+    cB[jj] = jj >= n ? INFINITY : (cosine ? 0.f : cn);
+    cB[n_pad + jj] = 0.f;
+    if (jj < n && !cosine) atomicMax(cmax_bits, __float_as_int(cn));
   }
   __syncthreads();
   const float cmax = __int_as_float(*cmax_bits);
@@ -128,55 +176,67 @@ __global__ __launch_bounds__(256) void predict_mfma_kernel(const float* __restri
   const int64_t n_tiles = (m + 31) / 32;
   const float unit = 5.9604645e-8f * (float)(4 * k + 16);
   const bool vec4 = (k % 8 == 0) && (KH % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+  const float xscale = cosine ? -1.f : -2.f;
+  const float xb = h == 0 ? 1.f : 0.f;
+  const float* ap = cT + (h * KH) * n_pad + j;
+  const float* bp = cB + h * n_pad + j;
 
-  for (int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); tile < n_tiles;
-       tile += (int64_t)gridDim.x * 4) {
+  // raw coordinates of this lane's x row (its half of the k dimensions) for one tile
+  auto load_x = [&](int64_t tile, float (&q)[KH]) {
     const int64_t row = tile * 32 + j;
     const bool valid = row < m;
-    float xr[KH];
-    float xn = 0.f;
     const float* xp = x + row * k + h * khalf;
     if (vec4) {
 #pragma unroll
       for (int t = 0; t < KH; t += 4) {
-        float4 q = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (valid && t < khalf) q = *reinterpret_cast<const float4*>(xp + t);
-        xr[t] = q.x; xr[t + 1] = q.y; xr[t + 2] = q.z; xr[t + 3] = q.w;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (valid && t < khalf) v = *reinterpret_cast<const float4*>(xp + t);
+        q[t] = v.x; q[t + 1] = v.y; q[t + 2] = v.z; q[t + 3] = v.w;
       }
     } else {
 #pragma unroll
       for (int t = 0; t < KH; ++t) {
         const int dim = h * khalf + t;
-        xr[t] = (valid && t < khalf && dim < k) ? xp[t] : 0.f;
+        q[t] = (valid && t < khalf && dim < k) ? xp[t] : 0.f;
       }
     }
+  };
+  const int64_t tile0 = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t tstride = (int64_t)gridDim.x * 4;
+  float xq[KH];
+  if (tile0 < n_tiles) load_x(tile0, xq);
+  for (int64_t tile = tile0; tile < n_tiles; tile += tstride) {
+    const int64_t row = tile * 32 + j;
+    const bool valid = row < m;
+    float xr[KH];
+    float xn = 0.f;
 #pragma unroll
-    for (int t = 0; t < KH; ++t) xn += xr[t] * xr[t];
+    for (int t = 0; t < KH; ++t) {
+      xn += xq[t] * xq[t];
+      xr[t] = xq[t] * xscale;
+    }
     xn += __shfl_xor(xn, 32);
+    // the next tile's rows travel from HBM while this tile is scored
+    load_x(tile + tstride < n_tiles ? tile + tstride : tile, xq);
+    asm volatile("" ::: "memory");
 
     float best = INFINITY, second = INFINITY;
-    int besti = 0;
-    for (int ct = 0; ct < n_pad; ct += 32) {
-      floatx16 acc;
+    int bv = 0, bct = 0;
+    for (int ct = 0; ct < n_pad; ct += 64) {
+      floatx16 zero;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-      const float* ap = cT + (h * KH) * n_pad + ct + j;
+      for (int v = 0; v < 16; ++v) zero[v] = 0.f;
+      floatx16 acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(bp[ct], xb, zero, 0, 0, 0);
+      floatx16 acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(bp[ct + 32], xb, zero, 0, 0, 0);
 #pragma unroll
-      for (int t = 0; t < KH; ++t)
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[t * n_pad], xr[t], acc, 0, 0, 0);
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int ci = ct + 8 * (v / 4) + 4 * h + (v % 4);
-        const float s = bias[ci] + mul[ci] * acc[v];
-        if (s < best) {
-          second = best;
-          best = s;
-          besti = ci;
-        } else if (s < second) {
-          second = s;
-        }
+      for (int t = 0; t < KH; ++t) {
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[t * n_pad + ct], xr[t], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[t * n_pad + ct + 32], xr[t], acc1, 0, 0, 0);
       }
+      argmin_update(acc0, ct, best, second, bv, bct);
+      argmin_update(acc1, ct + 32, best, second, bv, bct);
     }
+    int besti = bct + 8 * (bv >> 2) + 4 * h + (bv & 3);
     {  // merge the two halves of the wave (same x row, disjoint centres)
       const float ob = __shfl_xor(best, 32);
       const float os = __shfl_xor(second, 32);
@@ -189,14 +249,15 @@ __global__ __launch_bounds__(256) void predict_mfma_kernel(const float* __restri
         second = fminf(second, ob);
       }
     }
-    const float scale = metric == F2CGT_METRIC_COSINE ? sqrtf(xn) : xn + cmax;
+    const float scale = cosine ? sqrtf(xn) : xn + cmax;
     const bool near_tie = valid && h == 0 && !((second - best) > unit * scale);
     uint64_t todo = __ballot(near_tie);
     while (todo) {
       const int src = __ffsll((unsigned long long)todo) - 1;
       todo &= todo - 1;
       const int64_t rrow = tile * 32 + (src & 31);
-      const int exact = exact_argmin_row(x + rrow * k, centers, n, k, metric, lane);
+      const int exact = cosine ? exact_argmin_row(x + rrow * k, centers, n, k, metric, lane)
+                               : exact_argmin_row_l2_lds(x + rrow * k, cT, n, n_pad, KH, khalf, k, lane);
       if (lane == src) besti = exact;
     }
     if (valid && h == 0) {
@@ -296,8 +357,20 @@ int launch_mfma(const float* x, const float* centers, int64_t* l64, uint8_t* l8,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "kmeans_predict: cannot reserve %zu B of LDS", lds);
   }
-  int per_cu = (int)((144 * 1024) / lds);
-  per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
+  // The tiles are dealt round-robin to a grid that must be resident all at once (a workgroup
+  // that starts late does its whole share after the others have finished), so size the grid
+  // from the occupancy the registers and LDS of this instantiation really allow.
+  static thread_local size_t cached_lds = 0;   // per instantiation (KH) and thread
+  static thread_local int cached_per_cu = 0;
+  if (cached_per_cu == 0 || cached_lds != lds) {
+    int v = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, reinterpret_cast<const void*>(kern), 256, lds) !=
+            hipSuccess || v < 1)
+      v = 1;
+    cached_per_cu = v;
+    cached_lds = lds;
+  }
+  const int per_cu = cached_per_cu;
   int64_t need = ceil_div(ceil_div(m, 32), 4);
   int64_t cap = (int64_t)num_cus() * per_cu;
   const int grid = (int)(need < cap ? need : cap);
@@ -342,7 +415,7 @@ extern "C" int f2cgt_kmeans_predict(const float* x, const float* centers, int64_
   const int khalf = (int)((k + 1) / 2);
   int kh = pow2_ceil(khalf);
   if (kh < 4) kh = 4;
-  const int n_pad = (int)ceil_div(n, 32) * 32;
+  const int n_pad = (int)ceil_div(n, 64) * 64;  // two 32-centre tiles per step
   const size_t lds = ((size_t)2 * kh * n_pad + 2 * (size_t)n_pad + 4) * sizeof(float);
   if (kh <= 32 && lds <= 96 * 1024) {
     switch (kh) {
