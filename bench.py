@@ -31,11 +31,11 @@ MFMA_F32_PEAK_TFLOPS = 157.3
 # what the same counter reads for a plain copy of known size; see profiles/).  Keyed by
 # (workload name, index dtype).  Missing = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1_sq8_affine", "int64"): 18279493,
-    ("c2_sq4_affine", "int64"): 132288366,
-    ("c3_vq_16x8", "int64"): 487431606,
-    ("c4_hybrid", "int64"): 1003788187,
-    ("c5_vq_24x32", "int64"): 3306912153,
+    ("c1_sq8_affine", "int64"): 18288711,
+    ("c2_sq4_affine", "int64"): 134118977,
+    ("c3_vq_16x8", "int64"): 487330582,
+    ("c4_hybrid", "int64"): 1003957758,
+    ("c5_vq_24x32", "int64"): 2120850184,
 }
 
 
@@ -133,6 +133,9 @@ def _others(idx):
     params = torch.rand((2, d), device="cuda")
     _, ms = _time_steps(lambda: capi.sq_affine_decompress(packed, params, 4, d), 20, 3)
     res["sq_affine_decompress_4bit_2.4Mx100"] = {"launch_us": ms * 1e3, "GBps": n * d * 4.5 / (ms * 1e-3) / 1e9}
+    logcb = torch.tensor([[0.01, 3.0, -6.643856, 1.5849625, 0.4]], device="cuda")
+    _, ms = _time_steps(lambda: capi.sq_decompress(packed, logcb, 4, d, d), 20, 3)
+    res["sq_decompress_4bit_2.4Mx100"] = {"launch_us": ms * 1e3, "GBps": n * d * 4.5 / (ms * 1e-3) / 1e9}
     cb = torch.randn((16, 256, 8), device="cuda")
     vq = torch.randint(0, 256, (n, 16), dtype=torch.uint8, device="cuda")
     _, ms = _time_steps(lambda: capi.vq_decompress(vq, cb, 128), 20, 3)
