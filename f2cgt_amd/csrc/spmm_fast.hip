@@ -1025,6 +1025,10 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
 
 bool sq_block_eligible(const void* codes, const float* out, int64_t N, int64_t src_dim, int feat_dim,
                        int target_bits, int64_t lut_entries) {
+  if (target_bits <= 2 && target_bits >= 1 && feat_dim % 4 == 0 && (int64_t)feat_dim * target_bits >= 64 &&
+      src_dim >= 8 && feat_dim <= 4096 && aligned(out, 16) && N < (1ll << 32) && src_dim < (1ll << 24) &&
+      src_dim * (8 / target_bits) >= feat_dim && lut_entries * 4 <= 16 * 1024)
+    return true;  // staged-rows kernel (any row pitch, float4 column groups)
   int lb, nout;
   switch (target_bits) {
     case 8: lb = 4; nout = 4; break;
