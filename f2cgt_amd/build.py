@@ -25,6 +25,9 @@ HIP_SOURCES = ["runtime.hip", "packbits.hip", "sq.hip", "vq.hip", "spmm.hip", "s
 HIP_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results go to ordinary VGPRs: the arg-min update of the encode kernel then reads the
+    # scores directly instead of copying every accumulator out of the AGPR file first
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-pragmas",
 ]
 

@@ -62,8 +62,15 @@ __device__ int exact_argmin_row(const float* __restrict__ xrow, const float* __r
   return besti;
 }
 
+// LDS layout of the MFMA A operands: [pair of 32-centre tiles][step][half][centre % 32][tile of pair].
+// Step 0 is the bias step, step 1 + t holds dimension half * khalf + t.  A lane reads both tiles
+// of a step with one 8-byte access whose address is the pair base plus an immediate offset.
+__device__ __forceinline__ int a_index(int centre, int step, int half, int KH) {
+  return ((((centre >> 6) * (KH + 1) + step) * 2 + half) * 32 + (centre & 31)) * 2 + ((centre >> 5) & 1);
+}
+
 // Same for the L2 metric with the centres already staged in LDS, transposed as
-// cT[(half * KH + t) * n_pad + centre] (dimension = half * khalf + t): lanes read consecutive words.
+// (layout: a_index).
 __device__ int exact_argmin_row_l2_lds(const float* __restrict__ xrow, const float* cT, int n, int n_pad, int KH,
                                        int khalf, int k, int lane) {
   double bestv = DBL_MAX;
@@ -72,7 +79,7 @@ __device__ int exact_argmin_row_l2_lds(const float* __restrict__ xrow, const flo
     double d = 0.0;
     for (int dim = 0; dim < k; ++dim) {
       const int hh = dim >= khalf ? 1 : 0;
-      const double df = (double)xrow[dim] - (double)cT[(hh * KH + dim - hh * khalf) * n_pad + c];
+      const double df = (double)xrow[dim] - (double)cT[a_index(c, 1 + dim - hh * khalf, hh, KH)];
       d += df * df;
     }
     if (d < bestv) { bestv = d; besti = c; }
@@ -133,38 +140,38 @@ __global__ __launch_bounds__(256) void predict_mfma_kernel(const float* __restri
                                                            uint8_t* __restrict__ lab8, int64_t m,
                                                            int n, int k, int metric, int n_pad) {
   extern __shared__ float smem[];
-  float* cT = smem;                   // [2*KH][n_pad]  centre coordinates, transposed
-  float* cB = cT + 2 * KH * n_pad;    // [2][n_pad]  bias row (half 0) and a zero row (half 1)
-  int* cmax_bits = reinterpret_cast<int*>(cB + 2 * n_pad);  // max |c|^2 as ordered int bits
+  float* cT = smem;                   // [n_pad / 64][KH + 1][2][32][2], see a_index
+  const int a_floats = (n_pad >> 6) * (KH + 1) * 128;
+  int* cmax_bits = reinterpret_cast<int*>(cT + a_floats);  // max |c|^2 as ordered int bits
 
   const int khalf = (k + 1) / 2;
   const bool cosine = metric == F2CGT_METRIC_COSINE;
   if (threadIdx.x == 0) *cmax_bits = 0;
-  __syncthreads();
-  // stage the centres transposed: coalesced reads of the [n, k] array, scattered LDS writes
-  for (int i = threadIdx.x; i < 2 * KH * n_pad; i += blockDim.x) cT[i] = 0.f;
+  // stage the centres: coalesced reads of the [n, k] array, scattered LDS writes
+  for (int i = threadIdx.x; i < a_floats; i += blockDim.x) cT[i] = 0.f;
   __syncthreads();
 #pragma unroll 8
   for (int i = threadIdx.x; i < n * k; i += blockDim.x) {
     const int jj = i / k, dim = i - jj * k;
     const int hh = dim >= khalf ? 1 : 0;
-    cT[(hh * KH + dim - hh * khalf) * n_pad + jj] = centers[i];
+    cT[a_index(jj, 1 + dim - hh * khalf, hh, KH)] = centers[i];
   }
   __syncthreads();
   for (int jj = threadIdx.x; jj < n_pad; jj += blockDim.x) {
     float cn = 0.f;
+    for (int hh = 0; hh < 2; ++hh)
 #pragma unroll 4
-    for (int kk = 0; kk < 2 * KH; ++kk) {
-      const float v = cT[kk * n_pad + jj];
-      cn += v * v;
-    }
+      for (int t = 0; t < KH; ++t) {
+        const float v = cT[a_index(jj, 1 + t, hh, KH)];
+        cn += v * v;
+      }
     if (cosine) {
       const float nr = sqrtf(cn);
       const float scale = 1.f / (nr > 1e-30f ? nr : 1e-30f);
-      for (int kk = 0; kk < 2 * KH; ++kk) cT[kk * n_pad + jj] *= scale;
+      for (int hh = 0; hh < 2; ++hh)
+        for (int t = 0; t < KH; ++t) cT[a_index(jj, 1 + t, hh, KH)] *= scale;
     }
-    cB[jj] = jj >= n ? INFINITY : (cosine ? 0.f : cn);
-    cB[n_pad + jj] = 0.f;
+    cT[a_index(jj, 0, 0, KH)] = jj >= n ? INFINITY : (cosine ? 0.f : cn);  // bias, times 1 in half 0
     if (jj < n && !cosine) atomicMax(cmax_bits, __float_as_int(cn));
   }
   __syncthreads();
@@ -178,8 +185,7 @@ __global__ __launch_bounds__(256) void predict_mfma_kernel(const float* __restri
   const bool vec4 = (k % 8 == 0) && (KH % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
   const float xscale = cosine ? -1.f : -2.f;
   const float xb = h == 0 ? 1.f : 0.f;
-  const float* ap = cT + (h * KH) * n_pad + j;
-  const float* bp = cB + h * n_pad + j;
+  const float2* ap = reinterpret_cast<const float2*>(cT) + h * 32 + j;  // + (pair * (KH + 1) + step) * 64
 
   // raw coordinates of this lane's x row (its half of the k dimensions) for one tile
   auto load_x = [&](int64_t tile, float (&q)[KH]) {
@@ -226,12 +232,15 @@ __global__ __launch_bounds__(256) void predict_mfma_kernel(const float* __restri
       floatx16 zero;
 #pragma unroll
       for (int v = 0; v < 16; ++v) zero[v] = 0.f;
-      floatx16 acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(bp[ct], xb, zero, 0, 0, 0);
-      floatx16 acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(bp[ct + 32], xb, zero, 0, 0, 0);
+      const float2* pp = ap + (ct >> 6) * (KH + 1) * 64;
+      const float2 b01 = pp[0];
+      floatx16 acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(b01.x, xb, zero, 0, 0, 0);
+      floatx16 acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(b01.y, xb, zero, 0, 0, 0);
 #pragma unroll
       for (int t = 0; t < KH; ++t) {
-        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[t * n_pad + ct], xr[t], acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[t * n_pad + ct + 32], xr[t], acc1, 0, 0, 0);
+        const float2 a01 = pp[(t + 1) * 64];
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a01.x, xr[t], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a01.y, xr[t], acc1, 0, 0, 0);
       }
       argmin_update(acc0, ct, best, second, bv, bct);
       argmin_update(acc1, ct + 32, best, second, bv, bct);
