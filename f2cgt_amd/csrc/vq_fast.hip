@@ -268,6 +268,218 @@ __global__ __launch_bounds__(kThreads) void vq_pipe_kernel(VqArgs a, const Idx* 
   }
 }
 
+// ---- wave-granular variant ------------------------------------------------------------------
+// Same codebook tile, lane mapping and inner loop, but every wave of the workgroup runs its own
+// pipeline, with wave-private staging in LDS.  After the codebook is staged no workgroup barrier
+// is left: a wave that waits for its loads does not hold the other fifteen, and the LDS
+// operations of one wave execute in order, so its own stage hand-overs need no synchronisation.
+// A wave owns chunks of 48 consecutive destination rows and walks them as twelve 4-row
+// mini-blocks (<= 64 edges: one edge per lane in the I and C stages; larger ones are summed
+// straight from HBM):
+//     P  the 49 row offsets of a chunk     one load per chunk, issued while the previous chunk
+//                                          starts, parked half a chunk later (two LDS buffers)
+//     I  source id of edge `lane`          issued two mini-blocks ahead, stays in the register
+//     C  code bytes of edge `lane`         issued one mini-block ahead, parked in LDS when due
+// Everything that is the same for all lanes (mini-block bounds, row numbers, base addresses) is
+// kept in scalar registers; the vector instructions outside the inner loop are what bounded the
+// block-synchronous version of this kernel.
+constexpr int kWRows = 4;
+constexpr int kWEdges = 64;
+constexpr int kWMini = 12;                    // mini-blocks per chunk
+constexpr int kWChunk = kWRows * kWMini;      // rows per chunk
+constexpr int kWPtr = 56;                     // ints per offset buffer: [0..48] offsets, [52..53] first edge
+
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+template <int BT, typename Idx>
+__global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* __restrict__ indptr,
+                                                           const Idx* __restrict__ indices,
+                                                           float* __restrict__ out) {
+  using CW = typename code_word<BT>::type;
+  constexpr int kWaves = kThreads / 64;
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* s_cb = reinterpret_cast<float*>(smem);
+  const int wave = uni((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  unsigned char* s_codes = smem + (size_t)a.K * 128 * 4 + (size_t)wave * kWEdges * BT;
+  int* s_ptr = reinterpret_cast<int*>(smem + (size_t)a.K * 128 * 4 + (size_t)kWaves * kWEdges * BT) + wave * 2 * kWPtr;
+
+  int tile, stripe;
+  if (a.stripes_per_xcd > 0) {
+    const int xcd = blockIdx.x % kXcds, k = blockIdx.x / kXcds;
+    if (k >= a.stripes_per_xcd * a.n_tiles) return;
+    tile = k % a.n_tiles;
+    stripe = xcd * a.stripes_per_xcd + k / a.n_tiles;
+  } else {
+    tile = blockIdx.x % a.n_tiles;
+    stripe = blockIdx.x / a.n_tiles;
+  }
+  const int tile_cols = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
+  for (int i = threadIdx.x; i < a.K * 128; i += kThreads) {
+    const int code = i >> 7, c = i & 127;
+    float v = 0.f;
+    if (c < tile_cols) {
+      const int col = tile * 128 + c;
+      const int sub = col / a.w;
+      v = a.codebooks[((int64_t)sub * a.K + code) * a.w + (col - sub * a.w)];
+    }
+    s_cb[i] = v;
+  }
+  __syncthreads();
+
+  // A wave owns one contiguous range of rows (a multiple of 4, the same for every wave, so the
+  // work is balanced to one mini-block); chunk c of the wave covers rows [chunk_row0 + 48 c, +48).
+  const int64_t total_waves = (int64_t)a.n_stripes * kWaves;
+  const int64_t rows_per_wave = ((a.R + total_waves - 1) / total_waves + kWRows - 1) / kWRows * kWRows;
+  const int64_t chunk_stride = kWChunk;
+  const int64_t chunk_row0 = ((int64_t)stripe * kWaves + wave) * rows_per_wave;
+  if (chunk_row0 >= a.R) return;
+  const int64_t row_end = chunk_row0 + rows_per_wave < a.R ? chunk_row0 + rows_per_wave : a.R;
+  const int64_t n_chunks = (row_end - chunk_row0 + kWChunk - 1) / kWChunk;
+  const int64_t n_mini = (row_end - chunk_row0 + kWRows - 1) / kWRows;
+
+  const int c4 = lane & 31, half = lane >> 5;
+  const bool col_on = c4 * 4 < tile_cols;
+  const int byte_idx = (c4 * 4) / a.w;
+  const float* cbp = s_cb + c4 * 4;
+  const uint8_t* code_base = a.codes + tile * BT;
+  const uint32_t n_last = (uint32_t)(a.N - 1);
+
+  // loads and parks the offsets of chunk c into buffer (c & 1); returns nothing, the data is in LDS
+  int64_t Preg = 0;
+  auto issue_P = [&](int64_t c) {
+    const int64_t row0 = chunk_row0 + c * chunk_stride;
+    const int64_t left = row_end - row0;
+    const int nr = (int)(left < kWChunk ? left : kWChunk);
+    Preg = (int64_t)indptr[row0 + (lane < nr ? lane : nr)];
+  };
+  auto park_P = [&](int64_t c) {
+    int* buf = s_ptr + (int)(c & 1) * kWPtr;
+    const uint32_t lo = (uint32_t)uni((int)(uint32_t)Preg);
+    const uint32_t hi = (uint32_t)uni((int)(uint32_t)((uint64_t)Preg >> 32));
+    int64_t e0 = (int64_t)(((uint64_t)hi << 32) | lo);
+    e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
+    int64_t v = Preg;
+    v = v < e0 ? e0 : (v > a.E ? a.E : v);
+    const int64_t rel = v - e0;
+    if (lane <= kWChunk) buf[lane] = rel > 0x3fffffff ? 0x3fffffff : (int)rel;
+    if (lane == 1) { buf[52] = (int)(uint32_t)e0; buf[53] = (int)(uint32_t)((uint64_t)e0 >> 32); }
+  };
+  // bounds of mini-block g: first edge (relative to the chunk's e0) and edge count
+  auto bounds = [&](int64_t g, int& eb, int& ne) {
+    const int64_t c = g / kWMini;
+    const int m = (int)(g - c * kWMini);
+    const int* buf = s_ptr + (int)(c & 1) * kWPtr;
+    eb = uni(buf[m * kWRows]);
+    const int ee = uni(buf[m * kWRows + kWRows]);
+    ne = ee - eb;
+    ne = ne < 0 ? 0 : ne;
+  };
+  auto chunk_e0 = [&](int64_t c) {
+    const int* buf = s_ptr + (int)(c & 1) * kWPtr;
+    const uint32_t lo = (uint32_t)uni(buf[52]), hi = (uint32_t)uni(buf[53]);
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+  };
+
+  issue_P(0);
+  park_P(0);
+  int eb0 = 0, ne0 = 0;      // mini-block g
+  int eb1 = 0, ne1 = 0;      // g + 1
+  int64_t Ireg = 0;
+  CW Creg = {};
+  for (int64_t g = -2; g < n_mini; ++g) {
+    // chunk-level P stage, driven by the position of g inside its chunk
+    if (g >= 0) {
+      const int64_t c = g / kWMini;
+      const int m = (int)(g - c * kWMini);
+      if (m == 0 && c + 1 < n_chunks) issue_P(c + 1);
+      if (m == kWMini / 2 && c + 1 < n_chunks) park_P(c + 1);
+    }
+    // park C(g)
+    if (g >= 0 && ne0 <= kWEdges && lane < ne0) *reinterpret_cast<CW*>(s_codes + lane * BT) = Creg;
+    // issue C(g+1): the id fetched one step ago is clamped only now
+    {
+      const bool on = g + 1 >= 0 && g + 1 < n_mini && ne1 <= kWEdges && lane < ne1;
+      const uint64_t raw = (uint64_t)Ireg;
+      const uint32_t id = (raw >> 32) ? n_last : ((uint32_t)raw < n_last ? (uint32_t)raw : n_last);
+      Creg = *reinterpret_cast<const CW*>(code_base + (uint64_t)(on ? id : 0u) * (uint32_t)a.n_cb);
+    }
+    // issue I(g+2)
+    int eb2 = 0, ne2 = 0;
+    {
+      const bool v = g + 2 < n_mini;
+      int64_t e0 = 0;
+      if (v) {
+        bounds(g + 2, eb2, ne2);
+        e0 = chunk_e0((g + 2) / kWMini);
+      }
+      const bool on = v && ne2 <= kWEdges && lane < ne2;
+      const Idx* src = on ? indices + e0 + eb2 + lane : indptr;
+      Ireg = (int64_t)*src;
+    }
+    // compute mini-block g
+    if (g >= 0 && col_on) {
+      const int64_t c = g / kWMini;
+      const int m = (int)(g - c * kWMini);
+      const int* buf = s_ptr + (int)(c & 1) * kWPtr + m * kWRows;
+      const int64_t row0 = chunk_row0 + c * chunk_stride + m * kWRows;
+      const int64_t left = row_end - row0;
+      const int nr = (int)(left < kWRows ? left : kWRows);
+      const bool staged = ne0 <= kWEdges;
+      float* orow = out + row0 * (int64_t)a.feat_dim + tile * 128 + c4 * 4;
+#pragma unroll
+      for (int pass = 0; pass < kWRows / 2; ++pass) {
+        const int row = pass * 2 + half;
+        if (row >= nr) continue;
+        int rb = buf[row] - eb0, re = buf[row + 1] - eb0;
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        int n;
+        if (staged) {
+          rb = rb < 0 ? 0 : (rb > ne0 ? ne0 : rb);
+          re = re < 0 ? 0 : (re > ne0 ? ne0 : re);
+          n = re - rb;
+          const unsigned char* cp = s_codes + rb * BT + byte_idx;
+          int k = 0;
+          for (; k + kGroup <= n; k += kGroup) {
+            uint32_t code[kGroup];
+            float4 x[kGroup];
+#pragma unroll
+            for (int u = 0; u < kGroup; ++u) code[u] = cp[u * BT];
+            cp += kGroup * BT;
+#pragma unroll
+            for (int u = 0; u < kGroup; ++u) x[u] = *reinterpret_cast<const float4*>(cbp + code[u] * 128);
+#pragma unroll
+            for (int u = 0; u < kGroup; ++u) { a0 += x[u].x; a1 += x[u].y; a2 += x[u].z; a3 += x[u].w; }
+          }
+          for (; k < n; ++k) {
+            const uint32_t code = *cp;
+            cp += BT;
+            const float4 x = *reinterpret_cast<const float4*>(cbp + code * 128);
+            a0 += x.x; a1 += x.y; a2 += x.z; a3 += x.w;
+          }
+        } else {
+          n = re - rb;
+          const int64_t e0 = chunk_e0(c) + eb0;
+          for (int k = 0; k < n; ++k) {
+            const int64_t id = clamp_idx(indices[e0 + rb + k], a.N);
+            const uint32_t code = a.codes[id * a.n_cb + tile * BT + byte_idx];
+            const float4 x = *reinterpret_cast<const float4*>(cbp + code * 128);
+            a0 += x.x; a1 += x.y; a2 += x.z; a3 += x.w;
+          }
+        }
+        if (n > 1) {
+          const float d = (float)n;
+          float r = __builtin_amdgcn_rcpf(d);
+          r = __fmaf_rn(__fmaf_rn(-d, r, 1.f), r, r);
+          a0 = div_by(a0, d, r); a1 = div_by(a1, d, r); a2 = div_by(a2, d, r); a3 = div_by(a3, d, r);
+        }
+        store_nt4(orow + (int64_t)row * a.feat_dim, a0, a1, a2, a3);
+      }
+    }
+    eb0 = eb1; ne0 = ne1;
+    eb1 = eb2; ne1 = ne2;
+  }
+}
+
 template <int BT>
 int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
               const char* what) {
@@ -292,6 +504,25 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e1 != hipSuccess || e2 != hipSuccess)
     return fail((int)(e1 != hipSuccess ? e1 : e2), "%s: cannot reserve %zu B of LDS", what, lds);
+  const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 0.0;
+  // graphs whose 4-row mini-blocks mostly fit the 64-edge staging take the wave-granular kernel
+  if (avg_deg * kWRows <= 60.0) {
+    const size_t wlds = (size_t)a.K * 128 * 4 + (size_t)(kThreads / 64) * kWEdges * BT +
+                        (size_t)(kThreads / 64) * 2 * kWPtr * 4;
+    hipError_t w1 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_wave_kernel<BT, int32_t>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
+    hipError_t w2 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_wave_kernel<BT, int64_t>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
+    if (w1 != hipSuccess || w2 != hipSuccess)
+      return fail((int)(w1 != hipSuccess ? w1 : w2), "%s: cannot reserve %zu B of LDS", what, wlds);
+    if (idx_dtype == F2CGT_DT_I32)
+      vq_wave_kernel<BT, int32_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int32_t*>(indptr),
+                                                                static_cast<const int32_t*>(indices), out);
+    else
+      vq_wave_kernel<BT, int64_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int64_t*>(indptr),
+                                                                static_cast<const int64_t*>(indices), out);
+    return launch_status(what);
+  }
   if (idx_dtype == F2CGT_DT_I32)
     vq_pipe_kernel<BT, int32_t><<<grid, kThreads, lds, st>>>(a, static_cast<const int32_t*>(indptr),
                                                             static_cast<const int32_t*>(indices), out);
