@@ -287,6 +287,21 @@ def test_fused_vq_vs_oracle(idx, shape):
     assert close(got, unfused)
 
 
+@pytest.mark.parametrize("max_deg,rows", [(50, 1500), (200, 700), (3, 4099)])
+def test_fused_vq_degree_regimes(max_deg, rows):
+    # average degree above 15: block-synchronous pipeline (blocks above 1024 edges summed from
+    # HBM at max_deg 200); below: wave-granular pipeline, with a row count that leaves partial
+    # chunks and mini-blocks; both keep the sequential edge order, so the result is bit-exact
+    rng = np.random.default_rng(max_deg)
+    N = 3000
+    cb = rng.standard_normal((16, 256, 8)).astype(np.float32)
+    codes = rng.integers(0, 256, size=(N, 16), dtype=np.uint8)
+    indptr, indices = random_graph(rng, rows, N, max_deg)
+    got = host(capi.vq_decompress_spmm_csr(dev(codes), dev(cb), dev(indptr), dev(indices), 128))
+    want = oc.vq_decompress_spmm_csr(codes, cb, indptr, indices, 128)
+    assert np.array_equal(got, want)
+
+
 def test_fused_vq_int16_codes_big_codebook():
     rng = np.random.default_rng(5)
     cb = rng.standard_normal((2, 5000, 8)).astype(np.float32)   # 160 KB per slice: global path
