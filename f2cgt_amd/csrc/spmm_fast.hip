@@ -896,8 +896,10 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
       const int gslot = t / lanes;
       const int gslots = kBlock / lanes;
       constexpr int U = 4;
-      // lane j of the lanes that share an edge takes dwords j, j+q, j+2q, j+3q (q = chunks / 4):
-      // every load and every atomic instruction touches q consecutive words per edge
+      // lane j of the lanes that share an edge loads dwords 4j .. 4j+3 with one 16-byte access (the
+      // lanes of an edge cover its 128-byte line once; four strided dword loads per lane kept
+      // hitting lines still in flight and stalled the L1) and adds dword 4j+c to accumulator word
+      // c*q + j (q = chunks / 4), so every atomic instruction touches q consecutive words per edge
       const int per = (nb + gslots - 1) / gslots;
       const int e_begin = gslot * per;
       const int e_end = (e_begin + per) < nb ? (e_begin + per) : nb;
@@ -913,9 +915,12 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
           row[u] = s_row[ee];
           er[u] = s_erow[ee];
           const bool on = lane_on && (row[u] >> 30) == 0;
-          const uint32_t* src = codes32 + (int64_t)row[u] * dwords_per_row + j;
+          typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+          const u32x4 zero4 = {0u, 0u, 0u, 0u};
+          const u32x4 v4 = on ? *reinterpret_cast<const u32x4*>(codes32 + (int64_t)row[u] * dwords_per_row + 4 * j)
+                              : zero4;
 #pragma unroll
-          for (int c = 0; c < 4; ++c) w[u][c] = on ? src[c * q] : 0u;
+          for (int c = 0; c < 4; ++c) w[u][c] = v4[c];
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -966,8 +971,10 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
     const int r = (int)__umulhi((uint32_t)it, a.magic);
     const int c4 = it - r * a.chunks;
     uint2 q;
-    q.x = s_acc[r * acc_pitch + c4];
-    q.y = s_acc[r * acc_pitch + a.chunks + c4];
+    // (the 16-byte gather stores dword c4 of a row at word (c4 % 4) * chunks / 4 + c4 / 4)
+    const int pos = VEC == 4 ? (c4 & 3) * (a.chunks >> 2) + (c4 >> 2) : c4;
+    q.x = s_acc[r * acc_pitch + pos];
+    q.y = s_acc[r * acc_pitch + a.chunks + pos];
     const int b = s_ptr[r], e = s_ptr[r + 1];
     const int deg = e - b;
     const int nvq = s_nvq[r];
