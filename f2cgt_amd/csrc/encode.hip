@@ -1,8 +1,8 @@
 // VQ encode: pairwise distance and nearest-centre assignment.
 //
-// pairwise_distance materialises the [m,n] matrix and is bounded by that write; it
-// evaluates the unexpanded form sum((x-y)^2) (or 1 - cos) on the vector ALUs so the
-// numbers carry no cancellation error.
+// pairwise_distance materialises the [m,n] matrix; it evaluates the unexpanded form
+// sum((x-y)^2) (or 1 - cos) with fused multiply-adds on the vector ALUs, so the numbers carry
+// no cancellation error, and at small k the vector ALUs rather than the matrix write bound it.
 //
 // kmeans_predict never writes the matrix.  A wave owns 32 rows of x and walks the
 // centres 64 at a time with fp32 MFMA (v_mfma_f32_32x32x2_f32): A = centre tile,
@@ -277,29 +277,33 @@ __global__ __launch_bounds__(256) void predict_mfma_kernel(const float* __restri
 }
 
 // ---- pairwise distance --------------------------------------------------------------------
-constexpr int kTile = 64;   // rows of x and of y per workgroup
-constexpr int kChunk = 32;  // k dimensions staged per pass
+// 128 x 128 output tile per 256-thread workgroup, 8 x 8 per thread: per staged k step a thread
+// reads 8 + 8 values from LDS (four 16-byte reads) for 64 fused multiply-adds, so the vector
+// ALUs, not LDS, set the pace.  L2 is the unexpanded sum of squared differences.
+constexpr int kTile = 128;  // rows of x and of y per workgroup
+constexpr int kChunk = 16;  // k dimensions staged per pass
 
 __global__ __launch_bounds__(256) void pairwise_kernel(const float* __restrict__ x,
                                                        const float* __restrict__ y,
                                                        float* __restrict__ dist, int64_t m, int64_t n,
                                                        int k, int metric) {
-  __shared__ float xs[kChunk][kTile + 1];
-  __shared__ float ys[kChunk][kTile + 1];
-  const int tx = threadIdx.x & 15;  // 4 y rows each
-  const int ty = threadIdx.x >> 4;  // 4 x rows each
+  __shared__ __align__(16) float xs[kChunk][kTile + 4];
+  __shared__ __align__(16) float ys[kChunk][kTile + 4];
+  const int tx = threadIdx.x & 15;  // 8 y rows each
+  const int ty = threadIdx.x >> 4;  // 8 x rows each
+  const bool cosine = metric == F2CGT_METRIC_COSINE;
   const int64_t n_tiles_n = (n + kTile - 1) / kTile;
   const int64_t n_tiles = ((m + kTile - 1) / kTile) * n_tiles_n;
   for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
     const int64_t i0 = (tile / n_tiles_n) * kTile;
     const int64_t j0 = (tile % n_tiles_n) * kTile;
-    float acc[4][4], xn[4], yn[4];
+    float acc[8][8], xn[8], yn[8];
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
+    for (int a = 0; a < 8; ++a) {
       xn[a] = 0.f;
       yn[a] = 0.f;
 #pragma unroll
-      for (int b = 0; b < 4; ++b) acc[a][b] = 0.f;
+      for (int b = 0; b < 8; ++b) acc[a][b] = 0.f;
     }
     for (int k0 = 0; k0 < k; k0 += kChunk) {
       __syncthreads();
@@ -310,48 +314,57 @@ __global__ __launch_bounds__(256) void pairwise_kernel(const float* __restrict__
         ys[c][r] = (kin && j0 + r < n) ? y[(j0 + r) * k + k0 + c] : 0.f;
       }
       __syncthreads();
-      const int kc = (k - k0) < kChunk ? (k - k0) : kChunk;
-      for (int c = 0; c < kc; ++c) {
-        float xv[4], yv[4];
+#pragma unroll 4
+      for (int c = 0; c < kChunk; ++c) {
+        float xv[8], yv[8];
+        const float4 xa = *reinterpret_cast<const float4*>(&xs[c][ty * 8]);
+        const float4 xb = *reinterpret_cast<const float4*>(&xs[c][ty * 8 + 4]);
+        const float4 ya = *reinterpret_cast<const float4*>(&ys[c][tx * 8]);
+        const float4 yb = *reinterpret_cast<const float4*>(&ys[c][tx * 8 + 4]);
+        xv[0] = xa.x; xv[1] = xa.y; xv[2] = xa.z; xv[3] = xa.w; xv[4] = xb.x; xv[5] = xb.y; xv[6] = xb.z; xv[7] = xb.w;
+        yv[0] = ya.x; yv[1] = ya.y; yv[2] = ya.z; yv[3] = ya.w; yv[4] = yb.x; yv[5] = yb.y; yv[6] = yb.z; yv[7] = yb.w;
+        if (cosine) {
 #pragma unroll
-        for (int a = 0; a < 4; ++a) {
-          xv[a] = xs[c][ty * 4 + a];
-          yv[a] = ys[c][tx * 4 + a];
-        }
-        if (metric == F2CGT_METRIC_COSINE) {
+          for (int a = 0; a < 8; ++a) {
+            xn[a] = __fmaf_rn(xv[a], xv[a], xn[a]);
+            yn[a] = __fmaf_rn(yv[a], yv[a], yn[a]);
 #pragma unroll
-          for (int a = 0; a < 4; ++a) {
-            xn[a] += xv[a] * xv[a];
-            yn[a] += yv[a] * yv[a];
-#pragma unroll
-            for (int b = 0; b < 4; ++b) acc[a][b] += xv[a] * yv[b];
+            for (int b = 0; b < 8; ++b) acc[a][b] = __fmaf_rn(xv[a], yv[b], acc[a][b]);
           }
         } else {
 #pragma unroll
-          for (int a = 0; a < 4; ++a)
+          for (int a = 0; a < 8; ++a)
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
+            for (int b = 0; b < 8; ++b) {
               const float d = xv[a] - yv[b];
-              acc[a][b] += d * d;
+              acc[a][b] = __fmaf_rn(d, d, acc[a][b]);
             }
         }
       }
     }
+    const bool full = j0 + tx * 8 + 8 <= n && n % 4 == 0 && ((reinterpret_cast<uintptr_t>(dist) & 15) == 0);
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      const int64_t i = i0 + ty * 4 + a;
+    for (int a = 0; a < 8; ++a) {
+      const int64_t i = i0 + ty * 8 + a;
       if (i >= m) continue;
+      float v[8];
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const int64_t j = j0 + tx * 4 + b;
-        if (j >= n) continue;
-        float v = acc[a][b];
-        if (metric == F2CGT_METRIC_COSINE) {
+      for (int b = 0; b < 8; ++b) {
+        v[b] = acc[a][b];
+        if (cosine) {
           float den = sqrtf(xn[a]) * sqrtf(yn[b]);
           den = den > 1e-8f ? den : 1e-8f;
-          v = 1.f - v / den;
+          v[b] = 1.f - v[b] / den;
         }
-        dist[i * n + j] = v;
+      }
+      float* o = dist + i * n + j0 + tx * 8;
+      if (full) {
+        store_nt4(o, v[0], v[1], v[2], v[3]);
+        store_nt4(o + 4, v[4], v[5], v[6], v[7]);
+      } else {
+#pragma unroll
+        for (int b = 0; b < 8; ++b)
+          if (j0 + tx * 8 + b < n) o[b] = v[b];
       }
     }
   }
