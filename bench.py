@@ -116,6 +116,33 @@ def _others(idx):
                            "algorithmic_GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS}
         del wl
         torch.cuda.empty_cache()
+    # source ids passed through a fixed bijection (hot rows no longer contiguous), and int32 indices
+    for name, steps in (("c2", 500), ("c3", 100)):
+        wl = synth.scatter_ids(synth.WORKLOADS[name](device="cuda", idx_dtype=torch.int64))
+        out = torch.empty((wl["R"], wl["feat_dim"]), dtype=torch.float32, device="cuda")
+        _, ms_launch = _time_steps(_launcher(capi, wl, out), steps, steps // 10)
+        gbs = wl["algo_bytes"] / (ms_launch * 1e-3) / 1e9
+        res[wl["name"]] = {"launch_us": ms_launch * 1e3, "algorithmic_GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS}
+        del wl, out
+        torch.cuda.empty_cache()
+    other_idx = "int32" if idx == "int64" else "int64"
+    for name, steps in (("c2", 500), ("c3", 100), ("c4", 50)):
+        wl, ms_step, ms_launch = _run_workload(name, other_idx, steps, max(5, steps // 10))
+        gbs = wl["algo_bytes"] / (ms_launch * 1e-3) / 1e9
+        res[wl["name"] + "_" + other_idx] = {"launch_us": ms_launch * 1e3, "algorithmic_GBps": gbs,
+                                             "frac_hbm_peak": gbs / HBM_PEAK_GBS}
+        del wl
+        torch.cuda.empty_cache()
+    # the reference's own fused SQ operator (log-domain codes, [n,5] codebooks) on the C2 graph
+    wl = synth.WORKLOADS["c2"](device="cuda", idx_dtype=torch.int64)
+    out = torch.empty((wl["R"], wl["feat_dim"]), dtype=torch.float32, device="cuda")
+    logcb2 = torch.tensor([[0.01, 3.0, -6.643856, 1.5849625, 0.4]], device="cuda")
+    _, ms = _time_steps(lambda: capi.sq_decompress_spmm_csr(wl["codes"], logcb2, wl["indptr"], wl["indices"], 4,
+                                                            wl["feat_dim"], wl["feat_dim"], out=out), 300, 30)
+    res["c2_graph_log_sq4_fused"] = {"launch_us": ms * 1e3, "algorithmic_GBps": wl["algo_bytes"] / (ms * 1e-3) / 1e9,
+                                     "frac_hbm_peak": wl["algo_bytes"] / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    del wl, out
+    torch.cuda.empty_cache()
     enc = synth.c5_encode(device="cuda")
     labels = torch.empty((enc["m"],), dtype=torch.uint8, device="cuda")
     _, ms = _time_steps(lambda: capi.kmeans_predict(enc["x"], enc["centers"], "l2", u8=True, out=labels), 50, 5)

@@ -182,4 +182,25 @@ def c5_encode(device="cpu", m=1_000_000, k=32, n=256, seed=0):
                 flops=2.0 * m * n * k, algo_bytes=m * k * 4 + n * k * 4 + m)
 
 
+def scatter_ids(wl, mult=2_654_435_761):
+    """The same workload with every source id passed through a fixed bijection of [0, N)
+    (id -> id * mult mod N, mult coprime with N), so hot rows are no longer neighbours in the
+    table.  Only the id stream changes; row contents are i.i.d., so the tables stay as they are
+    (for the hybrid workload the row map is permuted with the ids)."""
+    n = wl["N"]
+    while math.gcd(mult, n) != 1:
+        mult += 2
+    idx = wl["indices"]
+    perm = (idx.to(torch.int64) * (mult % n)) % n if n < (1 << 31) else ((idx.to(torch.int64) % n) * (mult % n)) % n
+    out = dict(wl)
+    out["indices"] = perm.to(idx.dtype)
+    out["name"] = wl["name"] + "_scattered"
+    if wl["kind"] == "hybrid":
+        inv = torch.empty_like(wl["row_map"])
+        src = torch.arange(n, device=idx.device, dtype=torch.int64)
+        inv[(src * (mult % n)) % n] = wl["row_map"]
+        out["row_map"] = inv
+    return out
+
+
 WORKLOADS = {"c1": c1_sq8_affine, "c2": c2_sq4_affine, "c3": c3_vq, "c4": c4_hybrid, "c5": c5_vq_wide}
