@@ -1,0 +1,268 @@
+"""Callers of the operator library, mirrored from the reference's Python with plain tensors in
+place of DGL blocks, ShmTensor and torch.distributed (one process, one GPU):
+
+  * the offline encode pipeline: `sq_metadata`, `sq_compress`, `vq_metadata`, `vq_compress`
+    (examples/process_compress.py:16-68, 71-144, 147-292);
+  * `CompressionManager` (examples/compress.py:8-106): keeps the code tables and codebooks,
+    serves seed rows (first level) and neighbour rows (second level);
+  * `MySAGEConv` (examples/conv.py:9-76): GraphSAGE mean layer whose neighbour aggregation is the
+    fused decompress + mean operator.
+
+Everything numerical happens in `F2CGTLib` (f2cgt_amd.load()); this module only moves tensors.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+from torch import nn
+
+import f2cgt_amd
+
+
+def _capi():
+    return f2cgt_amd.load()
+
+
+# ---- encode pipeline -----------------------------------------------------------------------------
+def normalize(data):
+    """examples/process_compress.py:16-18."""
+    data_norm = data.norm(dim=1, p=2)
+    return data / data_norm.reshape(-1, 1) * data_norm.mean()
+
+
+def sampling(sample_size, num_items, hotness=None, generator=None):
+    """Row sample for the codebook statistics (examples/process_compress.py:21-34); with a
+    hotness vector the sample follows it, otherwise it is uniform without replacement."""
+    if hotness is None:
+        return torch.randperm(num_items, generator=generator)[:sample_size]
+    p = (hotness.double() / hotness.double().sum()).cpu().numpy()
+    p[-1] = 1.0 - p[:-1].sum()
+    size = min(sample_size, num_items)
+    return torch.from_numpy(np.random.choice(num_items, size, replace=False, p=p))
+
+
+def sq_metadata(sample):
+    """(fmin, fmax, emin, emax, mean) of one column slice from a sample of its rows:
+    float64 percentiles of |x| floored at 1e-5 / 2e-5, log2 in float64, mean lifted by 0.1 when
+    below 0.1 (examples/process_compress.py:45-68)."""
+    epsilon = 1e-5
+    sample = sample.float().abs().cpu()
+    fmin = max(np.percentile(sample.numpy(), 0.5), epsilon)
+    fmax = max(np.percentile(sample.numpy(), 99.5), 2 * epsilon)
+    fmin = torch.tensor(fmin)
+    fmax = torch.tensor(fmax)
+    emin = torch.log2(fmin)
+    emax = torch.log2(fmax).add(epsilon)
+    mean = sample.mean()
+    if mean < 0.1:
+        mean += 0.1
+    return fmin, fmax, emin, emax, mean
+
+
+def sq_compress(features, target_bits, column_slice, hotness=None, sample_index=None, batch_rows=1_000_000):
+    """-> (storage, codebooks).  storage: int8 [N, ceil(D * bits / 8)] holding the packed bit
+    patterns (bits <= 8) or int16 [N, D]; codebooks fp32 [ceil(D / column_slice), 5] on the GPU
+    (examples/process_compress.py:71-144, single process)."""
+    capi = _capi()
+    num_items, feat_dim = features.shape
+    if sample_index is None:
+        sample_index = sampling(250_000, num_items, hotness)
+    num_codebooks = (feat_dim + column_slice - 1) // column_slice
+    codebooks = torch.zeros((num_codebooks, 5), dtype=torch.float32)
+    for i in range(num_codebooks):
+        lo, hi = i * column_slice, min((i + 1) * column_slice, feat_dim)
+        vals = sq_metadata(features[sample_index.to(features.device), lo:hi])
+        for j, v in enumerate(vals):
+            codebooks[i, j] = v
+    codebooks = codebooks.cuda()
+    if target_bits <= 8:
+        dtype, tdim = torch.int8, int(math.ceil(feat_dim / 8 * target_bits))
+    elif target_bits <= 16:
+        dtype, tdim = torch.int16, feat_dim
+    else:
+        raise NotImplementedError
+    out = torch.empty((num_items, tdim), dtype=dtype, device="cuda")
+    for start in range(0, num_items, batch_rows):
+        end = min(start + batch_rows, num_items)
+        data = features[start:end].cuda().to(torch.float32)
+        codes = capi.sq_compress(data, codebooks, target_bits, column_slice)
+        if target_bits < 8:
+            exp = capi.packbits(codes.to(torch.uint8), target_bits).view(torch.int8)
+        elif target_bits == 8:
+            exp = codes.to(torch.int8)
+        else:
+            exp = codes.to(torch.int16)
+        out[start:end].copy_(exp)
+    return out, codebooks
+
+
+def vq_metadata(features, n_clusters, column_slice, hotness=None, sample_index=None, max_iter=30):
+    """Codebooks fp32 [ceil(D / column_slice), n_clusters, column_slice]: per slice, rows of a
+    sample inside the rim quantile are dropped, k-means (cosine, tol 5e-2) runs on the rest and the
+    centres are rescaled to their mean norm (examples/process_compress.py:147-182)."""
+    capi = _capi()
+    num_items, feat_dim = features.shape
+    if sample_index is None:
+        sample_index = sampling(150_000, num_items, hotness)
+    num_slice = (feat_dim + column_slice - 1) // column_slice
+    codebooks = torch.zeros((num_slice, n_clusters, column_slice), device="cuda", dtype=torch.float32)
+    for i in range(num_slice):
+        lo, hi = i * column_slice, min((i + 1) * column_slice, feat_dim)
+        data = features[sample_index.to(features.device), lo:hi].to(torch.float32).cuda()
+        distance = data.norm(dim=1, p=2)
+        rim = torch.quantile(distance, min(1.0, 0.00625 * (data.shape[1] / 8)))
+        data = data[torch.ge(distance, rim)].contiguous()
+        km = capi.KMeans(n_clusters, hi - lo, "cosine", max_iter=max_iter, tol=5e-2)
+        km.fit(data)
+        centers = normalize(km.get_centers())
+        codebooks[i, :, :hi - lo] = centers
+    if torch.isnan(codebooks).any():
+        raise ValueError("codebooks has nan")
+    return codebooks
+
+
+def vq_compress(features, n_clusters, column_slice, hotness=None, codebooks=None, sample_index=None,
+                batch_rows=1_000_000):
+    """-> (codes, codebooks).  codes: uint8 (K <= 256) or int16 [N, n_slices], one nearest
+    (cosine) centre per column slice (examples/process_compress.py:185-292, single process)."""
+    capi = _capi()
+    num_items, feat_dim = features.shape
+    if codebooks is None:
+        codebooks = vq_metadata(features, n_clusters, column_slice, hotness, sample_index)
+    num_slice = codebooks.shape[0]
+    if n_clusters <= 256:
+        dtype = torch.uint8
+    elif n_clusters <= 32767:
+        dtype = torch.int16
+    else:
+        raise NotImplementedError("more than 32767 centres do not fit the int16 code type")
+    out = torch.empty((num_items, num_slice), dtype=dtype, device="cuda")
+    predictors = [capi.KMeans(codebooks[i].contiguous(), "cosine") for i in range(num_slice)]
+    for start in range(0, num_items, batch_rows):
+        end = min(start + batch_rows, num_items)
+        for i in range(num_slice):
+            lo, hi = i * column_slice, min((i + 1) * column_slice, feat_dim)
+            if hi <= lo:
+                continue
+            data = torch.zeros((end - start, column_slice), device="cuda", dtype=torch.float32)
+            data[:, :hi - lo] = features[start:end, lo:hi].to(torch.float32)
+            labels = predictors[i].predict(data, normalize_weights=False)
+            out[start:end, i] = labels.to(dtype)
+    return out, codebooks
+
+
+# ---- runtime callers -------------------------------------------------------------------------------
+class CompressionManager:
+    """examples/compress.py:8-106 on plain tensors.
+
+    `compress_data` keys (the layout of the reference's `compression_meta.pt` + data tensors):
+    `methods` (list of 'sq' / 'vq', one entry, or two for seeds + everything), `feat_dim`,
+    `configs` (per level (column_slice, target_bits)), `codebooks` (per level), `compression_data`
+    (code table of the last level, [N, src_dim]), and for two levels `seeds_compression_data`
+    (code table of the seed rows) with `seeds` (their global ids).
+    """
+
+    def __init__(self, compress_data, fusion=False):
+        self.meta = compress_data
+        self.methods = compress_data["methods"]
+        self.feat_dim = compress_data["feat_dim"]
+        self.configs = compress_data["configs"]
+        self.codebooks = [c.cuda() for c in compress_data["codebooks"]]
+        self.data = compress_data["compression_data"].cuda()
+        self.seeds_data = None
+        self.is_two_level = len(self.methods) >= 2
+        self.is_fusion = fusion
+        if self.is_two_level:
+            self.seeds_data = compress_data["seeds_compression_data"].cuda()
+            keys = compress_data["seeds"].long().cuda()
+            # global id -> row of the seed table (the reference keeps a GPU hash map)
+            self.seed_slot = torch.full((self.data.shape[0],), -1, dtype=torch.int32, device="cuda")
+            self.seed_slot[keys] = torch.arange(keys.numel(), dtype=torch.int32, device="cuda")
+
+    def _decompress(self, level, data):
+        capi = _capi()
+        if self.methods[level] == "vq":
+            return capi.vq_decompress(data, self.codebooks[level], self.feat_dim)
+        return capi.sq_decompress(data, self.codebooks[level], self.configs[level][1], self.configs[level][0],
+                                  self.feat_dim)
+
+    def get_seeds_data(self, seeds_key):
+        if not self.is_two_level:
+            return None
+        slots = self.seed_slot[seeds_key.long()].long()
+        if bool((slots < 0).any()):
+            raise KeyError("a requested id is not a seed row")
+        return self._decompress(0, self.seeds_data[slots].contiguous())
+
+    def get_all_data(self, keys):
+        data = self.data[keys.long()].contiguous()
+        if self.is_fusion:
+            return data
+        return self._decompress(1 if self.is_two_level else 0, data)
+
+    def reorganize_seeds_data(self, seeds_feature, all_feature, num_dst):
+        if not self.is_fusion:
+            if seeds_feature is None:
+                return None
+            num_seeds = seeds_feature.shape[0]
+            return torch.cat([seeds_feature, all_feature[num_seeds:num_dst]], dim=0)
+        if self.is_two_level:
+            num_seeds = seeds_feature.shape[0]
+            part = all_feature[num_seeds:num_dst]
+        else:
+            part = all_feature[:num_dst]
+        part_feature = self._decompress(1 if self.is_two_level else 0, part.contiguous())
+        if self.is_two_level:
+            return torch.cat([seeds_feature, part_feature], dim=0)
+        return part_feature
+
+
+class MySAGEConv(nn.Module):
+    """examples/conv.py:9-76.  `forward(csc, feat)`: `csc = (indptr, indices)` of the block
+    (destination rows x source rows), `feat = (h_self, h_neigh)`; with a fusing manager `h_neigh`
+    is the compressed code rows of the source nodes and the aggregation decodes them on the fly."""
+
+    def __init__(self, in_feats, out_feats, aggregator_type, compression_manager, bias=True, norm=None,
+                 activation=None):
+        super().__init__()
+        if aggregator_type != "mean":
+            raise ValueError("For fusion SAGEConv, aggregator_type must be'mean'.")
+        self._in_src_feats, self._in_dst_feats = (in_feats, in_feats) if isinstance(in_feats, int) else in_feats
+        self._out_feats = out_feats
+        self.norm = norm
+        self.activation = activation
+        self.fc_neigh = nn.Linear(self._in_src_feats, out_feats, bias=False)
+        self.fc_self = nn.Linear(self._in_dst_feats, out_feats, bias=bias)
+        self.reset_parameters()
+        self.sm = compression_manager
+
+    def reset_parameters(self):
+        gain = nn.init.calculate_gain("relu")
+        nn.init.xavier_uniform_(self.fc_self.weight, gain=gain)
+        nn.init.xavier_uniform_(self.fc_neigh.weight, gain=gain)
+
+    def forward(self, csc, feat):
+        capi = _capi()
+        indptr, indices = csc
+        h_self, h_neigh = feat
+        num_dst = indptr.numel() - 1
+        if h_self is None:
+            h_self = h_neigh[:num_dst]
+        sm = self.sm
+        if sm is None or not sm.is_fusion:
+            h_neigh = capi.spmm_csr(h_neigh, indptr, indices)
+        else:
+            level = 1 if sm.is_two_level else 0
+            if sm.methods[level] == "vq":
+                h_neigh = capi.vq_decompress_spmm_csr(h_neigh, sm.codebooks[level], indptr, indices, sm.feat_dim)
+            else:
+                h_neigh = capi.sq_decompress_spmm_csr(h_neigh, sm.codebooks[level], indptr, indices,
+                                                      sm.configs[level][1], sm.configs[level][0], sm.feat_dim)
+        rst = self.fc_self(h_self) + self.fc_neigh(h_neigh)
+        if self.activation is not None:
+            rst = self.activation(rst)
+        if self.norm is not None:
+            rst = self.norm(rst)
+        return rst
