@@ -163,6 +163,13 @@ def _others(idx):
     logcb = torch.tensor([[0.01, 3.0, -6.643856, 1.5849625, 0.4]], device="cuda")
     _, ms = _time_steps(lambda: capi.sq_decompress(packed, logcb, 4, d, d), 20, 3)
     res["sq_decompress_4bit_2.4Mx100"] = {"launch_us": ms * 1e3, "GBps": n * d * 4.5 / (ms * 1e-3) / 1e9}
+    # encode to storage: one pass against the callers' three (sq_compress -> cast -> packbits)
+    xf = torch.randn((n, d), device="cuda")
+    _, ms = _time_steps(lambda: capi.sq_encode(xf, logcb, 4, d), 20, 3)
+    res["sq_encode_4bit_2.4Mx100"] = {"launch_us": ms * 1e3, "GBps": n * d * 4.5 / (ms * 1e-3) / 1e9}
+    _, ms = _time_steps(lambda: capi.packbits(capi.sq_compress(xf, logcb, 4, d).to(torch.uint8), 4), 10, 2)
+    res["sq_compress_cast_packbits_4bit_2.4Mx100"] = {"launch_us": ms * 1e3}
+    del xf
     cb = torch.randn((16, 256, 8), device="cuda")
     vq = torch.randint(0, 256, (n, 16), dtype=torch.uint8, device="cuda")
     _, ms = _time_steps(lambda: capi.vq_decompress(vq, cb, 128), 20, 3)

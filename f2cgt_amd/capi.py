@@ -24,6 +24,7 @@ SIGNATURES = {
     "f2cgt_packbits": ([P, P, L, L, I, P], c_int),
     "f2cgt_unpackbits": ([P, P, L, L, L, I, P], c_int),
     "f2cgt_sq_compress": ([P, P, P, L, L, L, I, L, P], c_int),
+    "f2cgt_sq_encode": ([P, P, P, L, L, L, I, L, P], c_int),
     "f2cgt_sq_decompress": ([P, I, P, P, L, L, L, L, I, L, P], c_int),
     "f2cgt_sq_affine_decompress": ([P, P, P, L, L, L, L, I, P], c_int),
     "f2cgt_vq_decompress": ([P, I, P, I, P, L, L, L, L, L, P], c_int),
@@ -103,6 +104,18 @@ def sq_compress(src, codebooks, bits, column_slice):
     out = torch.empty_like(src)
     _check(lib().f2cgt_sq_compress(_ptr(src), _ptr(out), _ptr(codebooks), src.shape[0], src.shape[1],
                                    codebooks.shape[0], bits, column_slice, _stream()), "sq_compress")
+    return out
+
+
+def sq_encode(src, codebooks, bits, column_slice):
+    import torch
+    rows, d = src.shape
+    if bits < 8:
+        out = torch.empty((rows, (d * bits + 7) // 8), dtype=torch.uint8, device=src.device)
+    else:
+        out = torch.empty((rows, d), dtype=torch.int8 if bits == 8 else torch.int16, device=src.device)
+    _check(lib().f2cgt_sq_encode(_ptr(src), _ptr(out), _ptr(codebooks), rows, d, codebooks.shape[0], bits,
+                                 column_slice, _stream()), "sq_encode")
     return out
 
 

@@ -147,6 +147,24 @@ torch::Tensor sq_compress(torch::Tensor src, torch::Tensor codebooks, int64_t ta
   return out;
 }
 
+// Extension: the storage tensor in one pass (= sq_compress -> cast -> packbits of the callers).
+torch::Tensor sq_encode(torch::Tensor src, torch::Tensor codebooks, int64_t target_bits, int64_t column_slice) {
+  src = dev_contig(src, "src");
+  TORCH_CHECK(src.dim() == 2 && src.scalar_type() == torch::kFloat32, "src must be float32 [rows, feat_dim]");
+  TORCH_CHECK(target_bits == 1 || target_bits == 2 || target_bits == 4 || target_bits == 8 || target_bits == 16,
+              "target_bits must be 1, 2, 4, 8 or 16");
+  codebooks = sq_codebooks_checked(codebooks);
+  c10::DeviceGuard guard(src.device());
+  const int64_t d = src.size(1);
+  auto out = target_bits < 8
+                 ? torch::empty({src.size(0), (d * target_bits + 7) / 8}, src.options().dtype(torch::kInt8))
+                 : torch::empty({src.size(0), d}, src.options().dtype(target_bits == 8 ? torch::kInt8 : torch::kInt16));
+  check_rc(f2cgt_sq_encode(src.data_ptr<float>(), out.data_ptr(), codebooks.data_ptr<float>(), src.size(0), d,
+                           codebooks.size(0), (int)target_bits, column_slice, current_stream()),
+           "sq_encode");
+  return out;
+}
+
 torch::Tensor sq_decompress(torch::Tensor compress_data, torch::Tensor codebooks, int64_t target_bits,
                             int64_t column_slice, int64_t feat_dim) {
   compress_data = dev_contig(compress_data, "compress_data");
@@ -441,6 +459,8 @@ PYBIND11_MODULE(F2CGTLib, m) {
       .def("hybrid_decompress_spmm_csr", &hybrid_decompress_spmm_csr, py::arg("row_map"),
            py::arg("sq_codes"), py::arg("sq_params"), py::arg("vq_codes"), py::arg("vq_codebooks"),
            py::arg("indptr"), py::arg("indices"), py::arg("feat_dim"))
+      .def("sq_encode", &sq_encode, py::arg("src"), py::arg("codebooks"), py::arg("target_bits"),
+           py::arg("column_slice"))
       .def("kmeans_predict", &kmeans_predict, py::arg("x"), py::arg("centers"), py::arg("metric"))
       .def("vq_encode", &vq_encode, py::arg("x"), py::arg("centers"), py::arg("metric"));
   py::class_<KMeans>(m, "KMeans")

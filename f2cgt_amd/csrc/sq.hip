@@ -18,6 +18,55 @@ int grid_for(int64_t items, int per_cu) {
 }
 
 // ---- encode -------------------------------------------------------------------
+// Code of one element as the float the encoder returns (see sq_compress_kernel).
+template <int BITS>
+__device__ __forceinline__ float sq_code_of(float x, const float* __restrict__ cb) {
+  if (BITS == 1) return x <= 0.f ? 0.f : 1.f;
+  const float drange = (float)(1 << (BITS - 1));
+  const float fmin = cb[0], fmax = cb[1], emin = cb[2], emax = cb[3];
+  const bool neg = x <= 0.f;
+  float v = fabsf(x);
+  v = fminf(fmaxf(v, fmin), fmax);
+  v = log2_cr(v);
+  v = __fmul_rn(__fdiv_rn(__fsub_rn(v, emin), __fsub_rn(emax, emin)), drange);
+  v = floorf(v);
+  v = neg ? -1.f - v : v;
+  if (BITS < 8) v += drange;
+  return v;
+}
+
+// Encode straight to the storage form: what `packbits(uint8(sq_compress(x)))` (bits < 8),
+// `int8(sq_compress(x))` or `int16(sq_compress(x))` give, in one pass over the fp32 input.  One
+// lane per stored element (a packed byte covers 8 / bits columns).
+template <int BITS, typename OT>
+__global__ __launch_bounds__(kBlock) void sq_encode_kernel(const float* __restrict__ src, OT* __restrict__ dst,
+                                                           const float* __restrict__ codebooks, int64_t rows,
+                                                           int64_t D, int64_t dst_dim, int64_t column_slice,
+                                                           int64_t num_codebooks) {
+  constexpr int PER = BITS < 8 ? 8 / BITS : 1;
+  const int64_t n = rows * dst_dim;
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+    const int64_t r = i / dst_dim;
+    const int64_t j = i - r * dst_dim;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int64_t col = j * PER + k;
+      if (col < D) {
+        int64_t cb = col / column_slice;
+        cb = cb < num_codebooks ? cb : num_codebooks - 1;
+        const float c = sq_code_of<BITS>(src[r * D + col], codebooks + cb * 5);
+        if (BITS < 8)
+          packed |= ((uint32_t)(int)c & ((1u << BITS) - 1u)) << (BITS * k);
+        else
+          packed = (uint32_t)(int)c;
+      }
+    }
+    dst[i] = (OT)packed;
+  }
+}
+
 template <int BITS>
 __global__ __launch_bounds__(kBlock) void sq_compress_kernel(const float* __restrict__ src,
                                                              float* __restrict__ dst,
@@ -321,6 +370,36 @@ extern "C" int f2cgt_sq_compress(const float* src, float* dst, const float* code
   }
 #undef F2CGT_CASE
   return launch_status("sq_compress");
+}
+
+extern "C" int f2cgt_sq_encode(const float* src, void* dst, const float* codebooks, int64_t rows,
+                               int64_t feat_dim, int64_t num_codebooks, int target_bits,
+                               int64_t column_slice, void* stream) {
+  F2CGT_REQUIRE(rows >= 0 && feat_dim >= 0, F2CGT_E_INVALID, "sq_encode: negative size");
+  F2CGT_REQUIRE(column_slice > 0 && num_codebooks > 0, F2CGT_E_INVALID,
+                "sq_encode: column_slice and num_codebooks must be positive");
+  F2CGT_REQUIRE(num_codebooks * column_slice >= feat_dim, F2CGT_E_INVALID,
+                "sq_encode: %lld codebooks of %lld columns do not cover feat_dim %lld",
+                (long long)num_codebooks, (long long)column_slice, (long long)feat_dim);
+  F2CGT_REQUIRE(target_bits == 1 || target_bits == 2 || target_bits == 4 || target_bits == 8 || target_bits == 16,
+                F2CGT_E_UNSUPPORTED, "sq_encode: target_bits must be 1,2,4,8 or 16 (got %d)", target_bits);
+  const int64_t dst_dim = target_bits < 8 ? ceil_div(feat_dim * target_bits, 8) : feat_dim;
+  const int64_t n = rows * dst_dim;
+  if (n == 0) return 0;
+  F2CGT_REQUIRE(src && dst && codebooks, F2CGT_E_INVALID, "sq_encode: null buffer");
+  hipStream_t st = as_stream(stream);
+  const int grid = grid_for(n, 16);
+#define F2CGT_CASE(B, T)                                                                              \
+  case B:                                                                                             \
+    sq_encode_kernel<B, T><<<grid, kBlock, 0, st>>>(src, static_cast<T*>(dst), codebooks, rows,      \
+                                                    feat_dim, dst_dim, column_slice, num_codebooks);  \
+    break;
+  switch (target_bits) {
+    F2CGT_CASE(1, uint8_t) F2CGT_CASE(2, uint8_t) F2CGT_CASE(4, uint8_t) F2CGT_CASE(8, int8_t)
+    default: F2CGT_CASE(16, int16_t)
+  }
+#undef F2CGT_CASE
+  return launch_status("sq_encode");
 }
 
 extern "C" int f2cgt_sq_decompress(const void* codes, int code_dtype, float* out,

@@ -87,14 +87,8 @@ def sq_compress(features, target_bits, column_slice, hotness=None, sample_index=
     for start in range(0, num_items, batch_rows):
         end = min(start + batch_rows, num_items)
         data = features[start:end].cuda().to(torch.float32)
-        codes = capi.sq_compress(data, codebooks, target_bits, column_slice)
-        if target_bits < 8:
-            exp = capi.packbits(codes.to(torch.uint8), target_bits).view(torch.int8)
-        elif target_bits == 8:
-            exp = codes.to(torch.int8)
-        else:
-            exp = codes.to(torch.int16)
-        out[start:end].copy_(exp)
+        # one pass; the reference calls sq_compress, casts and packs (process_compress.py:128-139)
+        out[start:end].copy_(capi.sq_encode(data, codebooks, target_bits, column_slice))
     return out, codebooks
 
 

@@ -79,6 +79,15 @@ int f2cgt_sq_compress(const float* src, float* dst, const float* codebooks, int6
                       int64_t feat_dim, int64_t num_codebooks, int target_bits,
                       int64_t column_slice, void* stream);
 
+/* One-pass form of the three calls every caller of sq_compress() makes next
+ * (examples/process_compress.py:128-139: sq_compress -> cast -> packbits): writes the storage
+ * tensor directly.  dst: uint8 [rows, ceil(feat_dim * bits / 8)] packed low bits first for
+ * bits in {1,2,4}; int8 [rows, feat_dim] for 8; int16 [rows, feat_dim] for 16.  Bit for bit what
+ * f2cgt_sq_compress + integer cast + f2cgt_packbits give. */
+int f2cgt_sq_encode(const float* src, void* dst, const float* codebooks, int64_t rows,
+                    int64_t feat_dim, int64_t num_codebooks, int target_bits, int64_t column_slice,
+                    void* stream);
+
 /* Replaces sq_decompress(), src/sq_quantization.cu:158-182 (kernel :85-156).
  * codes [rows, src_dim] of code_dtype (U8/I8 packed bytes for bits < 8, I8/U8 for 8,
  * I16 for 16) -> out fp32 [rows, feat_dim].  Codebook per OUTPUT column. */

@@ -122,6 +122,26 @@ def test_sq_compress_decompress_bit_exact(bits):
     assert np.array_equal(dec2, oc.sq_decompress(store2, cbs, bits, 60, 110))
 
 
+@pytest.mark.parametrize("bits", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("d,cs", [(200, 200), (110, 60), (13, 5)])
+def test_sq_encode_is_compress_cast_pack(bits, d, cs):
+    rng = np.random.default_rng(bits * 100 + d)
+    x = rng.uniform(-2, 2, size=(3001, d)).astype(np.float32)
+    x[0, :4] = [0.0, -0.0, 1e-9, 5.0]
+    cbs = np.stack([oc.sq_codebook(x[:, s:s + cs]) for s in range(0, d, cs)])
+    want = oc.sq_codes_to_storage(oc.sq_compress(x, cbs, bits, cs), bits)
+    got = host(capi.sq_encode(dev(x), dev(cbs), bits, cs))
+    assert got.shape == want.shape
+    assert np.array_equal(got.view(want.dtype) if got.dtype != want.dtype else got, want)
+    # and equals the three-call sequence on the GPU
+    codes = capi.sq_compress(dev(x), dev(cbs), bits, cs)
+    if bits < 8:
+        three = host(capi.packbits(codes.to(torch.uint8), bits))
+    else:
+        three = host(codes.to(torch.int8 if bits == 8 else torch.int16))
+    assert np.array_equal(got.view(three.dtype), three)
+
+
 @pytest.mark.parametrize("bits", [2, 4, 8, 16])
 def test_sq_decompress_every_code(bits):
     n = 1 << bits
