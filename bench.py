@@ -31,11 +31,11 @@ MFMA_F32_PEAK_TFLOPS = 157.3
 # what the same counter reads for a plain copy of known size; see profiles/).  Keyed by
 # (workload name, index dtype).  Missing = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1_sq8_affine", "int64"): 18288711,
-    ("c2_sq4_affine", "int64"): 134118977,
-    ("c3_vq_16x8", "int64"): 487330582,
-    ("c4_hybrid", "int64"): 1003957758,
-    ("c5_vq_24x32", "int64"): 2120850184,
+    ("c1_sq8_affine", "int64"): 18276432,
+    ("c2_sq4_affine", "int64"): 134094849,
+    ("c3_vq_16x8", "int64"): 487226838,
+    ("c4_hybrid", "int64"): 1004033889,
+    ("c5_vq_24x32", "int64"): 2120840107,
 }
 
 
