@@ -613,7 +613,9 @@ __global__ __launch_bounds__(kRowsBlock) void sq_rows_kernel(RowsArgs a, const I
   float* s_lut = reinterpret_cast<float*>(smem);
   const int lut_floats = AFFINE ? 0 : ((a.num_codebooks * NCODE + 3) & ~3);
   int* s_ptr = reinterpret_cast<int*>(s_lut + lut_floats);                       // [RB + 1] (+3 pad)
-  uint32_t* s_ids = reinterpret_cast<uint32_t*>(s_ptr + a.rows_per_block + 4);   // [edge_cap]
+  int* s_cnt = s_ptr + a.rows_per_block + 4;                                     // [16] rows per degree class
+  int* s_order = s_cnt + 16;                                                     // [RB] rows, heaviest first
+  uint32_t* s_ids = reinterpret_cast<uint32_t*>(s_order + a.rows_per_block);     // [edge_cap]
   unsigned char* s_codes = reinterpret_cast<unsigned char*>(s_ids + a.edge_cap); // [edge_cap][pitch]
 
   const int t = threadIdx.x;
@@ -626,6 +628,7 @@ __global__ __launch_bounds__(kRowsBlock) void sq_rows_kernel(RowsArgs a, const I
     v = v < e0 ? e0 : (v > a.E ? a.E : v);
     s_ptr[i] = (int)(v - e0 > 0x7fffffff ? 0x7fffffff : v - e0);
   }
+  if (t < 16) s_cnt[t] = 0;
   if (!AFFINE) {
     for (int i = t; i < a.num_codebooks * NCODE; i += TB) {
       const float* cb = a.table + (int64_t)(i >> BITS) * 5;
@@ -645,9 +648,33 @@ __global__ __launch_bounds__(kRowsBlock) void sq_rows_kernel(RowsArgs a, const I
   const int ne = s_ptr[nrows];
   const bool staged = ne <= a.edge_cap;
 
-  if (staged) {
+  // Rows are visited heaviest first (counting sort on min(degree, 15)), so the lanes of a wave,
+  // which each walk one row's edges, loop about equally long instead of all waiting for the
+  // longest row of an arbitrary group.
+  int my_class[(kRowsBlock + 63) / 64], my_rank[(kRowsBlock + 63) / 64];
+#pragma unroll
+  for (int k = 0; k < (kRowsBlock + 63) / 64; ++k) {
+    const int r = t + k * TB;
+    my_class[k] = my_rank[k] = 0;
+    if (r < nrows) {
+      const int d = s_ptr[r + 1] - s_ptr[r];
+      my_class[k] = d < 0 ? 0 : (d > 15 ? 15 : d);
+      my_rank[k] = atomicAdd(&s_cnt[my_class[k]], 1);
+    }
+  }
+  if (staged)
     for (int i = t; i < ne; i += TB) s_ids[i] = (uint32_t)clamp_idx(indices[e0 + i], a.N);
-    __syncthreads();
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < (kRowsBlock + 63) / 64; ++k) {
+    const int r = t + k * TB;
+    if (r < nrows) {
+      int before = 0;
+      for (int c = 15; c > my_class[k]; --c) before += s_cnt[c];
+      s_order[before + my_rank[k]] = r;
+    }
+  }
+  if (staged) {
     // gather: lane j of a group stages row bytes [8j, 8j+8) of its edge (see acc_gather)
     const int j = t & ((1 << a.lane_shift) - 1);
     const int gslot = t >> a.lane_shift;
@@ -674,8 +701,8 @@ __global__ __launch_bounds__(kRowsBlock) void sq_rows_kernel(RowsArgs a, const I
       }
       if (keep == 0x9e3779b9u && a.eff_bytes < 0) s_ids[0] = keep;  // never true; gives `keep` a use
     }
-    __syncthreads();
   }
+  __syncthreads();
 
   // decode + sum: a lane keeps one float4 column group and walks the rows
   const int g = (int)(((uint32_t)t * a.fin_magic) >> 16);
@@ -704,7 +731,8 @@ __global__ __launch_bounds__(kRowsBlock) void sq_rows_kernel(RowsArgs a, const I
     const unsigned char* sp = s_codes + boff;
     const uint8_t* gp = a.codes + boff;
     float* o = out + (row0 * (int64_t)a.feat_dim + c4 * 4);
-    for (int r = g; r < nrows; r += a.fin_slots) {
+    for (int ri = g; ri < nrows; ri += a.fin_slots) {
+      const int r = s_order[ri];
       const int b = s_ptr[r], e = s_ptr[r + 1];
       float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
       // two edges per trip (the second clamped to the first and masked at a row's odd end): the
@@ -783,7 +811,8 @@ int launch_sq_rows(RowsArgs a, const void* indptr, const void* indices, int idx_
   int rb = ((int)(0.6 * a.edge_cap / dg) + 4) / 8 * 8;
   rb = rb < 8 ? 8 : (rb > 64 ? 64 : rb);
   a.rows_per_block = rb;
-  const size_t lds = lut_bytes + (size_t)(rb + 4) * 4 + (size_t)a.edge_cap * 4 + (size_t)a.edge_cap * a.pitch + 16;
+  const size_t lds = lut_bytes + (size_t)(rb + 4) * 4 + 64 + (size_t)rb * 4 + (size_t)a.edge_cap * 4 +
+                     (size_t)a.edge_cap * a.pitch + 16;
   const int64_t grid = ceil_div(a.R, rb);
   if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
   if (idx_dtype == F2CGT_DT_I32)
@@ -1032,7 +1061,8 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
 
 bool sq_block_eligible(const void* codes, const float* out, int64_t N, int64_t src_dim, int feat_dim,
                        int target_bits, int64_t lut_entries) {
-  if (target_bits <= 2 && target_bits >= 1 && feat_dim % 4 == 0 && (int64_t)feat_dim * target_bits >= 64 &&
+  if ((target_bits == 1 || target_bits == 2 || target_bits == 4 || target_bits == 8) && feat_dim % 4 == 0 &&
+      (int64_t)feat_dim * target_bits >= 64 &&
       src_dim >= 8 && feat_dim <= 4096 && aligned(out, 16) && N < (1ll << 32) && src_dim < (1ll << 24) &&
       src_dim * (8 / target_bits) >= feat_dim && lut_entries * 4 <= 16 * 1024)
     return true;  // staged-rows kernel (any row pitch, float4 column groups)
@@ -1057,9 +1087,9 @@ int sq_block_run(bool affine, const uint8_t* codes, const float* table, int64_t 
                  int64_t column_slice, int num_codebooks, const void* indptr, const void* indices,
                  int idx_dtype, float* out, int64_t R, int64_t E, int64_t N, int64_t src_dim, int feat_dim,
                  int target_bits, hipStream_t st, const char* what) {
-  // measured at the 2.4 M-row / 250 k-destination workload: the 128-thread staged-rows kernel wins at 1 and 2
-  // bits (33 vs 40 us), the 256-thread block kernel below at 4 and 8 bits (43 vs 43-50 us)
-  if (target_bits <= 2 && feat_dim % 4 == 0 && (int64_t)feat_dim * target_bits >= 64 && src_dim >= 8 && feat_dim <= 4096 &&
+  // the 128-thread staged-rows kernel (degree-ordered rows) covers every shape with float4 column
+  // groups; the 256-thread block kernel below stays for the remaining ones
+  if (feat_dim % 4 == 0 && (int64_t)feat_dim * target_bits >= 64 && src_dim >= 8 && feat_dim <= 4096 &&
       ((feat_dim * target_bits + 63) / 64) * 8 + 4 <= 2048) {
     RowsArgs r{};
     r.codes = codes; r.table = table; r.param_stride = param_stride; r.column_slice = column_slice;
