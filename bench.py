@@ -240,10 +240,11 @@ def main():
         cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
         torch.set_num_threads(cores)
         host = {k: (v.cpu() if torch.is_tensor(v) else v) for k, v in wl.items()}
-        rows = min(wl["R"], 100_000)
+        rows = min(wl["R"], 250_000)
         _, secs, relabel_secs = cp.run(host, rows)        # warm-up, also sizes the sample
         edges = int(host["indptr"][rows])
-        reps = max(1, min(5, int(args.cpu_seconds / max(secs + relabel_secs, 1e-3))))
+        # repeat the sample until the budget (default 15 s of CPU work) is used, at least 3 times
+        reps = max(3, min(500, int(args.cpu_seconds / max(secs + relabel_secs, 1e-3))))
         times = sorted(cp.run(host, rows)[1] for _ in range(reps))
         med = times[len(times) // 2]
         result["cpu_baseline"] = {
