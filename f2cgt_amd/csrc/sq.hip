@@ -18,7 +18,27 @@ int grid_for(int64_t items, int per_cu) {
 }
 
 // ---- encode -------------------------------------------------------------------
-// Code of one element as the float the encoder returns (see sq_compress_kernel).
+// Bucket floor(g(L)) of a clamped magnitude v, L = correctly rounded fp32 log2(v).
+template <int BITS>
+__device__ __forceinline__ float sq_bucket_exact(float v, float emin, float span) {
+  const float drange = (float)(1 << (BITS - 1));
+  return floorf(__fmul_rn(__fdiv_rn(__fsub_rn(log2_cr(v), emin), span), drange));
+}
+
+// Same value, cheaper: g is non-decreasing and the hardware log2 is within a few ulp of L, so
+// when g gives one bucket a margin below and above the approximation that bucket is exact; only
+// values next to a bucket edge take the fp64 logarithm.  v must be a normal number.
+template <int BITS>
+__device__ __forceinline__ float sq_bucket_fast(float v, float emin, float span) {
+  const float drange = (float)(1 << (BITS - 1));
+  const float approx = __builtin_amdgcn_logf(v);
+  const float margin = fabsf(approx) * 1.0e-6f + 1.0e-37f;   // > 8 ulp
+  const float b_lo = floorf(__fmul_rn(__fdiv_rn(__fsub_rn(approx - margin, emin), span), drange));
+  const float b_hi = floorf(__fmul_rn(__fdiv_rn(__fsub_rn(approx + margin, emin), span), drange));
+  return b_lo == b_hi ? b_lo : sq_bucket_exact<BITS>(v, emin, span);
+}
+
+// Code of one element as the float the encoder returns (src/sq_quantization.cu:33-60).
 template <int BITS>
 __device__ __forceinline__ float sq_code_of(float x, const float* __restrict__ cb) {
   if (BITS == 1) return x <= 0.f ? 0.f : 1.f;
@@ -27,9 +47,7 @@ __device__ __forceinline__ float sq_code_of(float x, const float* __restrict__ c
   const bool neg = x <= 0.f;
   float v = fabsf(x);
   v = fminf(fmaxf(v, fmin), fmax);
-  v = log2_cr(v);
-  v = __fmul_rn(__fdiv_rn(__fsub_rn(v, emin), __fsub_rn(emax, emin)), drange);
-  v = floorf(v);
+  v = sq_bucket_exact<BITS>(v, emin, __fsub_rn(emax, emin));
   v = neg ? -1.f - v : v;
   if (BITS < 8) v += drange;
   return v;
@@ -74,30 +92,12 @@ __global__ __launch_bounds__(kBlock) void sq_compress_kernel(const float* __rest
                                                              int64_t n, int64_t D,
                                                              int64_t column_slice,
                                                              int64_t num_codebooks) {
-  const float drange = (float)(1 << (BITS - 1));
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
-    const float x = src[i];
-    if (BITS == 1) {
-      dst[i] = x <= 0.f ? 0.f : 1.f;
-      continue;
-    }
     const int64_t col = i % D;
     int64_t cb = col / column_slice;
     cb = cb < num_codebooks ? cb : num_codebooks - 1;
-    const float fmin = codebooks[cb * 5 + 0];
-    const float fmax = codebooks[cb * 5 + 1];
-    const float emin = codebooks[cb * 5 + 2];
-    const float emax = codebooks[cb * 5 + 3];
-    const bool neg = x <= 0.f;
-    float v = fabsf(x);
-    v = fminf(fmaxf(v, fmin), fmax);
-    v = log2_cr(v);
-    v = __fmul_rn(__fdiv_rn(__fsub_rn(v, emin), __fsub_rn(emax, emin)), drange);
-    v = floorf(v);
-    v = neg ? -1.f - v : v;
-    if (BITS < 8) v += drange;
-    dst[i] = v;
+    dst[i] = sq_code_of<BITS>(src[i], codebooks + cb * 5);
   }
 }
 
@@ -315,6 +315,125 @@ int decode_f4_launch(const uint8_t* codes, float* out, const float* table, int64
   return launch_status(what);
 }
 
+// ---- float4-per-lane encoders ----------------------------------------------------------------
+// Same indexing as the float4 decoders: a lane takes four consecutive columns of a row (eight
+// for 1-bit storage, so that it owns a whole byte), the codebook of each column comes from a
+// small table in LDS, and the result goes out as one float4 (codes as fp32, the reference form)
+// or as the 1-4 bytes of the storage form.
+template <int BITS, bool STORAGE>
+__global__ __launch_bounds__(kBlock) void sq_encode_f4_kernel(F4Args a, const float* __restrict__ src,
+                                                              void* __restrict__ dst) {
+  constexpr int COLS = (STORAGE && BITS == 1) ? 8 : 4;   // columns per lane
+  extern __shared__ __align__(16) float s_tab[];
+  // per codebook: fmin, fmax, emin, span, bucket(fmin), bucket(fmax) (+2 pad); then the table
+  // offset of every column.  Values clamped to fmin / fmax (about 1 % of a table by construction
+  // of the codebooks) sit exactly on a bucket edge, so their buckets are evaluated once, exactly.
+  float* s_cb = s_tab;
+  int* s_cbi = reinterpret_cast<int*>(s_tab + a.n_cb * 8);
+  const int feat_dim = (int)a.f4_per_row * COLS;
+  for (int i = threadIdx.x; i < a.n_cb; i += kBlock) {
+    const float* cb = a.table + (int64_t)i * 5;
+    const float span = __fsub_rn(cb[3], cb[2]);
+    s_cb[i * 8 + 0] = cb[0];
+    s_cb[i * 8 + 1] = cb[1];
+    s_cb[i * 8 + 2] = cb[2];
+    s_cb[i * 8 + 3] = span;
+    s_cb[i * 8 + 4] = BITS == 1 ? 0.f : sq_bucket_exact<BITS>(fminf(fmaxf(cb[0], cb[0]), cb[1]), cb[2], span);
+    s_cb[i * 8 + 5] = BITS == 1 ? 0.f : sq_bucket_exact<BITS>(fminf(fmaxf(cb[1], cb[0]), cb[1]), cb[2], span);
+  }
+  for (int i = threadIdx.x; i < feat_dim; i += kBlock) {
+    int64_t cb = i / a.column_slice;
+    cb = cb < a.n_cb ? cb : a.n_cb - 1;
+    s_cbi[i] = (int)cb * 8;
+  }
+  __syncthreads();
+  auto code_of = [&](float xv, int tab) -> float {
+    if (BITS == 1) return xv <= 0.f ? 0.f : 1.f;
+    const float drange = (float)(1 << (BITS - 1));
+    const float4 q = *reinterpret_cast<const float4*>(s_cb + tab);      // fmin, fmax, emin, span
+    const bool neg = xv <= 0.f;
+    const float m = fabsf(xv);
+    float bkt;
+    if (!(m > q.x)) bkt = s_cb[tab + 4];            // clamps to fmin (NaN goes the reference's way: fmaxf picks fmin)
+    else if (m >= q.y) bkt = s_cb[tab + 5];
+    else bkt = sq_bucket_fast<BITS>(m, q.z, q.w);
+    float v = neg ? -1.f - bkt : bkt;
+    if (BITS < 8) v += drange;
+    return v;
+  };
+  const int64_t base = (int64_t)blockIdx.x * (kF4Items * kBlock);
+  int64_t rb = (int64_t)((double)base / (double)a.f4_per_row);
+  if (rb * a.f4_per_row > base) --rb;
+  if ((rb + 1) * (int64_t)a.f4_per_row <= base) ++rb;
+  const uint32_t cb0 = (uint32_t)(base - rb * a.f4_per_row);
+  float4 x[kF4Items][COLS / 4];
+#pragma unroll
+  for (int k = 0; k < kF4Items; ++k) {
+    const int64_t i = base + threadIdx.x + k * kBlock;
+    const float4* p = reinterpret_cast<const float4*>(src) + (i < a.total_f4 ? i : 0) * (COLS / 4);
+#pragma unroll
+    for (int h = 0; h < COLS / 4; ++h) x[k][h] = p[h];
+  }
+#pragma unroll
+  for (int k = 0; k < kF4Items; ++k) {
+    const int64_t i = base + threadIdx.x + k * kBlock;
+    if (i >= a.total_f4) break;
+    const uint32_t li = cb0 + threadIdx.x + k * kBlock;
+    const uint32_t rl = __umulhi(li, a.magic);
+    const uint32_t g = li - rl * a.f4_per_row;            // column group of the row
+    float c[COLS];
+#pragma unroll
+    for (int h = 0; h < COLS / 4; ++h) {
+      const int4 cbi = *reinterpret_cast<const int4*>(s_cbi + g * COLS + 4 * h);
+      c[4 * h + 0] = code_of(x[k][h].x, cbi.x);
+      c[4 * h + 1] = code_of(x[k][h].y, cbi.y);
+      c[4 * h + 2] = code_of(x[k][h].z, cbi.z);
+      c[4 * h + 3] = code_of(x[k][h].w, cbi.w);
+    }
+    if (!STORAGE) {
+      store_nt4(static_cast<float*>(dst) + i * 4, c[0], c[1], c[2], c[3]);
+    } else if (BITS == 16) {
+      typedef short s4 __attribute__((ext_vector_type(4)));
+      s4 v = {(short)(int)c[0], (short)(int)c[1], (short)(int)c[2], (short)(int)c[3]};
+      __builtin_nontemporal_store(v, static_cast<s4*>(dst) + i);
+    } else {
+      uint32_t packed = 0;
+      constexpr int FIELD = BITS;                          // 8-bit codes: one byte each
+#pragma unroll
+      for (int q = 0; q < COLS; ++q) packed |= ((uint32_t)(int)c[q] & ((1u << FIELD) - 1u)) << (FIELD * q);
+      // storage bytes of the lane: COLS * BITS / 8, at the same offset in every row pitch
+      uint8_t* o = static_cast<uint8_t*>(dst) + (rb + rl) * a.src_dim + (int64_t)g * (COLS * BITS / 8);
+      if (COLS * BITS == 32) { __builtin_memcpy(o, &packed, 4); }
+      else if (COLS * BITS == 16) { const uint16_t h2 = (uint16_t)packed; __builtin_memcpy(o, &h2, 2); }
+      else *o = (uint8_t)packed;
+    }
+  }
+}
+
+// Launches the float4 encoder when the shape allows it; returns -1 when it does not.
+template <int BITS, bool STORAGE>
+int encode_f4_launch(const float* src, void* dst, const float* codebooks, int64_t column_slice, int n_cb,
+                     int64_t rows, int64_t feat_dim, int64_t dst_dim, hipStream_t st, const char* what) {
+  constexpr int COLS = (STORAGE && BITS == 1) ? 8 : 4;
+  if (feat_dim % COLS != 0 || feat_dim > 8192 || !aligned(src, 16) || (!STORAGE && !aligned(dst, 16)) ||
+      (STORAGE && BITS == 16 && !aligned(dst, 8)))
+    return -1;
+  F4Args a{};
+  a.table = codebooks;
+  a.column_slice = column_slice;
+  a.n_cb = n_cb;
+  a.src_dim = dst_dim;                       // bytes per storage row
+  a.f4_per_row = (uint32_t)(feat_dim / COLS);
+  a.total_f4 = rows * (feat_dim / COLS);
+  a.magic = (uint32_t)((0x100000000ull + a.f4_per_row - 1) / a.f4_per_row);
+  const int64_t grid = ceil_div(a.total_f4, kF4Items * kBlock);
+  if (grid > 0x7fffffffll) return -1;
+  const size_t lds = ((size_t)n_cb * 8 + (size_t)feat_dim) * 4;
+  if (lds > (size_t)kMaxLutBytes) return -1;
+  sq_encode_f4_kernel<BITS, STORAGE><<<(unsigned)grid, kBlock, lds, st>>>(a, src, dst);
+  return launch_status(what);
+}
+
 template <int BITS>
 int decompress_lut_launch(const uint8_t* codes, float* out, const float* codebooks, int64_t rows,
                           int64_t src_dim, int64_t feat_dim, int64_t column_slice, int n_cb,
@@ -356,6 +475,19 @@ extern "C" int f2cgt_sq_compress(const float* src, float* dst, const float* code
   if (n == 0) return 0;
   F2CGT_REQUIRE(src && dst && codebooks, F2CGT_E_INVALID, "sq_compress: null buffer");
   hipStream_t st = as_stream(stream);
+  {
+    int rc = -1;
+    const int ncb = (int)num_codebooks;
+    switch (target_bits) {
+      case 1: rc = encode_f4_launch<1, false>(src, dst, codebooks, column_slice, ncb, rows, feat_dim, 0, st, "sq_compress"); break;
+      case 2: rc = encode_f4_launch<2, false>(src, dst, codebooks, column_slice, ncb, rows, feat_dim, 0, st, "sq_compress"); break;
+      case 4: rc = encode_f4_launch<4, false>(src, dst, codebooks, column_slice, ncb, rows, feat_dim, 0, st, "sq_compress"); break;
+      case 8: rc = encode_f4_launch<8, false>(src, dst, codebooks, column_slice, ncb, rows, feat_dim, 0, st, "sq_compress"); break;
+      case 16: rc = encode_f4_launch<16, false>(src, dst, codebooks, column_slice, ncb, rows, feat_dim, 0, st, "sq_compress"); break;
+      default: break;
+    }
+    if (rc >= 0) return rc;
+  }
   const int grid = grid_for(n, 16);
 #define F2CGT_CASE(B)                                                                       \
   case B:                                                                                   \
@@ -388,6 +520,18 @@ extern "C" int f2cgt_sq_encode(const float* src, void* dst, const float* codeboo
   if (n == 0) return 0;
   F2CGT_REQUIRE(src && dst && codebooks, F2CGT_E_INVALID, "sq_encode: null buffer");
   hipStream_t st = as_stream(stream);
+  if (num_codebooks < (1 << 20)) {
+    int rc = -1;
+    const int ncb = (int)num_codebooks;
+    switch (target_bits) {
+      case 1: rc = encode_f4_launch<1, true>(src, dst, codebooks, column_slice, ncb, rows, feat_dim, dst_dim, st, "sq_encode"); break;
+      case 2: rc = encode_f4_launch<2, true>(src, dst, codebooks, column_slice, ncb, rows, feat_dim, dst_dim, st, "sq_encode"); break;
+      case 4: rc = encode_f4_launch<4, true>(src, dst, codebooks, column_slice, ncb, rows, feat_dim, dst_dim, st, "sq_encode"); break;
+      case 8: rc = encode_f4_launch<8, true>(src, dst, codebooks, column_slice, ncb, rows, feat_dim, dst_dim * 1, st, "sq_encode"); break;
+      default: rc = encode_f4_launch<16, true>(src, dst, codebooks, column_slice, ncb, rows, feat_dim, dst_dim * 2, st, "sq_encode"); break;
+    }
+    if (rc >= 0) return rc;
+  }
   const int grid = grid_for(n, 16);
 #define F2CGT_CASE(B, T)                                                                              \
   case B:                                                                                             \
