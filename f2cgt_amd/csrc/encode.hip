@@ -76,10 +76,15 @@ __device__ int exact_argmin_row_l2_lds(const float* __restrict__ xrow, const flo
   double bestv = DBL_MAX;
   int besti = INT_MAX;
   for (int c = lane; c < n; c += kWave) {
+    // dimension h * khalf + t of centre c sits 128 * t + 64 * h floats after its step-1 slot
+    const float* cp = cT + a_index(c, 1, 0, KH);
     double d = 0.0;
-    for (int dim = 0; dim < k; ++dim) {
-      const int hh = dim >= khalf ? 1 : 0;
-      const double df = (double)xrow[dim] - (double)cT[a_index(c, 1 + dim - hh * khalf, hh, KH)];
+    for (int t = 0; t < khalf; ++t) {
+      const double df = (double)xrow[t] - (double)cp[128 * t];
+      d += df * df;
+    }
+    for (int t = 0; khalf + t < k; ++t) {
+      const double df = (double)xrow[khalf + t] - (double)cp[128 * t + 64];
       d += df * df;
     }
     if (d < bestv) { bestv = d; besti = c; }
