@@ -26,15 +26,21 @@ __device__ __forceinline__ float sq_bucket_exact(float v, float emin, float span
 }
 
 // Same value, cheaper: g is non-decreasing and the hardware log2 is within a few ulp of L, so
-// when g gives one bucket a margin below and above the approximation that bucket is exact; only
-// values next to a bucket edge take the fp64 logarithm.  v must be a normal number.
+// when an error bound below and above the approximate g lands in one bucket that bucket is exact;
+// only values next to a bucket edge take the fp64 logarithm.  v must be a normal number.
 template <int BITS>
-__device__ __forceinline__ float sq_bucket_fast(float v, float emin, float span) {
-  const float drange = (float)(1 << (BITS - 1));
+__device__ __forceinline__ float sq_bucket_fast(float v, float emin, float span, float k) {
+  // k = fl(2^(BITS-1) / span).  With L the fp32 logarithm the exact chain starts from, that chain
+  // gives u = (L - emin) / span * 2^(BITS-1) with two roundings (the power of two is exact); the
+  // product t below is the same expression at the hardware logarithm with three.  So
+  // |u - t| <= |L - approx| * k + 6 * 2^-24 * |t|, and `mt` bounds that with room to spare for
+  // its own roundings; floor is monotone, so equal floors at t - mt and t + mt fix the bucket.
   const float approx = __builtin_amdgcn_logf(v);
-  const float margin = fabsf(approx) * 1.0e-6f + 1.0e-37f;   // > 8 ulp
-  const float b_lo = floorf(__fmul_rn(__fdiv_rn(__fsub_rn(approx - margin, emin), span), drange));
-  const float b_hi = floorf(__fmul_rn(__fdiv_rn(__fsub_rn(approx + margin, emin), span), drange));
+  const float m_log = fmaf(fabsf(approx), 1.0e-6f, 2.0e-7f);   // > 8 ulp, and 2^-22 absolute next to log = 0
+  const float t = __fmul_rn(__fsub_rn(approx, emin), k);
+  const float mt = fmaf(fabsf(t), 1.0e-6f, m_log * k * 1.001f);
+  const float b_lo = floorf(t - mt);
+  const float b_hi = floorf(t + mt);
   return b_lo == b_hi ? b_lo : sq_bucket_exact<BITS>(v, emin, span);
 }
 
@@ -325,7 +331,7 @@ __global__ __launch_bounds__(kBlock) void sq_encode_f4_kernel(F4Args a, const fl
                                                               void* __restrict__ dst) {
   constexpr int COLS = (STORAGE && BITS == 1) ? 8 : 4;   // columns per lane
   extern __shared__ __align__(16) float s_tab[];
-  // per codebook: fmin, fmax, emin, span, bucket(fmin), bucket(fmax) (+2 pad); then the table
+  // per codebook: fmin, fmax, emin, 2^(BITS-1)/span, span, bucket(fmin), bucket(fmax) (+1 pad); then the table
   // offset of every column.  Values clamped to fmin / fmax (about 1 % of a table by construction
   // of the codebooks) sit exactly on a bucket edge, so their buckets are evaluated once, exactly.
   float* s_cb = s_tab;
@@ -337,9 +343,10 @@ __global__ __launch_bounds__(kBlock) void sq_encode_f4_kernel(F4Args a, const fl
     s_cb[i * 8 + 0] = cb[0];
     s_cb[i * 8 + 1] = cb[1];
     s_cb[i * 8 + 2] = cb[2];
-    s_cb[i * 8 + 3] = span;
-    s_cb[i * 8 + 4] = BITS == 1 ? 0.f : sq_bucket_exact<BITS>(fminf(fmaxf(cb[0], cb[0]), cb[1]), cb[2], span);
-    s_cb[i * 8 + 5] = BITS == 1 ? 0.f : sq_bucket_exact<BITS>(fminf(fmaxf(cb[1], cb[0]), cb[1]), cb[2], span);
+    s_cb[i * 8 + 3] = __fdiv_rn((float)(1 << (BITS - 1)), span);
+    s_cb[i * 8 + 4] = span;
+    s_cb[i * 8 + 5] = BITS == 1 ? 0.f : sq_bucket_exact<BITS>(fminf(fmaxf(cb[0], cb[0]), cb[1]), cb[2], span);
+    s_cb[i * 8 + 6] = BITS == 1 ? 0.f : sq_bucket_exact<BITS>(fminf(fmaxf(cb[1], cb[0]), cb[1]), cb[2], span);
   }
   for (int i = threadIdx.x; i < feat_dim; i += kBlock) {
     int64_t cb = i / a.column_slice;
@@ -350,13 +357,13 @@ __global__ __launch_bounds__(kBlock) void sq_encode_f4_kernel(F4Args a, const fl
   auto code_of = [&](float xv, int tab) -> float {
     if (BITS == 1) return xv <= 0.f ? 0.f : 1.f;
     const float drange = (float)(1 << (BITS - 1));
-    const float4 q = *reinterpret_cast<const float4*>(s_cb + tab);      // fmin, fmax, emin, span
+    const float4 q = *reinterpret_cast<const float4*>(s_cb + tab);      // fmin, fmax, emin, 2^(BITS-1)/span
     const bool neg = xv <= 0.f;
     const float m = fabsf(xv);
     float bkt;
-    if (!(m > q.x)) bkt = s_cb[tab + 4];            // clamps to fmin (NaN goes the reference's way: fmaxf picks fmin)
-    else if (m >= q.y) bkt = s_cb[tab + 5];
-    else bkt = sq_bucket_fast<BITS>(m, q.z, q.w);
+    if (!(m > q.x)) bkt = s_cb[tab + 5];            // clamps to fmin (NaN goes the reference's way: fmaxf picks fmin)
+    else if (m >= q.y) bkt = s_cb[tab + 6];
+    else bkt = sq_bucket_fast<BITS>(m, q.z, s_cb[tab + 4], q.w);
     float v = neg ? -1.f - bkt : bkt;
     if (BITS < 8) v += drange;
     return v;

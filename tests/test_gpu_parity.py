@@ -143,6 +143,37 @@ def test_sq_encode_is_compress_cast_pack(bits, d, cs):
 
 
 @pytest.mark.parametrize("bits", [2, 4, 8, 16])
+def test_sq_encode_values_on_bucket_edges(bits):
+    # the encoder decides most buckets from a hardware logarithm with an error bound; magnitudes
+    # placed on and next to every bucket edge, and around 1.0 where log2 changes sign, are the
+    # ones that bound has to hand to the exact path
+    rng = np.random.default_rng(bits)
+    base = rng.uniform(-3, 3, size=(4096, 64)).astype(np.float32)
+    cb = np.stack([oc.sq_codebook(base)])
+    emin, emax = float(cb[0, 2]), float(cb[0, 3])
+    n_edges = min(1 << (bits - 1), 4096)
+    j = np.linspace(0, 1 << (bits - 1), n_edges + 1)
+    edge = np.exp2(emin + j * (emax - emin) / (1 << (bits - 1))).astype(np.float32)
+    near = [edge]
+    for _ in range(4):
+        near.append(np.nextafter(near[-1], np.float32(np.inf)))
+    lo = edge
+    for _ in range(4):
+        lo = np.nextafter(lo, np.float32(0))
+        near.append(lo)
+    one = np.float32(1.0) + np.arange(-32, 33, dtype=np.float32) * np.float32(2.0 ** -24)
+    vals = np.concatenate(near + [one])
+    vals = np.concatenate([vals, -vals])
+    pad = (-len(vals)) % 64
+    x = np.concatenate([vals, np.zeros(pad, np.float32)]).reshape(-1, 64)
+    want = oc.sq_compress(x, cb, bits, 64)
+    assert np.array_equal(host(capi.sq_compress(dev(x), dev(cb), bits, 64)), want)
+    got = host(capi.sq_encode(dev(x), dev(cb), bits, 64))
+    store = oc.sq_codes_to_storage(want, bits)
+    assert np.array_equal(got.view(store.dtype), store)
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8, 16])
 def test_sq_decompress_every_code(bits):
     n = 1 << bits
     raw = np.arange(n, dtype=np.int64)
