@@ -25,23 +25,23 @@ __device__ __forceinline__ float sq_bucket_exact(float v, float emin, float span
   return floorf(__fmul_rn(__fdiv_rn(__fsub_rn(log2_cr(v), emin), span), drange));
 }
 
-// Same value, cheaper: g is non-decreasing and the hardware log2 is within a few ulp of L, so
-// when an error bound below and above the approximate g lands in one bucket that bucket is exact;
-// only values next to a bucket edge take the fp64 logarithm.  v must be a normal number.
-template <int BITS>
-__device__ __forceinline__ float sq_bucket_fast(float v, float emin, float span, float k) {
-  // k = fl(2^(BITS-1) / span).  With L the fp32 logarithm the exact chain starts from, that chain
-  // gives u = (L - emin) / span * 2^(BITS-1) with two roundings (the power of two is exact); the
-  // product t below is the same expression at the hardware logarithm with three.  So
-  // |u - t| <= |L - approx| * k + 6 * 2^-24 * |t|, and `mt` bounds that with room to spare for
-  // its own roundings; floor is monotone, so equal floors at t - mt and t + mt fix the bucket.
+// The same bucket without the fp64 logarithm, for most values: g is non-decreasing and the
+// hardware log2 is within a few ulp of L, so when an error bound below and above the approximate g
+// lands in one bucket (b_lo == b_hi) that bucket is exact; the caller sends only the values next
+// to a bucket edge to sq_bucket_exact.  v must be a normal number; k = fl(2^(BITS-1) / span).
+//
+// With L the fp32 logarithm the exact chain starts from, that chain gives
+// u = (L - emin) / span * 2^(BITS-1) with two roundings (the power of two is exact); the product t
+// below is the same expression at the hardware logarithm with three.  So
+// |u - t| <= |L - approx| * k + 6 * 2^-24 * |t|, and `mt` bounds that with room to spare for its
+// own roundings; floor is monotone, so floor(u) lies between the two floors returned.
+__device__ __forceinline__ void sq_bucket_bounds(float v, float emin, float k, float& b_lo, float& b_hi) {
   const float approx = __builtin_amdgcn_logf(v);
   const float m_log = fmaf(fabsf(approx), 1.0e-6f, 2.0e-7f);   // > 8 ulp, and 2^-22 absolute next to log = 0
   const float t = __fmul_rn(__fsub_rn(approx, emin), k);
   const float mt = fmaf(fabsf(t), 1.0e-6f, m_log * k * 1.001f);
-  const float b_lo = floorf(t - mt);
-  const float b_hi = floorf(t + mt);
-  return b_lo == b_hi ? b_lo : sq_bucket_exact<BITS>(v, emin, span);
+  b_lo = floorf(t - mt);
+  b_hi = floorf(t + mt);
 }
 
 // Code of one element as the float the encoder returns (src/sq_quantization.cu:33-60).
@@ -326,12 +326,12 @@ int decode_f4_launch(const uint8_t* codes, float* out, const float* table, int64
 // for 1-bit storage, so that it owns a whole byte), the codebook of each column comes from a
 // small table in LDS, and the result goes out as one float4 (codes as fp32, the reference form)
 // or as the 1-4 bytes of the storage form.
-template <int BITS, bool STORAGE>
+template <int BITS, bool STORAGE, bool SINGLE>
 __global__ __launch_bounds__(kBlock) void sq_encode_f4_kernel(F4Args a, const float* __restrict__ src,
                                                               void* __restrict__ dst) {
   constexpr int COLS = (STORAGE && BITS == 1) ? 8 : 4;   // columns per lane
   extern __shared__ __align__(16) float s_tab[];
-  // per codebook: fmin, fmax, emin, 2^(BITS-1)/span, span, bucket(fmin), bucket(fmax) (+1 pad); then the table
+  // per codebook: fmin, fmax, emin, 2^(BITS-1)/span, bucket(fmin), bucket(fmax), span (+1 pad); then the table
   // offset of every column.  Values clamped to fmin / fmax (about 1 % of a table by construction
   // of the codebooks) sit exactly on a bucket edge, so their buckets are evaluated once, exactly.
   float* s_cb = s_tab;
@@ -344,9 +344,9 @@ __global__ __launch_bounds__(kBlock) void sq_encode_f4_kernel(F4Args a, const fl
     s_cb[i * 8 + 1] = cb[1];
     s_cb[i * 8 + 2] = cb[2];
     s_cb[i * 8 + 3] = __fdiv_rn((float)(1 << (BITS - 1)), span);
-    s_cb[i * 8 + 4] = span;
-    s_cb[i * 8 + 5] = BITS == 1 ? 0.f : sq_bucket_exact<BITS>(fminf(fmaxf(cb[0], cb[0]), cb[1]), cb[2], span);
-    s_cb[i * 8 + 6] = BITS == 1 ? 0.f : sq_bucket_exact<BITS>(fminf(fmaxf(cb[1], cb[0]), cb[1]), cb[2], span);
+    s_cb[i * 8 + 4] = BITS == 1 ? 0.f : sq_bucket_exact<BITS>(fminf(fmaxf(cb[0], cb[0]), cb[1]), cb[2], span);
+    s_cb[i * 8 + 5] = BITS == 1 ? 0.f : sq_bucket_exact<BITS>(fminf(fmaxf(cb[1], cb[0]), cb[1]), cb[2], span);
+    s_cb[i * 8 + 6] = span;
   }
   for (int i = threadIdx.x; i < feat_dim; i += kBlock) {
     int64_t cb = i / a.column_slice;
@@ -354,19 +354,49 @@ __global__ __launch_bounds__(kBlock) void sq_encode_f4_kernel(F4Args a, const fl
     s_cbi[i] = (int)cb * 8;
   }
   __syncthreads();
-  auto code_of = [&](float xv, int tab) -> float {
-    if (BITS == 1) return xv <= 0.f ? 0.f : 1.f;
+  // Codes of four columns.  The common part runs without a branch for all four; the columns whose
+  // error bound straddles a bucket edge are collected in a mask and take the exact path in one
+  // rolled loop, so the fp64 logarithm exists once in the code, not once per column.
+  auto code4 = [&](const float4 xv, const int4 tabs, float* c) {
+    const float xs[4] = {xv.x, xv.y, xv.z, xv.w};
+    if (BITS == 1) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) c[e] = xs[e] <= 0.f ? 0.f : 1.f;
+      return;
+    }
     const float drange = (float)(1 << (BITS - 1));
-    const float4 q = *reinterpret_cast<const float4*>(s_cb + tab);      // fmin, fmax, emin, 2^(BITS-1)/span
-    const bool neg = xv <= 0.f;
-    const float m = fabsf(xv);
-    float bkt;
-    if (!(m > q.x)) bkt = s_cb[tab + 5];            // clamps to fmin (NaN goes the reference's way: fmaxf picks fmin)
-    else if (m >= q.y) bkt = s_cb[tab + 6];
-    else bkt = sq_bucket_fast<BITS>(m, q.z, s_cb[tab + 4], q.w);
-    float v = neg ? -1.f - bkt : bkt;
-    if (BITS < 8) v += drange;
-    return v;
+    const int tb[4] = {SINGLE ? 0 : tabs.x, SINGLE ? 0 : tabs.y, SINGLE ? 0 : tabs.z, SINGLE ? 0 : tabs.w};
+    float m[4], bkt[4];
+    uint32_t need = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float4 q = *reinterpret_cast<const float4*>(s_cb + tb[e]);      // fmin, fmax, emin, 2^(BITS-1)/span
+      const float2 cl = *reinterpret_cast<const float2*>(s_cb + tb[e] + 4);  // bucket(fmin), bucket(fmax)
+      m[e] = fabsf(xs[e]);
+      float b_lo, b_hi;
+      sq_bucket_bounds(m[e], q.z, q.w, b_lo, b_hi);
+      const bool at_min = !(m[e] > q.x);        // clamps to fmin (NaN too: the reference's fmaxf picks fmin)
+      const bool at_max = m[e] >= q.y;
+      bkt[e] = at_min ? cl.x : at_max ? cl.y : b_lo;
+      need |= (!at_min && !at_max && !(b_lo == b_hi)) ? 1u << e : 0u;
+    }
+    if (need) {
+#pragma nounroll
+      for (int e = 0; e < 4; ++e) {
+        if (!((need >> e) & 1u)) continue;
+        const float me = e == 0 ? m[0] : e == 1 ? m[1] : e == 2 ? m[2] : m[3];
+        const int te = e == 0 ? tb[0] : e == 1 ? tb[1] : e == 2 ? tb[2] : tb[3];
+        const float r = sq_bucket_exact<BITS>(me, s_cb[te + 2], s_cb[te + 6]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bkt[j] = e == j ? r : bkt[j];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float v = xs[e] <= 0.f ? -1.f - bkt[e] : bkt[e];
+      if (BITS < 8) v += drange;
+      c[e] = v;
+    }
   };
   const int64_t base = (int64_t)blockIdx.x * (kF4Items * kBlock);
   int64_t rb = (int64_t)((double)base / (double)a.f4_per_row);
@@ -391,11 +421,9 @@ __global__ __launch_bounds__(kBlock) void sq_encode_f4_kernel(F4Args a, const fl
     float c[COLS];
 #pragma unroll
     for (int h = 0; h < COLS / 4; ++h) {
-      const int4 cbi = *reinterpret_cast<const int4*>(s_cbi + g * COLS + 4 * h);
-      c[4 * h + 0] = code_of(x[k][h].x, cbi.x);
-      c[4 * h + 1] = code_of(x[k][h].y, cbi.y);
-      c[4 * h + 2] = code_of(x[k][h].z, cbi.z);
-      c[4 * h + 3] = code_of(x[k][h].w, cbi.w);
+      int4 cbi = {0, 0, 0, 0};
+      if (!SINGLE) cbi = *reinterpret_cast<const int4*>(s_cbi + g * COLS + 4 * h);
+      code4(x[k][h], cbi, c + 4 * h);
     }
     if (!STORAGE) {
       store_nt4(static_cast<float*>(dst) + i * 4, c[0], c[1], c[2], c[3]);
@@ -437,7 +465,8 @@ int encode_f4_launch(const float* src, void* dst, const float* codebooks, int64_
   if (grid > 0x7fffffffll) return -1;
   const size_t lds = ((size_t)n_cb * 8 + (size_t)feat_dim) * 4;
   if (lds > (size_t)kMaxLutBytes) return -1;
-  sq_encode_f4_kernel<BITS, STORAGE><<<(unsigned)grid, kBlock, lds, st>>>(a, src, dst);
+  if (n_cb == 1) sq_encode_f4_kernel<BITS, STORAGE, true><<<(unsigned)grid, kBlock, lds, st>>>(a, src, dst);
+  else sq_encode_f4_kernel<BITS, STORAGE, false><<<(unsigned)grid, kBlock, lds, st>>>(a, src, dst);
   return launch_status(what);
 }
 
