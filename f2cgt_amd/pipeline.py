@@ -2,7 +2,8 @@
 place of DGL blocks, ShmTensor and torch.distributed (one process, one GPU):
 
   * the offline encode pipeline: `sq_metadata`, `sq_compress`, `vq_metadata`, `vq_compress`
-    (examples/process_compress.py:16-68, 71-144, 147-292);
+    (examples/process_compress.py:16-68, 71-144, 147-292), `run` that writes the artefact files
+    (`:295-388`) and `load_compress_data` that reads them back (examples/load_dataset.py:63-85);
   * `CompressionManager` (examples/compress.py:8-106): keeps the code tables and codebooks,
     serves seed rows (first level) and neighbour rows (second level);
   * `MySAGEConv` (examples/conv.py:9-76): GraphSAGE mean layer whose neighbour aggregation is the
@@ -145,6 +146,71 @@ def vq_compress(features, n_clusters, column_slice, hotness=None, codebooks=None
             labels = predictors[i].predict(data, normalize_weights=False)
             out[start:end, i] = labels.to(dtype)
     return out, codebooks
+
+
+def run(root, features, seeds=None, hotness=None, target_compression_ratio=32, n_clusters=256):
+    """Compresses a feature table and writes the artefacts the training scripts load
+    (examples/process_compress.py:295-388, single process, column slices as for one rank):
+
+      * `compression_meta.pt`: dict with `methods` (['sq'] / ['vq'], preceded by 'sq' when seed
+        rows get their own table), `codebooks` (CPU tensors, one per level), `configs`
+        ((column_slice, target_bits) per level, target_bits -1 for VQ), `feat_dim`, `data`
+        (name -> (dtype, shape) of each code table) and `seeds` (ids of the seed rows);
+      * `compression_data.pt`: the code table of every row;
+      * `seeds_compression_data.pt`: the code table of the seed rows (SQ at one eighth of the
+        element width in bits, i.e. 4-bit codes for fp32 features).
+
+    A ratio up to the element width in bits selects SQ with `width / ratio` bits per value; a
+    larger one selects VQ with `ratio / element_size` columns per code byte (twice that for
+    more than 256 centres).  Returns the meta dict."""
+    import os
+    feat_dim = features.shape[1]
+    width_bits = features.element_size() * 8
+    methods, configs, codebook_list, data, meta = [], [], [], {}, {}
+    slice_of_row = (feat_dim + 7) // 8 * 8
+    if seeds is not None:
+        seed_bits = width_bits // 8
+        seed_rows = features[seeds.to(features.device)]
+        seed_codes, seed_cbs = sq_compress(seed_rows, seed_bits, slice_of_row, None)
+        methods.append("sq")
+        configs.append((slice_of_row, seed_bits))
+        codebook_list.append(seed_cbs.cpu())
+        data["seeds_compression_data"] = (seed_codes.dtype, seed_codes.shape)
+        meta["seeds"] = seeds.cpu()
+        torch.save(seed_codes.cpu(), os.path.join(root, "seeds_compression_data.pt"))
+        del seed_codes
+    if target_compression_ratio <= width_bits:
+        target_bits = int(width_bits / target_compression_ratio)
+        codes, cbs = sq_compress(features, target_bits, slice_of_row, hotness)
+        methods.append("sq")
+        configs.append((slice_of_row, target_bits))
+    else:
+        column_slice = target_compression_ratio // features.element_size()
+        if n_clusters > 256:
+            column_slice *= 2
+        codes, cbs = vq_compress(features, n_clusters, column_slice, hotness)
+        methods.append("vq")
+        configs.append((column_slice, -1))
+    codebook_list.append(cbs.cpu())
+    data["compression_data"] = (codes.dtype, codes.shape)
+    meta.update(methods=methods, codebooks=codebook_list, configs=configs, feat_dim=feat_dim, data=data)
+    torch.save(meta, os.path.join(root, "compression_meta.pt"))
+    torch.save(codes.cpu(), os.path.join(root, "compression_data.pt"))
+    return meta
+
+
+def load_compress_data(root):
+    """The dict `CompressionManager` takes, read back from the files `run` wrote: the meta dict
+    with every code table named in `data` added under its name
+    (examples/load_dataset.py:63-85 without the shared-memory staging)."""
+    import os
+    meta = torch.load(os.path.join(root, "compression_meta.pt"), weights_only=True)
+    for name, (dtype, shape) in meta["data"].items():
+        table = torch.load(os.path.join(root, name + ".pt"), weights_only=True)
+        if table.dtype != dtype or tuple(table.shape) != tuple(shape):
+            raise ValueError("%s.pt does not match its entry in compression_meta.pt" % name)
+        meta[name] = table
+    return meta
 
 
 # ---- runtime callers -------------------------------------------------------------------------------

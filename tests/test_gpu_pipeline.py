@@ -129,3 +129,60 @@ def test_two_level_manager_serves_seeds_from_the_first_table():
     assert np.allclose(out.detach().cpu().numpy(), want, rtol=1e-4, atol=1e-4 * np.abs(want).max())
     with pytest.raises(KeyError):
         sm.get_seeds_data(src_ids[100:110])
+
+
+@pytest.mark.parametrize("ratio,with_seeds", [(8, False), (32, False), (64, True), (128, True)])
+def test_artefact_files_round_trip_into_the_manager(tmp_path, ratio, with_seeds):
+    # ratio 8 / 32: SQ at 4 / 1 bits per fp32 value; 64 / 128: VQ, 16 / 32 columns per code byte,
+    # with the seed rows in an SQ table of their own (4-bit)
+    from f2cgt_amd import pipeline
+    rng = np.random.default_rng(ratio)
+    n, d = 5000, 64
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    seeds = torch.from_numpy(np.sort(rng.permutation(n)[:400])) if with_seeds else None
+    torch.manual_seed(3)
+    np.random.seed(3)
+    meta = pipeline.run(str(tmp_path), torch.from_numpy(x), seeds=seeds, target_compression_ratio=ratio,
+                        n_clusters=64)
+    names = {"compression_meta.pt", "compression_data.pt"} | ({"seeds_compression_data.pt"} if with_seeds else set())
+    assert {p.name for p in tmp_path.iterdir()} == names
+    loaded = pipeline.load_compress_data(str(tmp_path))
+    assert loaded["methods"] == (["sq"] if with_seeds else []) + (["sq"] if ratio <= 32 else ["vq"])
+    assert loaded["feat_dim"] == d and loaded["configs"] == meta["configs"]
+    if ratio <= 32:
+        bits = 32 // ratio
+        assert loaded["configs"][-1] == (64, bits)
+        assert tuple(loaded["compression_data"].shape) == (n, d * bits // 8) and loaded["compression_data"].dtype == torch.int8
+    else:
+        w = ratio // 4
+        assert loaded["configs"][-1] == (w, -1)
+        assert tuple(loaded["compression_data"].shape) == (n, d // w) and loaded["compression_data"].dtype == torch.uint8
+        assert tuple(loaded["codebooks"][-1].shape) == (d // w, 64, w)
+    if with_seeds:
+        assert loaded["configs"][0] == (64, 4) and torch.equal(loaded["seeds"], seeds)
+        assert tuple(loaded["seeds_compression_data"].shape) == (400, d // 2)
+
+    sm = pipeline.CompressionManager(loaded, fusion=True)
+    src = np.concatenate([seeds.numpy()[:50], np.setdiff1d(np.arange(n), seeds.numpy())[:450]]) if with_seeds \
+        else rng.permutation(n)[:500]
+    src_ids = torch.from_numpy(src).cuda()
+    indptr, indices = _graph(rng, 120, 500, 7)
+    all_feat = sm.get_all_data(src_ids)
+    n_seed_dst = 50 if with_seeds else 120
+    h_self = sm.reorganize_seeds_data(sm.get_seeds_data(src_ids[:n_seed_dst]), all_feat, 120)
+    conv = pipeline.MySAGEConv(d, 8, "mean", sm).cuda()
+    out = conv((torch.from_numpy(indptr).cuda(), torch.from_numpy(indices).cuda()), (h_self, all_feat))
+
+    table = loaded["compression_data"].numpy()[src]
+    cb = loaded["codebooks"][-1].numpy()
+    if ratio <= 32:
+        dec = oc.sq_decompress_per_byte_codebook(table.view(np.uint8), cb, 32 // ratio, 64, d)
+    else:
+        dec = oc.vq_decompress(table, cb, d)
+    want_self = dec[:120].copy()
+    if with_seeds:
+        seed_rows = loaded["seeds_compression_data"].numpy()[:50].view(np.uint8)
+        want_self[:50] = oc.sq_decompress(seed_rows, loaded["codebooks"][0].numpy(), 4, 64, d)
+    assert np.array_equal(h_self.cpu().numpy(), want_self)
+    want = _reference_layer(want_self, oc.spmm_csr(dec, indptr, indices), conv)
+    assert np.allclose(out.detach().cpu().numpy(), want, rtol=1e-4, atol=1e-4 * np.abs(want).max())
