@@ -86,6 +86,65 @@ __device__ __forceinline__ void store_nt4(float* p, float a, float b, float c, f
   __builtin_nontemporal_store(v, reinterpret_cast<f4*>(p));
 }
 
+// Stages the 128-column tile `tile` of VQ codebooks [n_cb][K][w] (w a multiple of 4) into LDS as
+// [code][128 columns], columns from tile_cols on zero.  A thread issues UNROLL loads back to back
+// before it waits for the first, so the 128 KB of a 256-code tile cost a few load latencies
+// instead of one per element.  PAIR places column 8 j + 4 h + t at h * 64 + 4 j + t (the layout
+// of the kernels that give one lane a whole 8-column code).  With 16-byte aligned codebooks and
+// tile_cols a multiple of 4 the loads are float4.
+template <int THREADS, bool PAIR>
+__device__ __forceinline__ void stage_codebook_tile(float* __restrict__ s_cb, const float* __restrict__ codebooks,
+                                                    int K, int w, int tile, int tile_cols) {
+  constexpr int UNROLL = 8;
+  const bool vec = (reinterpret_cast<uintptr_t>(codebooks) & 15) == 0 && (tile_cols & 3) == 0 && (w & 3) == 0;
+  if (vec) {
+    const int n4 = K * 32;
+    for (int i0 = threadIdx.x; i0 < n4; i0 += THREADS * UNROLL) {
+      float4 v[UNROLL];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int i = i0 + u * THREADS;
+        const int code = i >> 5, c = (i & 31) * 4;
+        const bool on = i < n4 && c < tile_cols;
+        const int col = tile * 128 + c;
+        const int sub = col / w;
+        const int64_t at = on ? ((int64_t)sub * K + code) * w + (col - sub * w) : 0;
+        v[u] = *reinterpret_cast<const float4*>(codebooks + at);
+        if (!on) v[u] = float4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int i = i0 + u * THREADS;
+        const int code = i >> 5, c = (i & 31) * 4;
+        const int pos = PAIR ? ((c >> 2) & 1) * 64 + (c >> 3) * 4 : c;
+        if (i < n4) *reinterpret_cast<float4*>(s_cb + (code << 7) + pos) = v[u];
+      }
+    }
+    return;
+  }
+  const int n = K * 128;
+  for (int i0 = threadIdx.x; i0 < n; i0 += THREADS * UNROLL) {
+    float v[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int i = i0 + u * THREADS;
+      const int code = i >> 7, c = i & 127;
+      const bool on = i < n && c < tile_cols;
+      const int col = tile * 128 + c;
+      const int sub = col / w;
+      const int64_t at = on ? ((int64_t)sub * K + code) * w + (col - sub * w) : 0;
+      v[u] = on ? codebooks[at] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int i = i0 + u * THREADS;
+      const int code = i >> 7, c = i & 127;
+      const int pos = PAIR ? ((c >> 2) & 1) * 64 + (c >> 3) * 4 + (c & 3) : c;
+      if (i < n) s_cb[(code << 7) + pos] = v[u];
+    }
+  }
+}
+
 // Correctly rounded fp32 exp2 / log2: the fp64 library result rounded once.
 __device__ __forceinline__ float exp2_cr(float x) { return (float)exp2((double)x); }
 __device__ __forceinline__ float log2_cr(float x) { return (float)log2((double)x); }

@@ -73,16 +73,7 @@ __global__ __launch_bounds__(kTileThreads) void vq_decompress_tile_kernel(VqTile
   const int tile = blockIdx.x % a.n_tiles;
   const int stripe = blockIdx.x / a.n_tiles;
   const int tile_cols = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
-  for (int i = threadIdx.x; i < a.K * 128; i += kTileThreads) {
-    const int code = i >> 7, c = i & 127;
-    float v = 0.f;
-    if (c < tile_cols) {
-      const int col = tile * 128 + c;
-      const int sub = col / a.w;
-      v = a.codebooks[((int64_t)sub * a.K + code) * a.w + (col - sub * a.w)];
-    }
-    s_cb[i] = v;
-  }
+  stage_codebook_tile<kTileThreads, false>(s_cb, a.codebooks, a.K, a.w, tile, tile_cols);
   __syncthreads();
   const int c4 = threadIdx.x & 31;
   const int rs = threadIdx.x >> 5;

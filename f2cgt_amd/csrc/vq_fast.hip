@@ -249,16 +249,7 @@ __global__ __launch_bounds__(kThreads) void vq_pipe_kernel(VqArgs a, const Idx* 
 
   // codebook tile -> LDS as [code][piece][8]
   const int tile_cols = (a.feat_dim - pipe.tile * 128) >= 128 ? 128 : (a.feat_dim - pipe.tile * 128);
-  for (int i = threadIdx.x; i < a.K * 128; i += kThreads) {
-    const int code = i >> 7, c = i & 127;
-    float v = 0.f;
-    if (c < tile_cols) {
-      const int col = pipe.tile * 128 + c;
-      const int sub = col / a.w;
-      v = a.codebooks[((int64_t)sub * a.K + code) * a.w + (col - sub * a.w)];
-    }
-    pipe.s_cb[i] = v;
-  }
+  stage_codebook_tile<kThreads, false>(pipe.s_cb, a.codebooks, a.K, a.w, pipe.tile, tile_cols);
   for (int i = threadIdx.x; i < kRing * (kRows + 2); i += kThreads) pipe.s_ptr[i] = 0;
   __syncthreads();
 
@@ -291,7 +282,7 @@ constexpr int kWPtr = 56;                     // ints per offset buffer: [0..48]
 
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
-template <int BT, typename Idx>
+template <int BT, int H, typename Idx>
 __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* __restrict__ indptr,
                                                            const Idx* __restrict__ indices,
                                                            float* __restrict__ out) {
@@ -314,16 +305,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     stripe = blockIdx.x / a.n_tiles;
   }
   const int tile_cols = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
-  for (int i = threadIdx.x; i < a.K * 128; i += kThreads) {
-    const int code = i >> 7, c = i & 127;
-    float v = 0.f;
-    if (c < tile_cols) {
-      const int col = tile * 128 + c;
-      const int sub = col / a.w;
-      v = a.codebooks[((int64_t)sub * a.K + code) * a.w + (col - sub * a.w)];
-    }
-    s_cb[i] = v;
-  }
+  stage_codebook_tile<kThreads, H == 2>(s_cb, a.codebooks, a.K, a.w, tile, tile_cols);
   __syncthreads();
 
   // A wave owns one contiguous range of rows (a multiple of 4, the same for every wave, so the
@@ -337,9 +319,13 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   const int64_t n_chunks = (row_end - chunk_row0 + kWChunk - 1) / kWChunk;
   const int64_t n_mini = (row_end - chunk_row0 + kWRows - 1) / kWRows;
 
-  const int c4 = lane & 31, half = lane >> 5;
-  const bool col_on = c4 * 4 < tile_cols;
-  const int byte_idx = (c4 * 4) / a.w;
+  // lanes per row: 32 lanes with one float4 each (H == 1) or 16 lanes with a whole 8-column code
+  // each (H == 2); the wave then works on 2 or 4 rows at a time
+  constexpr int kLanesPerRow = 32 / H, kRowsPerPass = 64 / kLanesPerRow;
+  const int c4 = lane & (kLanesPerRow - 1), half = lane / kLanesPerRow;
+  const int col0 = c4 * 4 * H;                 // first column of the lane inside the tile
+  const bool col_on = col0 < tile_cols;
+  const int byte_idx = col0 / a.w;
   const float* cbp = s_cb + c4 * 4;
   const uint8_t* code_base = a.codes + tile * BT;
   const uint32_t n_last = (uint32_t)(a.N - 1);
@@ -425,13 +411,15 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       const int64_t left = row_end - row0;
       const int nr = (int)(left < kWRows ? left : kWRows);
       const bool staged = ne0 <= kWEdges;
-      float* orow = out + row0 * (int64_t)a.feat_dim + tile * 128 + c4 * 4;
+      float* orow = out + row0 * (int64_t)a.feat_dim + tile * 128 + col0;
 #pragma unroll
-      for (int pass = 0; pass < kWRows / 2; ++pass) {
-        const int row = pass * 2 + half;
+      for (int pass = 0; pass < kWRows / kRowsPerPass; ++pass) {
+        const int row = pass * kRowsPerPass + half;
         if (row >= nr) continue;
         int rb = buf[row] - eb0, re = buf[row + 1] - eb0;
-        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        float acc[H][4];
+#pragma unroll
+        for (int h = 0; h < H; ++h) acc[h][0] = acc[h][1] = acc[h][2] = acc[h][3] = 0.f;
         int n;
         if (staged) {
           rb = rb < 0 ? 0 : (rb > ne0 ? ne0 : rb);
@@ -441,20 +429,29 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
           int k = 0;
           for (; k + kGroup <= n; k += kGroup) {
             uint32_t code[kGroup];
-            float4 x[kGroup];
+            float4 x[kGroup][H];
 #pragma unroll
             for (int u = 0; u < kGroup; ++u) code[u] = cp[u * BT];
             cp += kGroup * BT;
 #pragma unroll
-            for (int u = 0; u < kGroup; ++u) x[u] = *reinterpret_cast<const float4*>(cbp + code[u] * 128);
+            for (int u = 0; u < kGroup; ++u)
 #pragma unroll
-            for (int u = 0; u < kGroup; ++u) { a0 += x[u].x; a1 += x[u].y; a2 += x[u].z; a3 += x[u].w; }
+              for (int h = 0; h < H; ++h) x[u][h] = *reinterpret_cast<const float4*>(cbp + code[u] * 128 + h * 64);
+#pragma unroll
+            for (int u = 0; u < kGroup; ++u)
+#pragma unroll
+              for (int h = 0; h < H; ++h) {
+                acc[h][0] += x[u][h].x; acc[h][1] += x[u][h].y; acc[h][2] += x[u][h].z; acc[h][3] += x[u][h].w;
+              }
           }
           for (; k < n; ++k) {
             const uint32_t code = *cp;
             cp += BT;
-            const float4 x = *reinterpret_cast<const float4*>(cbp + code * 128);
-            a0 += x.x; a1 += x.y; a2 += x.z; a3 += x.w;
+#pragma unroll
+            for (int h = 0; h < H; ++h) {
+              const float4 x = *reinterpret_cast<const float4*>(cbp + code * 128 + h * 64);
+              acc[h][0] += x.x; acc[h][1] += x.y; acc[h][2] += x.z; acc[h][3] += x.w;
+            }
           }
         } else {
           n = re - rb;
@@ -462,22 +459,48 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
           for (int k = 0; k < n; ++k) {
             const int64_t id = clamp_idx(indices[e0 + rb + k], a.N);
             const uint32_t code = a.codes[id * a.n_cb + tile * BT + byte_idx];
-            const float4 x = *reinterpret_cast<const float4*>(cbp + code * 128);
-            a0 += x.x; a1 += x.y; a2 += x.z; a3 += x.w;
+#pragma unroll
+            for (int h = 0; h < H; ++h) {
+              const float4 x = *reinterpret_cast<const float4*>(cbp + code * 128 + h * 64);
+              acc[h][0] += x.x; acc[h][1] += x.y; acc[h][2] += x.z; acc[h][3] += x.w;
+            }
           }
         }
         if (n > 1) {
           const float d = (float)n;
           float r = __builtin_amdgcn_rcpf(d);
           r = __fmaf_rn(__fmaf_rn(-d, r, 1.f), r, r);
-          a0 = div_by(a0, d, r); a1 = div_by(a1, d, r); a2 = div_by(a2, d, r); a3 = div_by(a3, d, r);
+#pragma unroll
+          for (int h = 0; h < H; ++h)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc[h][t] = div_by(acc[h][t], d, r);
         }
-        store_nt4(orow + (int64_t)row * a.feat_dim, a0, a1, a2, a3);
+#pragma unroll
+        for (int h = 0; h < H; ++h)
+          store_nt4(orow + (int64_t)row * a.feat_dim + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
       }
     }
     eb0 = eb1; ne0 = ne1;
     eb1 = eb2; ne1 = ne2;
   }
+}
+
+template <int BT, int H>
+int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
+                const char* what, unsigned grid, size_t wlds) {
+  hipError_t w1 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_wave_kernel<BT, H, int32_t>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
+  hipError_t w2 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_wave_kernel<BT, H, int64_t>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
+  if (w1 != hipSuccess || w2 != hipSuccess)
+    return fail((int)(w1 != hipSuccess ? w1 : w2), "%s: cannot reserve %zu B of LDS", what, wlds);
+  if (idx_dtype == F2CGT_DT_I32)
+    vq_wave_kernel<BT, H, int32_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int32_t*>(indptr),
+                                                                 static_cast<const int32_t*>(indices), out);
+  else
+    vq_wave_kernel<BT, H, int64_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int64_t*>(indptr),
+                                                                 static_cast<const int64_t*>(indices), out);
+  return launch_status(what);
 }
 
 template <int BT>
@@ -509,19 +532,10 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
   if (avg_deg * kWRows <= 60.0) {
     const size_t wlds = (size_t)a.K * 128 * 4 + (size_t)(kThreads / 64) * kWEdges * BT +
                         (size_t)(kThreads / 64) * 2 * kWPtr * 4;
-    hipError_t w1 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_wave_kernel<BT, int32_t>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
-    hipError_t w2 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_wave_kernel<BT, int64_t>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
-    if (w1 != hipSuccess || w2 != hipSuccess)
-      return fail((int)(w1 != hipSuccess ? w1 : w2), "%s: cannot reserve %zu B of LDS", what, wlds);
-    if (idx_dtype == F2CGT_DT_I32)
-      vq_wave_kernel<BT, int32_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int32_t*>(indptr),
-                                                                static_cast<const int32_t*>(indices), out);
-    else
-      vq_wave_kernel<BT, int64_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int64_t*>(indptr),
-                                                                static_cast<const int64_t*>(indices), out);
-    return launch_status(what);
+    // 8-column codes with whole codes in every tile: one lane per code (two float4 per edge)
+    constexpr int H = BT == 16 ? 2 : 1;
+    if (H == 2 && a.feat_dim % 8 == 0) return launch_wave<BT, H>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    return launch_wave<BT, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
   }
   if (idx_dtype == F2CGT_DT_I32)
     vq_pipe_kernel<BT, int32_t><<<grid, kThreads, lds, st>>>(a, static_cast<const int32_t*>(indptr),
