@@ -532,9 +532,8 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
   if (avg_deg * kWRows <= 60.0) {
     const size_t wlds = (size_t)a.K * 128 * 4 + (size_t)(kThreads / 64) * kWEdges * BT +
                         (size_t)(kThreads / 64) * 2 * kWPtr * 4;
-    // 8-column codes with whole codes in every tile: one lane per code (two float4 per edge)
-    constexpr int H = BT == 16 ? 2 : 1;
-    if (H == 2 && a.feat_dim % 8 == 0) return launch_wave<BT, H>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    // whole 8-column groups in every tile: one lane per group (two float4 per edge)
+    if (a.feat_dim % 8 == 0) return launch_wave<BT, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
     return launch_wave<BT, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
   }
   if (idx_dtype == F2CGT_DT_I32)
