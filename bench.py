@@ -141,7 +141,13 @@ def _others(idx):
                                                             wl["feat_dim"], wl["feat_dim"], out=out), 300, 30)
     res["c2_graph_log_sq4_fused"] = {"launch_us": ms * 1e3, "algorithmic_GBps": wl["algo_bytes"] / (ms * 1e-3) / 1e9,
                                      "frac_hbm_peak": wl["algo_bytes"] / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
-    del wl, out
+    # the uncompressed baseline operator (spmm_csr) on the same graph: fp32 rows, 400 B per edge
+    feat = torch.randn((wl["N"], wl["feat_dim"]), dtype=torch.float32, device="cuda")
+    _, ms = _time_steps(lambda: capi.spmm_csr(feat, wl["indptr"], wl["indices"], out=out), 300, 30)
+    nbytes = wl["E"] * (wl["feat_dim"] * 4 + 8) + (wl["R"] + 1) * 8 + wl["R"] * wl["feat_dim"] * 4
+    res["c2_graph_spmm_csr_fp32"] = {"launch_us": ms * 1e3, "algorithmic_GBps": nbytes / (ms * 1e-3) / 1e9,
+                                     "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    del wl, out, feat
     torch.cuda.empty_cache()
     enc = synth.c5_encode(device="cuda")
     labels = torch.empty((enc["m"],), dtype=torch.uint8, device="cuda")
