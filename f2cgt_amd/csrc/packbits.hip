@@ -2,7 +2,8 @@
 //
 // Two shapes each:
 //   * flat: unpack_dim is a multiple of 8/bits, so the whole tensor is one stream and a
-//     lane converts 4 packed bytes <-> 4*(8/bits) code bytes with dword accesses;
+//     lane converts 16 code bytes <-> 16/(8/bits) packed bytes, one dense 16-byte access on the
+//     code side and one dense 2/4/8-byte access on the packed side;
 //   * rows: ragged tails (unpack_dim not a multiple of 8/bits), one lane per packed byte
 //     (pack) or per code byte (unpack).
 #include "common.hpp"
@@ -34,25 +35,40 @@ __global__ __launch_bounds__(kBlock) void pack_rows_kernel(const uint8_t* __rest
   }
 }
 
-// Flat stream: lane g turns code bytes [4*PER*g, 4*PER*(g+1)) into packed dword g.
+// Flat stream in units of 16 code bytes: a lane turns one 16-byte load of codes into 16 / PER
+// packed bytes (one dense store per lane), four units per lane with the loads issued first.
+constexpr int kUnitsPerThread = 4;
+template <int BYTES> struct uint_of;
+template <> struct uint_of<2> { using type = uint16_t; };
+template <> struct uint_of<4> { using type = uint32_t; };
+template <> struct uint_of<8> { using type = uint64_t; };
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
 template <int BITS>
-__global__ __launch_bounds__(kBlock) void pack_flat_kernel(const uint32_t* __restrict__ unpack,
-                                                           uint32_t* __restrict__ pack,
-                                                           int64_t n_words) {
+__global__ __launch_bounds__(kBlock) void pack_flat_kernel(const u32x4* __restrict__ unpack,
+                                                           typename uint_of<2 * BITS>::type* __restrict__ pack,
+                                                           int64_t n_units) {
   constexpr int PER = 8 / BITS;
   constexpr uint32_t MASK = (1u << BITS) - 1u;
-  const int64_t stride = (int64_t)gridDim.x * kBlock;
-  for (int64_t g = (int64_t)blockIdx.x * kBlock + threadIdx.x; g < n_words; g += stride) {
-    uint32_t in[PER];
+  using OT = typename uint_of<2 * BITS>::type;       // 16 / PER bytes
+  const int64_t base = (int64_t)blockIdx.x * (kBlock * kUnitsPerThread) + threadIdx.x;
+  u32x4 in[kUnitsPerThread];
 #pragma unroll
-    for (int w = 0; w < PER; ++w) in[w] = unpack[g * PER + w];
-    uint32_t out = 0;
+  for (int u = 0; u < kUnitsPerThread; ++u) {
+    const int64_t q = base + u * kBlock;
+    in[u] = __builtin_nontemporal_load(unpack + (q < n_units ? q : 0));
+  }
 #pragma unroll
-    for (int e = 0; e < 4 * PER; ++e) {
-      const uint32_t code = (in[e / 4] >> (8 * (e % 4))) & MASK;
+  for (int u = 0; u < kUnitsPerThread; ++u) {
+    const int64_t q = base + u * kBlock;
+    if (q >= n_units) break;
+    uint64_t out = 0;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const uint64_t code = (in[u][e / 4] >> (8 * (e % 4))) & MASK;
       out |= code << (8 * (e / PER) + BITS * (e % PER));
     }
-    pack[g] = out;
+    __builtin_nontemporal_store((OT)out, pack + q);
   }
 }
 
@@ -73,25 +89,35 @@ __global__ __launch_bounds__(kBlock) void unpack_rows_kernel(const uint8_t* __re
 }
 
 template <int BITS>
-__global__ __launch_bounds__(kBlock) void unpack_flat_kernel(const uint32_t* __restrict__ pack,
-                                                             uint32_t* __restrict__ unpack,
-                                                             int64_t n_words) {
+__global__ __launch_bounds__(kBlock) void unpack_flat_kernel(const typename uint_of<2 * BITS>::type* __restrict__ pack,
+                                                             u32x4* __restrict__ unpack, int64_t n_units) {
   constexpr int PER = 8 / BITS;
   constexpr uint32_t MASK = (1u << BITS) - 1u;
-  const int64_t stride = (int64_t)gridDim.x * kBlock;
-  for (int64_t g = (int64_t)blockIdx.x * kBlock + threadIdx.x; g < n_words; g += stride) {
-    const uint32_t in = pack[g];
+  using IT = typename uint_of<2 * BITS>::type;
+  const int64_t base = (int64_t)blockIdx.x * (kBlock * kUnitsPerThread) + threadIdx.x;
+  IT in[kUnitsPerThread];
 #pragma unroll
-    for (int w = 0; w < PER; ++w) {
-      uint32_t out = 0;
+  for (int u = 0; u < kUnitsPerThread; ++u) {
+    const int64_t q = base + u * kBlock;
+    in[u] = __builtin_nontemporal_load(pack + (q < n_units ? q : 0));
+  }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int e = 4 * w + j;
-        const uint32_t code = (in >> (8 * (e / PER) + BITS * (e % PER))) & MASK;
-        out |= code << (8 * j);
+  for (int u = 0; u < kUnitsPerThread; ++u) {
+    const int64_t q = base + u * kBlock;
+    if (q >= n_units) break;
+    const uint64_t v = (uint64_t)in[u];
+    u32x4 out;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint32_t w = 0;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int e = 4 * j + t;
+        w |= (uint32_t)((v >> (8 * (e / PER) + BITS * (e % PER))) & MASK) << (8 * t);
       }
-      unpack[g * PER + w] = out;
+      out[j] = w;
     }
+    __builtin_nontemporal_store(out, unpack + q);
   }
 }
 
@@ -108,12 +134,13 @@ int pack_launch(const uint8_t* unpack, uint8_t* pack, int64_t rows, int64_t U, h
   const int64_t n_out = rows * P;
   if (n_out == 0) return 0;
   int64_t done = 0;
-  if (U % PER == 0 && aligned(unpack, 4) && aligned(pack, 4)) {
-    const int64_t n_words = n_out / 4;
-    if (n_words > 0) {
-      pack_flat_kernel<BITS><<<grid_for(n_words), kBlock, 0, st>>>(
-          reinterpret_cast<const uint32_t*>(unpack), reinterpret_cast<uint32_t*>(pack), n_words);
-      done = n_words * 4;
+  if (U % PER == 0 && aligned(unpack, 16) && aligned(pack, 16 / PER)) {
+    const int64_t n_units = (rows * U) / 16;
+    const int64_t blocks = ceil_div(n_units, kBlock * kUnitsPerThread);
+    if (n_units > 0 && blocks <= 0x7fffffffll) {
+      pack_flat_kernel<BITS><<<(unsigned)blocks, kBlock, 0, st>>>(
+          reinterpret_cast<const u32x4*>(unpack), reinterpret_cast<typename uint_of<2 * BITS>::type*>(pack), n_units);
+      done = n_units * (16 / PER);
     }
   }
   if (done < n_out)
@@ -128,12 +155,13 @@ int unpack_launch(const uint8_t* pack, uint8_t* unpack, int64_t rows, int64_t P,
   const int64_t n_out = rows * U;
   if (n_out == 0) return 0;
   int64_t done = 0;
-  if (U == P * PER && aligned(unpack, 4) && aligned(pack, 4)) {
-    const int64_t n_words = (rows * P) / 4;
-    if (n_words > 0) {
-      unpack_flat_kernel<BITS><<<grid_for(n_words), kBlock, 0, st>>>(
-          reinterpret_cast<const uint32_t*>(pack), reinterpret_cast<uint32_t*>(unpack), n_words);
-      done = n_words * 4 * PER;
+  if (U == P * PER && aligned(unpack, 16) && aligned(pack, 16 / PER)) {
+    const int64_t n_units = (rows * U) / 16;
+    const int64_t blocks = ceil_div(n_units, kBlock * kUnitsPerThread);
+    if (n_units > 0 && blocks <= 0x7fffffffll) {
+      unpack_flat_kernel<BITS><<<(unsigned)blocks, kBlock, 0, st>>>(
+          reinterpret_cast<const typename uint_of<2 * BITS>::type*>(pack), reinterpret_cast<u32x4*>(unpack), n_units);
+      done = n_units * 16;
     }
   }
   if (done < n_out)
