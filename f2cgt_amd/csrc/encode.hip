@@ -4,16 +4,19 @@
 // sum((x-y)^2) (or 1 - cos) with fused multiply-adds on the vector ALUs, so the numbers carry
 // no cancellation error, and at small k the vector ALUs rather than the matrix write bound it.
 //
-// kmeans_predict never writes the matrix.  A wave owns 32 rows of x and walks the
-// centres 64 at a time with fp32 MFMA (v_mfma_f32_32x32x2_f32): A = centre tile,
-// B = x tile, so every lane holds 16 centre scores of ONE x row per tile and the running
-// arg-min stays in registers.  Scores use the expanded form (|c|^2 - 2 x.c, the row
-// constant |x|^2 dropped); rows whose two best scores are closer than the rounding
-// bound of that form are re-evaluated exactly in fp64 by the whole wave, so the label
-// is the true first minimum.  On this chip vector instructions do not run in the shadow of
-// matrix instructions of the same SIMD (measured: a 128-instruction update per 34 MFMAs costs
-// its full issue time with one to three waves per SIMD), so the update is kept to four
-// instructions per score and everything else is folded into the MFMA operands.
+// kmeans_predict never writes the matrix.  A wave owns rows of x and walks the centres a tile
+// at a time on the matrix core: A = centre tile, B = x tile, so every lane holds 16 centre
+// scores of ONE x row per tile and the running arg-min stays in registers.  Scores use the
+// expanded form (|c|^2 - 2 x.c, the row constant |x|^2 dropped); rows whose two best scores are
+// closer than the rounding bound of that evaluation are re-evaluated exactly in fp64 by the
+// whole wave, so the label is the true first minimum.  Two evaluations of x.c:
+//   * predict_split_kernel (up to 64 dimensions, operands within 96 KB of LDS): every fp32
+//     value as three bf16 pieces, six v_mfma_f32_32x32x16_bf16 per 16 dimensions;
+//   * predict_mfma_kernel: fp32 MFMA (v_mfma_f32_32x32x2_f32).  Vector instructions do not run in
+//     the shadow of fp32 matrix instructions of the same SIMD (measured: a 128-instruction update
+//     per 34 MFMAs costs its full issue time with one to three waves per SIMD), so there the
+//     update is kept to four instructions per score and everything else is folded into the
+//     MFMA operands.
 #include "common.hpp"
 
 #include <cfloat>
@@ -281,6 +284,443 @@ __global__ __launch_bounds__(256) void predict_mfma_kernel(const float* __restri
   }
 }
 
+// ---- split-bf16 MFMA path ------------------------------------------------------------------
+// The same scores at the bf16 matrix rate.  An fp32 value is the exact sum of three bf16 pieces
+// (round to nearest, then the residual, then its residual: 3 x 8 significand bits plus the signs
+// cover 24), a product of two pieces is exact in fp32, and of the nine piece products of x * c the
+// three of relative size <= 2^-26 are dropped, so six v_mfma_f32_32x32x16_bf16 per 16 dimensions
+// give x . c to fp32 accuracy at a sixth of the bf16 rate, 2.7 times the fp32 MFMA rate, and, unlike
+// fp32 MFMA, with the vector ALUs free for the arg-min update while the matrix core runs.  The
+// centre pieces sit in LDS in operand order ([piece][tile][step][lane] x 16 B, one ds_read_b128 per
+// operand), a wave keeps the pieces of NB x 32 rows of x in registers so that every operand read
+// feeds NB instructions, and the bias |c|^2 enters as the C operand of a tile's first instruction.
+// Labels are decided as in the fp32 kernel: rows whose two best scores are closer than the
+// rounding bound of this evaluation are re-evaluated exactly in fp64.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ void split3(float v, __bf16& p0, __bf16& p1, __bf16& p2) {
+  p0 = (__bf16)v;
+  float r = v - (float)p0;      // exact: the rounding error of a narrower format
+  p1 = (__bf16)r;
+  r = r - (float)p1;
+  p2 = (__bf16)r;
+}
+
+// Exact L2 assignment of one row by a whole wave from the centre pieces in LDS (their sum is the
+// fp32 centre, exactly); same result as exact_argmin_row on the array in HBM.  The unexpanded fp32
+// distance has relative error <= (k + 3) 2^-24 (all terms positive), so it decides which centres
+// can be the minimum at all; only those, usually two, are evaluated in fp64.
+template <int S>
+__device__ int exact_argmin_row_l2_pieces(const float* __restrict__ xrow, float* xs, const bf16x8* ap, int n, int n_ct,
+                                          int k, int lane) {
+  // the row goes through a wave-private LDS slot (16 S floats, zero padded) and the loops over the
+  // 8-dimension chunks stay rolled: this rare path must not raise the kernel's register count
+  const int piece_stride = n_ct * S * 64;                // operands per piece
+  if (lane < 16 * S) xs[lane] = lane < k ? xrow[lane] : 0.f;
+  __builtin_amdgcn_wave_barrier();                       // LDS operations of one wave execute in order
+  // fp32 centre values of chunk ch (dimensions [8 ch, 8 ch + 8)) of centre c: one operand per piece
+  auto centre8 = [&](int c, int ch, float (&cv)[8]) {
+    const bf16x8* q = ap + (c >> 5) * S * 64 + (ch >> 1) * 64 + (ch & 1) * 32 + (c & 31);
+    const bf16x8 p0 = q[0], p1 = q[piece_stride], p2 = q[2 * piece_stride];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) cv[e] = ((float)p0[e] + (float)p1[e]) + (float)p2[e];
+  };
+  // first pass: distance from the leading pieces only (relative error of a centre value 2^-9, of
+  // a distance well below 2^-3 of itself plus 2^-3 of the smallest one), one operand per chunk
+  auto dist_lead = [&](int c) -> float {
+    float d = 0.f;
+#pragma nounroll
+    for (int ch = 0; ch < 2 * S; ++ch) {
+      const bf16x8 p0 = ap[(c >> 5) * S * 64 + (ch >> 1) * 64 + (ch & 1) * 32 + (c & 31)];
+      const float4 xa = *reinterpret_cast<const float4*>(xs + 8 * ch);
+      const float4 xb = *reinterpret_cast<const float4*>(xs + 8 * ch + 4);
+      const float xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float df = xv[e] - (float)p0[e];
+        d = __fmaf_rn(df, df, d);
+      }
+    }
+    return d;
+  };
+  auto dist32 = [&](int c) -> float {
+    float d = 0.f;
+#pragma nounroll
+    for (int ch = 0; ch < 2 * S; ++ch) {
+      float cv[8];
+      centre8(c, ch, cv);
+      const float4 xa = *reinterpret_cast<const float4*>(xs + 8 * ch);
+      const float4 xb = *reinterpret_cast<const float4*>(xs + 8 * ch + 4);
+      const float xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float df = xv[e] - cv[e];                  // dimensions >= k hold zeros on both sides
+        d = __fmaf_rn(df, df, d);
+      }
+    }
+    return d;
+  };
+  // With c' the leading pieces, |c - c'| <= 2^-9 |c| per component, so
+  // | sqrt(d) - sqrt(d') | <= 2^-9 |c| <= 2^-9 (|x| + sqrt(d)): a centre can only be the minimum if
+  // sqrt(d') <= (sqrt(dmin') + 2^-8 |x|) * (1 + 2^-7) (slack for the fp32 sums included).
+  constexpr int kKeep = 4;            // first-pass distances kept in registers (all of them up to 256 centres)
+  float dkeep[kKeep] = {0.f, 0.f, 0.f, 0.f};
+  float dmin = INFINITY;
+  // the lane's first four centres two at a time: two independent chains per chunk
+#pragma unroll
+  for (int i0 = 0; i0 < kKeep; i0 += 2) {
+    int slot[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      int c = lane + (i0 + i) * kWave;
+      c = c < n ? c : 0;
+      slot[i] = (c >> 5) * S * 64 + (c & 31);
+    }
+#pragma nounroll
+    for (int ch = 0; ch < 2 * S; ++ch) {
+      const int at = (ch >> 1) * 64 + (ch & 1) * 32;
+      const bf16x8 pa = ap[slot[0] + at], pb = ap[slot[1] + at];
+      const float4 xa = *reinterpret_cast<const float4*>(xs + 8 * ch);
+      const float4 xb = *reinterpret_cast<const float4*>(xs + 8 * ch + 4);
+      const float xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float da = xv[e] - (float)pa[e], db = xv[e] - (float)pb[e];
+        dkeep[i0] = __fmaf_rn(da, da, dkeep[i0]);
+        dkeep[i0 + 1] = __fmaf_rn(db, db, dkeep[i0 + 1]);
+      }
+    }
+    asm volatile("" ::: "memory");
+  }
+#pragma unroll
+  for (int i = 0; i < kKeep; ++i) {
+    if (lane + i * kWave >= n) dkeep[i] = INFINITY;
+    dmin = fminf(dmin, dkeep[i]);
+  }
+  for (int c = lane + kKeep * kWave; c < n; c += kWave) dmin = fminf(dmin, dist_lead(c));
+  float xnorm2 = lane < 16 * S ? xs[lane] * xs[lane] : 0.f;
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    dmin = fminf(dmin, __shfl_xor(dmin, off));
+    xnorm2 += __shfl_xor(xnorm2, off);
+  }
+  const float reach = (sqrtf(dmin) + 0.00390625f * sqrtf(xnorm2)) * 1.0078125f;
+  const float lead_limit = reach * reach * 1.0001f + 1e-37f;
+  // second pass: full fp32 distance of the survivors, then the exact fp64 one of those that can
+  // still be the minimum (relative error of the fp32 sum <= (k + 3) 2^-24, all terms positive)
+  float d32min = INFINITY;
+#pragma unroll
+  for (int i = 0; i < kKeep; ++i) {      // the kept distances become the fp32 ones
+    const int c = lane + i * kWave;
+    dkeep[i] = (c < n && dkeep[i] <= lead_limit) ? dist32(c) : INFINITY;
+    d32min = fminf(d32min, dkeep[i]);
+    asm volatile("" ::: "memory");
+  }
+  for (int c = lane + kKeep * kWave; c < n; c += kWave)
+    if (dist_lead(c) <= lead_limit) d32min = fminf(d32min, dist32(c));
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) d32min = fminf(d32min, __shfl_xor(d32min, off));
+  const float limit = d32min * (1.f + 1.1920929e-7f * (float)(k + 4)) + 1e-37f;
+  double bestv = DBL_MAX;
+  int besti = INT_MAX;
+  for (int c = lane, i = 0; c < n; c += kWave, ++i) {
+    float d32 = dkeep[0];
+#pragma unroll
+    for (int q = 1; q < kKeep; ++q) d32 = i == q ? dkeep[q] : d32;
+    if (i >= kKeep) d32 = dist_lead(c) <= lead_limit ? dist32(c) : INFINITY;
+    if (!(d32 <= limit)) continue;
+    double dd = 0.0;
+#pragma nounroll
+    for (int ch = 0; ch < 2 * S; ++ch) {
+      float cv[8];
+      centre8(c, ch, cv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const double df = (double)xs[8 * ch + e] - (double)cv[e];
+        dd += df * df;
+      }
+    }
+    if (dd < bestv) { bestv = dd; besti = c; }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const double ov = __shfl_xor(bestv, off);
+    const int oi = __shfl_xor(besti, off);
+    if (ov < bestv || (ov == bestv && oi < besti)) { bestv = ov; besti = oi; }
+  }
+  return besti;
+}
+
+// Exact cosine assignment of one row by a whole wave.  The LDS pieces hold the centres divided by
+// their norms; with c' their leading pieces, |x . c/|c| - x . c'| <= 2^-9 |x| (1 + 2^-20), so only
+// centres whose leading-piece dot product is within 2^-7 |x| of the largest can have the smallest
+// distance; those are evaluated exactly, in fp64 from the centres in HBM, by the formula of
+// exact_argmin_row.  Needs every centre to have a direction (|c|^2 > 1e-12).
+template <int S>
+__device__ int exact_argmin_row_cosine_pieces(const float* __restrict__ xrow, float* xs, const bf16x8* ap,
+                                              const float* __restrict__ centers, int n, int n_ct, int k,
+                                              int lane) {
+  if (lane < 16 * S) xs[lane] = lane < k ? xrow[lane] : 0.f;
+  __builtin_amdgcn_wave_barrier();
+  float xnorm2 = lane < 16 * S ? xs[lane] * xs[lane] : 0.f;
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) xnorm2 += __shfl_xor(xnorm2, off);
+  auto dot_lead = [&](int c) -> float {
+    float d = 0.f;
+#pragma nounroll
+    for (int ch = 0; ch < 2 * S; ++ch) {
+      const bf16x8 p0 = ap[(c >> 5) * S * 64 + (ch >> 1) * 64 + (ch & 1) * 32 + (c & 31)];
+      const float4 xa = *reinterpret_cast<const float4*>(xs + 8 * ch);
+      const float4 xb = *reinterpret_cast<const float4*>(xs + 8 * ch + 4);
+      const float xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) d = __fmaf_rn(xv[e], (float)p0[e], d);
+    }
+    return d;
+  };
+  float smax = -INFINITY;
+  for (int c = lane; c < n; c += kWave) smax = fmaxf(smax, dot_lead(c));
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) smax = fmaxf(smax, __shfl_xor(smax, off));
+  const float floor_s = smax - 0.0078125f * sqrtf(xnorm2) - 1e-30f;
+  double xn = 0.0;
+  for (int t = 0; t < k; ++t) xn += (double)xrow[t] * (double)xrow[t];
+  double bestv = DBL_MAX;
+  int besti = INT_MAX;
+  for (int c = lane; c < n; c += kWave) {
+    if (!(dot_lead(c) >= floor_s)) continue;
+    const float* cr = centers + (int64_t)c * k;
+    double dot = 0.0, cn = 0.0;
+    for (int t = 0; t < k; ++t) {
+      dot += (double)xrow[t] * (double)cr[t];
+      cn += (double)cr[t] * (double)cr[t];
+    }
+    double den = sqrt(xn) * sqrt(cn);
+    den = den > 1e-8 ? den : 1e-8;
+    const double d = 1.0 - dot / den;
+    if (d < bestv) { bestv = d; besti = c; }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const double ov = __shfl_xor(bestv, off);
+    const int oi = __shfl_xor(besti, off);
+    if (ov < bestv || (ov == bestv && oi < besti)) { bestv = ov; besti = oi; }
+  }
+  return besti;
+}
+
+template <int S, int NB>
+__global__ __launch_bounds__(256) void predict_split_kernel(const float* __restrict__ x,
+                                                            const float* __restrict__ centers,
+                                                            int64_t* __restrict__ lab64,
+                                                            uint8_t* __restrict__ lab8, int64_t m,
+                                                            int n, int k, int metric, int n_pad) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int n_ct = n_pad >> 5;                                   // 32-centre tiles
+  bf16x8* ap = reinterpret_cast<bf16x8*>(smem_raw);              // [3][n_ct][S][64]
+  float* bias = reinterpret_cast<float*>(smem_raw + (size_t)3 * n_ct * S * 64 * 16);   // [n_pad]
+  float* inv = bias + n_pad;                                     // [n_pad] 1 / |c| (cosine) or 1
+  int* cmax_bits = reinterpret_cast<int*>(inv + n_pad);
+  float* xs = reinterpret_cast<float*>(cmax_bits + 4) + (threadIdx.x >> 6) * 16 * S;   // one row of x per wave
+  const bool cosine = metric == F2CGT_METRIC_COSINE;
+  if (threadIdx.x == 0) { cmax_bits[0] = 0; cmax_bits[1] = 0; }
+  __syncthreads();
+  for (int jj = threadIdx.x; jj < n_pad; jj += blockDim.x) {
+    float cn = 0.f;
+    if (jj < n) {
+      const float* cr = centers + (int64_t)jj * k;
+      int t = 0;
+      for (; t + 8 <= k; t += 8) {       // eight loads in flight, summed in dimension order
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = cr[t + e];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) cn += v[e] * v[e];
+      }
+      for (; t < k; ++t) cn += cr[t] * cr[t];
+    }
+    float sc = 1.f;
+    if (cosine) {
+      const float nr = sqrtf(cn);
+      sc = 1.f / (nr > 1e-30f ? nr : 1e-30f);
+    }
+    inv[jj] = sc;
+    bias[jj] = jj >= n ? INFINITY : (cosine ? 0.f : cn);
+    if (jj < n && !cosine) atomicMax(cmax_bits, __float_as_int(cn));
+    if (jj < n && cosine && !(cn > 1e-12f)) atomicOr(cmax_bits + 1, 1);   // a centre without a direction
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < n_ct * S * 64; idx += blockDim.x) {
+    const int ln = idx & 63, ts = idx >> 6;
+    const int st = ts % S, tile = ts / S;
+    const int c = tile * 32 + (ln & 31);
+    const int kk0 = 16 * st + 8 * (ln >> 5);
+    bf16x8 p0, p1, p2;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float v = 0.f;
+      if (c < n && kk0 + e < k) v = centers[(int64_t)c * k + kk0 + e] * inv[c];
+      __bf16 a0, a1, a2;
+      split3(v, a0, a1, a2);
+      p0[e] = a0; p1[e] = a1; p2[e] = a2;
+    }
+    ap[(0 * n_ct + tile) * S * 64 + st * 64 + ln] = p0;
+    ap[(1 * n_ct + tile) * S * 64 + st * 64 + ln] = p1;
+    ap[(2 * n_ct + tile) * S * 64 + st * 64 + ln] = p2;
+  }
+  __syncthreads();
+  const float cmax = __int_as_float(cmax_bits[0]);
+  const bool plain_cosine = cmax_bits[1] != 0;   // degenerate centres: no candidate filter for cosine
+
+  const int lane = threadIdx.x & 63;
+  const int j = lane & 31;
+  const int g = lane >> 5;
+  constexpr int kGroupRows = 32 * NB;
+  const int64_t n_groups = (m + kGroupRows - 1) / kGroupRows;
+  // Error bound of one score in units of 2^-24 (|x|^2 + max |c|^2), which is >= 2 |x||c| = P and
+  // >= |c|^2: each of the S leading instructions cuts its 17 addends at 2^-22 of the largest
+  // (<= P): 68 S; the small pairs together stay below 4; the bias sum k + 1; its addition 2; the
+  // dropped pairs 1.  Doubled for the two scores of a gap.
+  const float unit = 5.9604645e-8f * (float)(2 * (68 * S + k + 8));
+  const float xscale = cosine ? -1.f : -2.f;
+  const bool vec4 = (k % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+  const int64_t group0 = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t gstride = (int64_t)gridDim.x * 4;
+  for (int64_t grp = group0; grp < n_groups; grp += gstride) {
+    bf16x8 xp[NB][S][3];
+    float xn[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int64_t row = grp * kGroupRows + 32 * b + j;
+      const bool valid = row < m;
+      float sum = 0.f;
+#pragma unroll
+      for (int st = 0; st < S; ++st) {
+        const int kk0 = 16 * st + 8 * g;
+        float q[8];
+        if (vec4) {
+          float4 u = make_float4(0.f, 0.f, 0.f, 0.f), w = u;
+          if (valid && kk0 < k) {
+            const float4* xp4 = reinterpret_cast<const float4*>(x + row * k + kk0);
+            u = xp4[0];
+            w = xp4[1];
+          }
+          q[0] = u.x; q[1] = u.y; q[2] = u.z; q[3] = u.w; q[4] = w.x; q[5] = w.y; q[6] = w.z; q[7] = w.w;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) q[e] = (valid && kk0 + e < k) ? x[row * k + kk0 + e] : 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          sum += q[e] * q[e];
+          __bf16 a0, a1, a2;
+          split3(q[e] * xscale, a0, a1, a2);
+          xp[b][st][0][e] = a0; xp[b][st][1][e] = a1; xp[b][st][2][e] = a2;
+        }
+      }
+      sum += __shfl_xor(sum, 32);
+      xn[b] = sum;
+    }
+
+    float best[NB], second[NB];
+    int bv[NB], bct[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) { best[b] = INFINITY; second[b] = INFINITY; bv[b] = 0; bct[b] = 0; }
+    for (int ct = 0; ct < n_ct; ++ct) {
+      floatx16 bz;
+      const float* bp = bias + ct * 32 + 4 * g;
+#pragma unroll
+      for (int v4 = 0; v4 < 4; ++v4) {
+        const float4 t4 = *reinterpret_cast<const float4*>(bp + 8 * v4);
+        bz[4 * v4] = t4.x; bz[4 * v4 + 1] = t4.y; bz[4 * v4 + 2] = t4.z; bz[4 * v4 + 3] = t4.w;
+      }
+      bf16x8 a[3][S];
+#pragma unroll
+      for (int q = 0; q < 3; ++q)
+#pragma unroll
+        for (int st = 0; st < S; ++st) a[q][st] = ap[(q * n_ct + ct) * S * 64 + st * 64 + lane];
+      floatx16 acc[NB];
+      // Piece pairs (x piece, centre piece).  The matrix core aligns the 16 products and C of an
+      // instruction to the largest of them and keeps about 24 bits below it (measured: a unit
+      // product next to +-2^24 survives, next to +-2^28 it does not), so the small pairs are
+      // summed first, from zero, the leading pair last, and the bias, as large as the whole dot
+      // product, is added on the vector ALU: the leading products are then cut at 2^-22 of their
+      // own size, not of |c|^2 plus the running sum.
+      constexpr int px[6] = {2, 0, 1, 1, 0, 0};
+      constexpr int pc[6] = {0, 2, 1, 0, 1, 0};
+      floatx16 zero;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) zero[v] = 0.f;
+#pragma unroll
+      for (int b = 0; b < NB; ++b) acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[pc[0]][0], xp[b][0][px[0]], zero, 0, 0, 0);
+#pragma unroll
+      for (int term = 0; term < 6; ++term)
+#pragma unroll
+        for (int st = 0; st < S; ++st) {
+          if (term == 0 && st == 0) continue;
+#pragma unroll
+          for (int b = 0; b < NB; ++b)
+            acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[pc[term]][st], xp[b][st][px[term]], acc[b], 0, 0, 0);
+        }
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[b][v] += bz[v];
+        argmin_update(acc[b], ct * 32, best[b], second[b], bv[b], bct[b]);
+      }
+    }
+    int besti[NB];
+    uint64_t todo[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const bool valid = grp * kGroupRows + 32 * b + j < m;
+      int bi = bct[b] + 8 * (bv[b] >> 2) + 4 * g + (bv[b] & 3);
+      float bs = best[b], sd = second[b];
+      {  // merge the two halves of the wave (same x row, disjoint centres)
+        const float ob = __shfl_xor(bs, 32);
+        const float os = __shfl_xor(sd, 32);
+        const int oi = __shfl_xor(bi, 32);
+        if (ob < bs || (ob == bs && oi < bi)) {
+          sd = fminf(bs, os);
+          bs = ob;
+          bi = oi;
+        } else {
+          sd = fminf(sd, ob);
+        }
+      }
+      const float scale = cosine ? sqrtf(xn[b]) : xn[b] + cmax;
+      besti[b] = bi;
+      todo[b] = __ballot(valid && g == 0 && !((sd - bs) > unit * scale));
+    }
+    // exact re-evaluation of the flagged rows: one copy of the code, whichever tile the row is in
+#pragma nounroll
+    for (int b = 0; b < NB; ++b) {
+      uint64_t td = todo[0];
+#pragma unroll
+      for (int q = 1; q < NB; ++q) td = b == q ? todo[q] : td;
+      while (td) {
+        const int src = __ffsll((unsigned long long)td) - 1;
+        td &= td - 1;
+        const int64_t rrow = grp * kGroupRows + 32 * b + (src & 31);
+        int exact;
+        if (!cosine) exact = exact_argmin_row_l2_pieces<S>(x + rrow * k, xs, ap, n, n_ct, k, lane);
+        else if (plain_cosine) exact = exact_argmin_row(x + rrow * k, centers, n, k, metric, lane);
+        else exact = exact_argmin_row_cosine_pieces<S>(x + rrow * k, xs, ap, centers, n, n_ct, k, lane);
+#pragma unroll
+        for (int q = 0; q < NB; ++q) besti[q] = (b == q && lane == src) ? exact : besti[q];
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int64_t row = grp * kGroupRows + 32 * b + j;
+      if (row < m && g == 0) {
+        if (lab64) lab64[row] = besti[b];
+        if (lab8) lab8[row] = (uint8_t)besti[b];
+      }
+    }
+  }
+}
+
 // ---- pairwise distance --------------------------------------------------------------------
 // 128 x 128 output tile per 256-thread workgroup, 8 x 8 per thread: per staged k step a thread
 // reads 8 + 8 values from LDS (four 16-byte reads) for 64 fused multiply-adds, so the vector
@@ -405,6 +845,32 @@ int launch_mfma(const float* x, const float* centers, int64_t* l64, uint8_t* l8,
   return launch_status("kmeans_predict");
 }
 
+template <int S, int NB>
+int launch_split(const float* x, const float* centers, int64_t* l64, uint8_t* l8, int64_t m, int n, int k,
+                 int metric, int n_pad, size_t lds, hipStream_t st) {
+  auto kern = predict_split_kernel<S, NB>;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail((int)e, "kmeans_predict: cannot reserve %zu B of LDS", lds);
+  }
+  // resident grid, as for the fp32 kernel
+  static thread_local size_t cached_lds = 0;
+  static thread_local int cached_per_cu = 0;
+  if (cached_per_cu == 0 || cached_lds != lds) {
+    int v = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, reinterpret_cast<const void*>(kern), 256, lds) !=
+            hipSuccess || v < 1)
+      v = 1;
+    cached_per_cu = v;
+    cached_lds = lds;
+  }
+  const int64_t need = ceil_div(ceil_div(m, 32 * NB), 4);
+  const int64_t cap = (int64_t)num_cus() * cached_per_cu;
+  kern<<<(int)(need < cap ? need : cap), 256, lds, st>>>(x, centers, l64, l8, m, n, k, metric, n_pad);
+  return launch_status("kmeans_predict");
+}
+
 }  // namespace
 }  // namespace f2cgt
 
@@ -439,6 +905,20 @@ extern "C" int f2cgt_kmeans_predict(const float* x, const float* centers, int64_
   F2CGT_REQUIRE(x && centers && (labels_i64 || labels_u8), F2CGT_E_INVALID,
                 "kmeans_predict: null buffer");
   hipStream_t st = as_stream(stream);
+  {  // split-bf16 path: up to 64 dimensions, operand pieces and biases within 96 KB of LDS
+    const int steps = (int)ceil_div(k, 16);
+    const int n_pad32 = (int)ceil_div(n, 32) * 32;
+    const size_t lds = (size_t)3 * (n_pad32 / 32) * steps * 64 * 16 + (size_t)2 * n_pad32 * 4 + 16 +
+                       (size_t)4 * 16 * steps * 4;
+    if (steps <= 4 && lds <= 96 * 1024) {
+      switch (steps) {
+        case 1: return launch_split<1, 2>(x, centers, labels_i64, labels_u8, m, (int)n, (int)k, metric, n_pad32, lds, st);
+        case 2: return launch_split<2, 2>(x, centers, labels_i64, labels_u8, m, (int)n, (int)k, metric, n_pad32, lds, st);
+        case 3: return launch_split<3, 2>(x, centers, labels_i64, labels_u8, m, (int)n, (int)k, metric, n_pad32, lds, st);
+        default: return launch_split<4, 2>(x, centers, labels_i64, labels_u8, m, (int)n, (int)k, metric, n_pad32, lds, st);
+      }
+    }
+  }
   const int khalf = (int)((k + 1) / 2);
   int kh = pow2_ceil(khalf);
   if (kh < 4) kh = 4;

@@ -1,6 +1,8 @@
 // Library-level state: per-thread error text and the cached device description.
 #include "common.hpp"
 
+#include <atomic>
+
 namespace f2cgt {
 
 char* error_buffer() {
@@ -9,18 +11,16 @@ char* error_buffer() {
 }
 
 int num_cus() {
-  static int cached[64];
-  static bool known[64];
+  static std::atomic<int> cached[64];   // 0 = not asked yet; callers may come from several threads
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (!known[dev]) {
-    int n = 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
       n = 256;
-    cached[dev] = n;
-    known[dev] = true;
+    cached[dev].store(n, std::memory_order_relaxed);
   }
-  return cached[dev];
+  return n;
 }
 
 }  // namespace f2cgt

@@ -488,12 +488,10 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
 template <int BT, int H>
 int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
                 const char* what, unsigned grid, size_t wlds) {
-  hipError_t w1 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_wave_kernel<BT, H, int32_t>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
-  hipError_t w2 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_wave_kernel<BT, H, int64_t>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
-  if (w1 != hipSuccess || w2 != hipSuccess)
-    return fail((int)(w1 != hipSuccess ? w1 : w2), "%s: cannot reserve %zu B of LDS", what, wlds);
+  const void* kern = idx_dtype == F2CGT_DT_I32 ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, int32_t>)
+                                               : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, int64_t>);
+  const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
+  if (e != hipSuccess) return fail((int)e, "%s: cannot reserve %zu B of LDS", what, wlds);
   if (idx_dtype == F2CGT_DT_I32)
     vq_wave_kernel<BT, H, int32_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int32_t*>(indptr),
                                                                  static_cast<const int32_t*>(indices), out);
@@ -521,12 +519,6 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     a.n_stripes = kXcds * a.stripes_per_xcd;
     grid = (unsigned)cus;
   }
-  hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_pipe_kernel<BT, int32_t>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_pipe_kernel<BT, int64_t>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e1 != hipSuccess || e2 != hipSuccess)
-    return fail((int)(e1 != hipSuccess ? e1 : e2), "%s: cannot reserve %zu B of LDS", what, lds);
   const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 0.0;
   // graphs whose 4-row mini-blocks mostly fit the 64-edge staging take the wave-granular kernel
   if (avg_deg * kWRows <= 60.0) {
@@ -536,6 +528,10 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     if (a.feat_dim % 8 == 0) return launch_wave<BT, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
     return launch_wave<BT, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
   }
+  const void* kern = idx_dtype == F2CGT_DT_I32 ? reinterpret_cast<const void*>(vq_pipe_kernel<BT, int32_t>)
+                                               : reinterpret_cast<const void*>(vq_pipe_kernel<BT, int64_t>);
+  const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return fail((int)e, "%s: cannot reserve %zu B of LDS", what, lds);
   if (idx_dtype == F2CGT_DT_I32)
     vq_pipe_kernel<BT, int32_t><<<grid, kThreads, lds, st>>>(a, static_cast<const int32_t*>(indptr),
                                                             static_cast<const int32_t*>(indices), out);

@@ -546,6 +546,29 @@ def test_kmeans_predict_exact_ties_pick_first():
     assert np.array_equal(got_c, oc.kmeans_predict(c, c, "l2")[0])
 
 
+@pytest.mark.parametrize("metric", ["l2", "cosine"])
+def test_kmeans_predict_when_the_expanded_form_cancels(metric):
+    # a common offset makes |x|^2 and |c|^2 about 1e4 times the distances between them, so most rows
+    # fall inside the rounding bound of the matrix-core scores and take the exact re-evaluation
+    rng = np.random.default_rng(21)
+    x = (rng.standard_normal((6000, 32)) * 0.3 + 17.0).astype(np.float32)
+    c = (rng.standard_normal((256, 32)) * 0.3 + 17.0).astype(np.float32)
+    want, near = oc.kmeans_predict(x, c, metric)
+    got = host(capi.kmeans_predict(dev(x), dev(c), metric))
+    assert np.array_equal(got[~near], want[~near])
+    assert near.mean() < 0.05
+
+
+def test_kmeans_predict_cosine_with_a_centre_without_direction():
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((3000, 32)).astype(np.float32)
+    c = rng.standard_normal((256, 32)).astype(np.float32)
+    c[17] = 0.0
+    want, near = oc.kmeans_predict(x, c, "cosine")
+    got = host(capi.kmeans_predict(dev(x), dev(c), "cosine"))
+    assert np.array_equal(got[~near], want[~near])
+
+
 # ---- the F2CGTLib module (same kernels through the pybind shim) ------------------------------------
 def test_module_surface_end_to_end():
     import f2cgt_amd
