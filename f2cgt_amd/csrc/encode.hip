@@ -524,21 +524,47 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
   float* xs = reinterpret_cast<float*>(cmax_bits + 4) + (threadIdx.x >> 6) * 16 * S;   // one row of x per wave
   const bool cosine = metric == F2CGT_METRIC_COSINE;
   if (threadIdx.x == 0) { cmax_bits[0] = 0; cmax_bits[1] = 0; }
+  // Staging works on items (centre, chunk of 8 dimensions) = one half-operand, four items per
+  // thread with their loads issued together: first the sums of squares of the chunks, then, once
+  // the norms are known, the pieces.  Dimensions from k on and centres from n on read as zeros.
+  const bool cvec = (k % 8 == 0) && ((reinterpret_cast<uintptr_t>(centers) & 15) == 0);
+  auto load8 = [&](int c, int ch, float (&v)[8]) {
+    const bool in = c < n && 8 * ch < k;
+    const float* cr = centers + (in ? (int64_t)c * k + 8 * ch : 0);
+    if (cvec) {
+      const float4 u = reinterpret_cast<const float4*>(cr)[0], w = reinterpret_cast<const float4*>(cr)[1];
+      v[0] = u.x; v[1] = u.y; v[2] = u.z; v[3] = u.w; v[4] = w.x; v[5] = w.y; v[6] = w.z; v[7] = w.w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = in ? v[e] : 0.f;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = (in && 8 * ch + e < k) ? cr[e] : 0.f;
+    }
+  };
+  constexpr int kChunks = 2 * S;
+  const int n_items = n_pad * kChunks;
+  float* partial = reinterpret_cast<float*>(smem_raw);          // [n_pad][2 S], overwritten by the pieces later
+  for (int i0 = threadIdx.x; i0 < n_items; i0 += blockDim.x * 4) {
+    float v[4][8];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int it = i0 + u * blockDim.x;
+      load8(it < n_items ? it / kChunks : n, it % kChunks, v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int it = i0 + u * blockDim.x;
+      float sq = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sq += v[u][e] * v[u][e];
+      if (it < n_items) partial[it] = sq;
+    }
+  }
   __syncthreads();
   for (int jj = threadIdx.x; jj < n_pad; jj += blockDim.x) {
     float cn = 0.f;
-    if (jj < n) {
-      const float* cr = centers + (int64_t)jj * k;
-      int t = 0;
-      for (; t + 8 <= k; t += 8) {       // eight loads in flight, summed in dimension order
-        float v[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = cr[t + e];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) cn += v[e] * v[e];
-      }
-      for (; t < k; ++t) cn += cr[t] * cr[t];
-    }
+    for (int ch = 0; ch < kChunks; ++ch) cn += partial[jj * kChunks + ch];
     float sc = 1.f;
     if (cosine) {
       const float nr = sqrtf(cn);
@@ -550,23 +576,32 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
     if (jj < n && cosine && !(cn > 1e-12f)) atomicOr(cmax_bits + 1, 1);   // a centre without a direction
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < n_ct * S * 64; idx += blockDim.x) {
-    const int ln = idx & 63, ts = idx >> 6;
-    const int st = ts % S, tile = ts / S;
-    const int c = tile * 32 + (ln & 31);
-    const int kk0 = 16 * st + 8 * (ln >> 5);
-    bf16x8 p0, p1, p2;
+  for (int i0 = threadIdx.x; i0 < n_items; i0 += blockDim.x * 4) {
+    float v[4][8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float v = 0.f;
-      if (c < n && kk0 + e < k) v = centers[(int64_t)c * k + kk0 + e] * inv[c];
-      __bf16 a0, a1, a2;
-      split3(v, a0, a1, a2);
-      p0[e] = a0; p1[e] = a1; p2[e] = a2;
+    for (int u = 0; u < 4; ++u) {
+      const int it = i0 + u * blockDim.x;
+      load8(it < n_items ? it / kChunks : n, it % kChunks, v[u]);
     }
-    ap[(0 * n_ct + tile) * S * 64 + st * 64 + ln] = p0;
-    ap[(1 * n_ct + tile) * S * 64 + st * 64 + ln] = p1;
-    ap[(2 * n_ct + tile) * S * 64 + st * 64 + ln] = p2;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int it = i0 + u * blockDim.x;
+      if (it >= n_items) break;
+      const int c = it / kChunks, ch = it % kChunks;
+      const float sc = inv[c];
+      bf16x8 p0, p1, p2;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        __bf16 a0, a1, a2;
+        split3(v[u][e] * sc, a0, a1, a2);
+        p0[e] = a0; p1[e] = a1; p2[e] = a2;
+      }
+      // chunk ch of centre c is lane (c % 32) + 32 (ch % 2) of step ch / 2 of tile c / 32
+      const int at = ((c >> 5) * S + (ch >> 1)) * 64 + (ch & 1) * 32 + (c & 31);
+      ap[at] = p0;
+      ap[n_ct * S * 64 + at] = p1;
+      ap[2 * n_ct * S * 64 + at] = p2;
+    }
   }
   __syncthreads();
   const float cmax = __int_as_float(cmax_bits[0]);
@@ -599,13 +634,12 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
         const int kk0 = 16 * st + 8 * g;
         float q[8];
         if (vec4) {
-          float4 u = make_float4(0.f, 0.f, 0.f, 0.f), w = u;
-          if (valid && kk0 < k) {
-            const float4* xp4 = reinterpret_cast<const float4*>(x + row * k + kk0);
-            u = xp4[0];
-            w = xp4[1];
-          }
+          const bool in = valid && kk0 < k;                   // loads always issued, from row 0 when idle
+          const float4* xp4 = reinterpret_cast<const float4*>(x + (in ? row * k + kk0 : 0));
+          const float4 u = xp4[0], w = xp4[1];
           q[0] = u.x; q[1] = u.y; q[2] = u.z; q[3] = u.w; q[4] = w.x; q[5] = w.y; q[6] = w.z; q[7] = w.w;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) q[e] = in ? q[e] : 0.f;
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e) q[e] = (valid && kk0 + e < k) ? x[row * k + kk0 + e] : 0.f;
