@@ -523,7 +523,7 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
   int* cmax_bits = reinterpret_cast<int*>(inv + n_pad);
   float* xs = reinterpret_cast<float*>(cmax_bits + 4) + (threadIdx.x >> 6) * 16 * S;   // one row of x per wave
   const bool cosine = metric == F2CGT_METRIC_COSINE;
-  if (threadIdx.x == 0) { cmax_bits[0] = 0; cmax_bits[1] = 0; }
+  if (threadIdx.x == 0) { cmax_bits[0] = 0; cmax_bits[1] = 0; cmax_bits[2] = 0; }
   // Staging works on items (centre, chunk of 8 dimensions) = one half-operand, four items per
   // thread with their loads issued together: first the sums of squares of the chunks, then, once
   // the norms are known, the pieces.  Dimensions from k on and centres from n on read as zeros.
@@ -619,9 +619,16 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
   const float unit = 5.9604645e-8f * (float)(2 * (68 * S + k + 8));
   const float xscale = cosine ? -1.f : -2.f;
   const bool vec4 = (k % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
-  const int64_t group0 = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int64_t gstride = (int64_t)gridDim.x * 4;
-  for (int64_t grp = group0; grp < n_groups; grp += gstride) {
+  // A workgroup owns a contiguous share of the row groups and its four waves draw from it through
+  // a counter in LDS: a wave held up by exact re-evaluations simply takes fewer groups.
+  const int64_t per_wg = (n_groups + gridDim.x - 1) / gridDim.x;
+  const int64_t wg_lo = (int64_t)blockIdx.x * per_wg;
+  const int64_t wg_hi = wg_lo + per_wg < n_groups ? wg_lo + per_wg : n_groups;
+  for (;;) {
+    int draw = 0;
+    if (lane == 0) draw = atomicAdd(cmax_bits + 2, 1);
+    const int64_t grp = wg_lo + __builtin_amdgcn_readfirstlane(draw);
+    if (grp >= wg_hi) break;
     bf16x8 xp[NB][S][3];
     float xn[NB];
 #pragma unroll
