@@ -264,9 +264,10 @@ __global__ __launch_bounds__(kThreads) void vq_pipe_kernel(VqArgs a, const Idx* 
 // pipeline, with wave-private staging in LDS.  After the codebook is staged no workgroup barrier
 // is left: a wave that waits for its loads does not hold the other fifteen, and the LDS
 // operations of one wave execute in order, so its own stage hand-overs need no synchronisation.
-// A wave owns chunks of 48 consecutive destination rows and walks them as twelve 4-row
-// mini-blocks (<= 64 edges: one edge per lane in the I and C stages; larger ones are summed
-// straight from HBM):
+// A wave owns chunks of 48 consecutive destination rows and walks them as mini-blocks of RPM rows
+// (<= 64 edges: one edge per lane in the I and C stages; larger ones are summed straight from
+// HBM).  RPM follows the average degree: 4 up to 15 edges per row, and 2 or 1 above, where the
+// lane groups left over in a pass share a row's edges and add their partial sums:
 //     P  the 49 row offsets of a chunk     one load per chunk, issued while the previous chunk
 //                                          starts, parked half a chunk later (two LDS buffers)
 //     I  source id of edge `lane`          issued two mini-blocks ahead, stays in the register
@@ -282,12 +283,13 @@ constexpr int kWPtr = 56;                     // ints per offset buffer: [0..48]
 
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
-template <int BT, int H, typename Idx>
+template <int BT, int H, int RPM, typename Idx>
 __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* __restrict__ indptr,
                                                            const Idx* __restrict__ indices,
                                                            float* __restrict__ out) {
   using CW = typename code_word<BT>::type;
   constexpr int kWaves = kThreads / 64;
+  constexpr int kMini = kWChunk / RPM;          // mini-blocks (RPM rows each) per chunk
   extern __shared__ __align__(16) unsigned char smem[];
   float* s_cb = reinterpret_cast<float*>(smem);
   const int wave = uni((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
@@ -317,7 +319,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   if (chunk_row0 >= a.R) return;
   const int64_t row_end = chunk_row0 + rows_per_wave < a.R ? chunk_row0 + rows_per_wave : a.R;
   const int64_t n_chunks = (row_end - chunk_row0 + kWChunk - 1) / kWChunk;
-  const int64_t n_mini = (row_end - chunk_row0 + kWRows - 1) / kWRows;
+  const int64_t n_mini = (row_end - chunk_row0 + RPM - 1) / RPM;
 
   // lanes per row: 32 lanes with one float4 each (H == 1) or 16 lanes with a whole 8-column code
   // each (H == 2); the wave then works on 2 or 4 rows at a time
@@ -352,11 +354,11 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   };
   // bounds of mini-block g: first edge (relative to the chunk's e0) and edge count
   auto bounds = [&](int64_t g, int& eb, int& ne) {
-    const int64_t c = g / kWMini;
-    const int m = (int)(g - c * kWMini);
+    const int64_t c = g / kMini;
+    const int m = (int)(g - c * kMini);
     const int* buf = s_ptr + (int)(c & 1) * kWPtr;
-    eb = uni(buf[m * kWRows]);
-    const int ee = uni(buf[m * kWRows + kWRows]);
+    eb = uni(buf[m * RPM]);
+    const int ee = uni(buf[m * RPM + RPM]);
     ne = ee - eb;
     ne = ne < 0 ? 0 : ne;
   };
@@ -375,10 +377,10 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   for (int64_t g = -2; g < n_mini; ++g) {
     // chunk-level P stage, driven by the position of g inside its chunk
     if (g >= 0) {
-      const int64_t c = g / kWMini;
-      const int m = (int)(g - c * kWMini);
+      const int64_t c = g / kMini;
+      const int m = (int)(g - c * kMini);
       if (m == 0 && c + 1 < n_chunks) issue_P(c + 1);
-      if (m == kWMini / 2 && c + 1 < n_chunks) park_P(c + 1);
+      if (m == kMini / 2 && c + 1 < n_chunks) park_P(c + 1);
     }
     // park C(g)
     if (g >= 0 && ne0 <= kWEdges && lane < ne0) *reinterpret_cast<CW*>(s_codes + lane * BT) = Creg;
@@ -396,7 +398,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       int64_t e0 = 0;
       if (v) {
         bounds(g + 2, eb2, ne2);
-        e0 = chunk_e0((g + 2) / kWMini);
+        e0 = chunk_e0((g + 2) / kMini);
       }
       const bool on = v && ne2 <= kWEdges && lane < ne2;
       const Idx* src = on ? indices + e0 + eb2 + lane : indptr;
@@ -404,17 +406,22 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     }
     // compute mini-block g
     if (g >= 0 && col_on) {
-      const int64_t c = g / kWMini;
-      const int m = (int)(g - c * kWMini);
-      const int* buf = s_ptr + (int)(c & 1) * kWPtr + m * kWRows;
-      const int64_t row0 = chunk_row0 + c * chunk_stride + m * kWRows;
+      const int64_t c = g / kMini;
+      const int m = (int)(g - c * kMini);
+      const int* buf = s_ptr + (int)(c & 1) * kWPtr + m * RPM;
+      const int64_t row0 = chunk_row0 + c * chunk_stride + m * RPM;
       const int64_t left = row_end - row0;
-      const int nr = (int)(left < kWRows ? left : kWRows);
+      const int nr = (int)(left < RPM ? left : RPM);
       const bool staged = ne0 <= kWEdges;
       float* orow = out + row0 * (int64_t)a.feat_dim + tile * 128 + col0;
+      // RPM < 4 (H == 2 only): the 4 / RPM lane groups ("slots") of a pass share a row, slot s of
+      // them takes the row's edges s, s + SPR, ... and the partial sums are added across the slots
+      constexpr int SPR = kRowsPerPass / (RPM < kRowsPerPass ? RPM : kRowsPerPass);
+      constexpr int kPasses = RPM * SPR / kRowsPerPass;
 #pragma unroll
-      for (int pass = 0; pass < kWRows / kRowsPerPass; ++pass) {
-        const int row = pass * kRowsPerPass + half;
+      for (int pass = 0; pass < kPasses; ++pass) {
+        const int slot = pass * kRowsPerPass + half;
+        const int row = slot / SPR, sub = slot % SPR;
         if (row >= nr) continue;
         int rb = buf[row] - eb0, re = buf[row + 1] - eb0;
         float acc[H][4];
@@ -425,14 +432,15 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
           rb = rb < 0 ? 0 : (rb > ne0 ? ne0 : rb);
           re = re < 0 ? 0 : (re > ne0 ? ne0 : re);
           n = re - rb;
-          const unsigned char* cp = s_codes + rb * BT + byte_idx;
+          const int ns = n > sub ? (n - sub + SPR - 1) / SPR : 0;   // edges of this slot
+          const unsigned char* cp = s_codes + (rb + sub) * BT + byte_idx;
           int k = 0;
-          for (; k + kGroup <= n; k += kGroup) {
+          for (; k + kGroup <= ns; k += kGroup) {
             uint32_t code[kGroup];
             float4 x[kGroup][H];
 #pragma unroll
-            for (int u = 0; u < kGroup; ++u) code[u] = cp[u * BT];
-            cp += kGroup * BT;
+            for (int u = 0; u < kGroup; ++u) code[u] = cp[u * SPR * BT];
+            cp += kGroup * SPR * BT;
 #pragma unroll
             for (int u = 0; u < kGroup; ++u)
 #pragma unroll
@@ -444,9 +452,9 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
                 acc[h][0] += x[u][h].x; acc[h][1] += x[u][h].y; acc[h][2] += x[u][h].z; acc[h][3] += x[u][h].w;
               }
           }
-          for (; k < n; ++k) {
+          for (; k < ns; ++k) {
             const uint32_t code = *cp;
-            cp += BT;
+            cp += SPR * BT;
 #pragma unroll
             for (int h = 0; h < H; ++h) {
               const float4 x = *reinterpret_cast<const float4*>(cbp + code * 128 + h * 64);
@@ -456,7 +464,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
         } else {
           n = re - rb;
           const int64_t e0 = chunk_e0(c) + eb0;
-          for (int k = 0; k < n; ++k) {
+          for (int k = sub; k < n; k += SPR) {
             const int64_t id = clamp_idx(indices[e0 + rb + k], a.N);
             const uint32_t code = a.codes[id * a.n_cb + tile * BT + byte_idx];
 #pragma unroll
@@ -465,6 +473,16 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
               acc[h][0] += x.x; acc[h][1] += x.y; acc[h][2] += x.z; acc[h][3] += x.w;
             }
           }
+        }
+        if (SPR > 1) {
+#pragma unroll
+          for (int h = 0; h < H; ++h)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+              acc[h][t] += __shfl_xor(acc[h][t], kLanesPerRow);
+              if (SPR > 2) acc[h][t] += __shfl_xor(acc[h][t], 2 * kLanesPerRow);
+            }
+          if (sub != 0) continue;
         }
         if (n > 1) {
           const float d = (float)n;
@@ -485,19 +503,19 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   }
 }
 
-template <int BT, int H>
+template <int BT, int H, int RPM>
 int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
                 const char* what, unsigned grid, size_t wlds) {
-  const void* kern = idx_dtype == F2CGT_DT_I32 ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, int32_t>)
-                                               : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, int64_t>);
+  const void* kern = idx_dtype == F2CGT_DT_I32 ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t>)
+                                               : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t>);
   const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
   if (e != hipSuccess) return fail((int)e, "%s: cannot reserve %zu B of LDS", what, wlds);
   if (idx_dtype == F2CGT_DT_I32)
-    vq_wave_kernel<BT, H, int32_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int32_t*>(indptr),
-                                                                 static_cast<const int32_t*>(indices), out);
+    vq_wave_kernel<BT, H, RPM, int32_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int32_t*>(indptr),
+                                                                      static_cast<const int32_t*>(indices), out);
   else
-    vq_wave_kernel<BT, H, int64_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int64_t*>(indptr),
-                                                                 static_cast<const int64_t*>(indices), out);
+    vq_wave_kernel<BT, H, RPM, int64_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int64_t*>(indptr),
+                                                                      static_cast<const int64_t*>(indices), out);
   return launch_status(what);
 }
 
@@ -520,13 +538,18 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     grid = (unsigned)cus;
   }
   const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 0.0;
-  // graphs whose 4-row mini-blocks mostly fit the 64-edge staging take the wave-granular kernel
-  if (avg_deg * kWRows <= 60.0) {
-    const size_t wlds = (size_t)a.K * 128 * 4 + (size_t)(kThreads / 64) * kWEdges * BT +
-                        (size_t)(kThreads / 64) * 2 * kWPtr * 4;
-    // whole 8-column groups in every tile: one lane per group (two float4 per edge)
-    if (a.feat_dim % 8 == 0) return launch_wave<BT, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
-    return launch_wave<BT, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+  // Graphs whose mini-blocks mostly fit the 64-edge staging take the wave-granular kernel: 4-row
+  // mini-blocks up to 15 edges per row, and, with whole 8-column groups in every tile (one lane
+  // per group, two float4 per edge), 2-row and 1-row mini-blocks up to 30 and 60 edges per row
+  // (larger mini-blocks for sparse rows were tried and were slower than 4-row ones).
+  const size_t wlds = (size_t)a.K * 128 * 4 + (size_t)(kThreads / 64) * kWEdges * BT +
+                      (size_t)(kThreads / 64) * 2 * kWPtr * 4;
+  if (a.feat_dim % 8 == 0) {
+    if (avg_deg <= 15.0) return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    if (avg_deg <= 30.0) return launch_wave<BT, 2, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    if (avg_deg <= 60.0) return launch_wave<BT, 2, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+  } else if (avg_deg <= 15.0) {
+    return launch_wave<BT, 1, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
   }
   const void* kern = idx_dtype == F2CGT_DT_I32 ? reinterpret_cast<const void*>(vq_pipe_kernel<BT, int32_t>)
                                                : reinterpret_cast<const void*>(vq_pipe_kernel<BT, int64_t>);
