@@ -720,10 +720,13 @@ extern "C" int f2cgt_sq_affine_decompress_spmm_csr(const uint8_t* codes, const f
   F2CGT_REQUIRE(params && (num_edges == 0 || codes), F2CGT_E_INVALID, "%s: null buffer", what);
   hipStream_t st = as_stream(stream);
   const int D = (int)feat_dim;
-  if (sq_affine_acc_eligible(codes, out, num_src_rows, src_dim, D, target_bits))
+  // rows of more than ~250 edges overflow the row-block kernels' edge staging; the
+  // per-row skeleton, whose cost per row is amortised over a long row, takes those graphs
+  const bool long_rows = num_edges > 200 * num_rows;
+  if (!long_rows && sq_affine_acc_eligible(codes, out, num_src_rows, src_dim, D, target_bits))
     return sq_affine_acc_run(codes, params, param_stride, indptr, indices, idx_dtype, out, num_rows,
                               num_edges, num_src_rows, src_dim, D, target_bits, st, what);
-  if (sq_block_eligible(codes, out, num_src_rows, src_dim, D, target_bits, 0))
+  if (!long_rows && sq_block_eligible(codes, out, num_src_rows, src_dim, D, target_bits, 0))
     return sq_block_run(true, codes, params, param_stride, 1, 1, indptr, indices, idx_dtype, out, num_rows,
                         num_edges, num_src_rows, src_dim, D, target_bits, st, what);
   switch (target_bits) {
