@@ -27,6 +27,11 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+// Absolute part of the near-tie bound: the matrix core flushes products (and, for the split form,
+// piece products 2^-9 and 2^-18 of the full one) that fall below the smallest normal fp32 number,
+// which the relative bound does not see.  A few hundred such terms stay below this.
+constexpr float kTinyGap = 1e-33f;
+
 // ---- exact assignment of one row by a whole wave (fp64) ------------------------------
 __device__ int exact_argmin_row(const float* __restrict__ xrow, const float* __restrict__ centers,
                                 int n, int k, int metric, int lane) {
@@ -267,7 +272,8 @@ __global__ __launch_bounds__(256) void predict_mfma_kernel(const float* __restri
       }
     }
     const float scale = cosine ? sqrtf(xn) : xn + cmax;
-    const bool near_tie = valid && h == 0 && !((second - best) > unit * scale);
+    // + kTinyGap: products below the smallest normal number are flushed inside the matrix core
+    const bool near_tie = valid && h == 0 && !((second - best) > unit * scale + kTinyGap);
     uint64_t todo = __ballot(near_tie);
     while (todo) {
       const int src = __ffsll((unsigned long long)todo) - 1;
@@ -731,7 +737,7 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
       }
       const float scale = cosine ? sqrtf(xn[b]) : xn[b] + cmax;
       besti[b] = bi;
-      todo[b] = __ballot(valid && g == 0 && !((sd - bs) > unit * scale));
+      todo[b] = __ballot(valid && g == 0 && !((sd - bs) > unit * scale + kTinyGap));
     }
     // exact re-evaluation of the flagged rows: one copy of the code, whichever tile the row is in
 #pragma nounroll

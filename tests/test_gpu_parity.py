@@ -585,6 +585,18 @@ def test_kmeans_predict_when_the_expanded_form_cancels(metric):
     assert near.mean() < 0.05
 
 
+@pytest.mark.parametrize("scale", [1e-19, 3e-17, 1e15])
+def test_kmeans_predict_extreme_magnitudes(scale):
+    # tiny values: the second-order piece products (and at 1e-19 the products themselves) fall below
+    # the smallest normal fp32 number inside the matrix core; huge ones: squares near 1e32
+    rng = np.random.default_rng(23)
+    x = (rng.standard_normal((3000, 32)) * scale).astype(np.float32)
+    c = (rng.standard_normal((256, 32)) * scale).astype(np.float32)
+    want, near = oc.kmeans_predict(x, c, "l2")
+    got = host(capi.kmeans_predict(dev(x), dev(c), "l2"))
+    assert np.array_equal(got[~near], want[~near])
+
+
 def test_kmeans_predict_cosine_with_a_centre_without_direction():
     rng = np.random.default_rng(22)
     x = rng.standard_normal((3000, 32)).astype(np.float32)
