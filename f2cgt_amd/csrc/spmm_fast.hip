@@ -373,9 +373,30 @@ __device__ __forceinline__ void acc_gather(const AccArgs& a, uint32_t* s_acc, co
 
 // Means of the rows [rb, rb + nr) of the block from the accumulator rows [0, nr): a lane keeps
 // one float4 column group (its parameters in registers) and walks the rows.
+// min / scale of a lane's first column group, fetched when the kernel starts: the loads would
+// otherwise sit behind the last barrier of a block, one more round trip in its dependent chain.
+struct FinParams {
+  float mn[4], sc[4];
+};
+
+__device__ __forceinline__ FinParams acc_fin_params(const AccArgs& a) {
+  FinParams p;
+  const int t = threadIdx.x;
+  const int g = (int)(((uint32_t)t * a.fin_magic) >> 16);
+  const int l = t - g * a.fin_group;
+  const int c4 = (g < a.fin_slots && l < a.f4_per_row) ? l : 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    p.mn[i] = a.params[c4 * 4 + i];
+    p.sc[i] = a.params[a.param_stride + c4 * 4 + i];
+  }
+  return p;
+}
+
 template <int TB, int BITS, int NW>
-__device__ __forceinline__ void acc_finalize(const AccArgs& a, const uint32_t* s_acc, const float* s_rdeg,
-                                             int64_t row0, int rb, int nr, int pitch, float* __restrict__ out) {
+__device__ __forceinline__ void acc_finalize(const AccArgs& a, const FinParams& first, const uint32_t* s_acc,
+                                             const float* s_rdeg, int64_t row0, int rb, int nr, int pitch,
+                                             float* __restrict__ out) {
   const int t = threadIdx.x;
   const int lanes = a.lanes;
   const int g = (int)(((uint32_t)t * a.fin_magic) >> 16);
@@ -385,8 +406,15 @@ __device__ __forceinline__ void acc_finalize(const AccArgs& a, const uint32_t* s
     float mn[4], sc[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      mn[i] = a.params[c4 * 4 + i];
-      sc[i] = a.params[a.param_stride + c4 * 4 + i];
+      mn[i] = first.mn[i];
+      sc[i] = first.sc[i];
+    }
+    if (c4 != l) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        mn[i] = a.params[c4 * 4 + i];
+        sc[i] = a.params[a.param_stride + c4 * 4 + i];
+      }
     }
     const int d = BITS == 4 ? (c4 >> 1) : c4;     // code dword that holds these 4 columns
     const int fsh = BITS == 4 ? (c4 & 1) * 16 : 0;
@@ -428,8 +456,8 @@ __device__ __forceinline__ void acc_finalize(const AccArgs& a, const uint32_t* s
 
 // All rows of the block, `sub` rows at a time through the accumulators.
 template <int TB, int BITS, int NW, typename Idx>
-__device__ __forceinline__ void acc_block(const AccArgs& a, uint32_t* s_acc, const int* s_ptr, const float* s_rdeg,
-                                          uint2* s_edge, int64_t e0, int64_t row0, int nrows,
+__device__ __forceinline__ void acc_block(const AccArgs& a, const FinParams& first, uint32_t* s_acc, const int* s_ptr,
+                                          const float* s_rdeg, uint2* s_edge, int64_t e0, int64_t row0, int nrows,
                                           const Idx* __restrict__ indices, float* __restrict__ out) {
   const int pitch = NW == 4 ? a.pitch_w : a.pitch_n;
   const int sub = NW == 4 ? a.sub_rows >> 1 : a.sub_rows;
@@ -443,7 +471,7 @@ __device__ __forceinline__ void acc_block(const AccArgs& a, uint32_t* s_acc, con
       const int nr = (nrows - sb) < sub ? (nrows - sb) : sub;
       acc_gather<TB, BITS, NW>(a, s_acc, s_edge, s_ptr[sb], s_ptr[sb + nr], sb, pitch);
       __syncthreads();
-      acc_finalize<TB, BITS, NW>(a, s_acc, s_rdeg, row0, sb, nr, pitch, out);
+      acc_finalize<TB, BITS, NW>(a, first, s_acc, s_rdeg, row0, sb, nr, pitch, out);
       if (sb + sub < nrows) {
         __syncthreads();
         acc_zero<TB>(s_acc, sub * pitch);
@@ -464,7 +492,7 @@ __device__ __forceinline__ void acc_block(const AccArgs& a, uint32_t* s_acc, con
         acc_gather<TB, BITS, NW>(a, s_acc, s_edge, 0, nb, 0, pitch);
       }
       __syncthreads();
-      acc_finalize<TB, BITS, NW>(a, s_acc, s_rdeg, row0, sb, nr, pitch, out);
+      acc_finalize<TB, BITS, NW>(a, first, s_acc, s_rdeg, row0, sb, nr, pitch, out);
     }
   }
 }
@@ -485,6 +513,7 @@ __global__ __launch_bounds__(TB) void sq_affine_acc_kernel(AccArgs a, const Idx*
   const int t = threadIdx.x;
   const int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block;
   const int nrows = (int)((a.R - row0) < a.rows_per_block ? (a.R - row0) : a.rows_per_block);
+  const FinParams first = acc_fin_params(a);
   int64_t e0 = (int64_t)indptr[row0];
   e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
   uint32_t level = 0;
@@ -517,9 +546,9 @@ __global__ __launch_bounds__(TB) void sq_affine_acc_kernel(AccArgs a, const Idx*
     return;
   }
   if (BITS == 4 && (block_level & 1u))
-    acc_block<TB, BITS, 4, Idx>(a, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
+    acc_block<TB, BITS, 4, Idx>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
   else
-    acc_block<TB, BITS, 2, Idx>(a, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
+    acc_block<TB, BITS, 2, Idx>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
 }
 
 template <int TB, int BITS>
