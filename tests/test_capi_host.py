@@ -152,3 +152,19 @@ def test_small_workloads_are_consistent():
     assert (m[:200] == np.arange(200)).all() and m[200] == -1 and m[-1] == -(4000 - 200)
     assert wl4["sq_codes"].shape[0] == 200 and wl4["vq_codes"].shape[0] == 3800
     assert 0 < wl4["hot_edges"] <= wl4["E"]
+
+
+def test_bench_refuses_more_than_one_gpu_and_needs_a_gpu():
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    two = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True,
+                         text=True, timeout=120)
+    assert two.returncode != 0
+    assert "one GPU" in (two.stdout + two.stderr)
+    import torch
+    if not torch.cuda.is_available():
+        one = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--steps", "1", "--warmup", "0"],
+                             capture_output=True, text=True, timeout=300)
+        assert one.returncode != 0          # no CPU stand-in for the measured path
+        assert one.stdout.strip() == ""     # and no result line
