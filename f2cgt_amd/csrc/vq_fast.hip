@@ -35,6 +35,7 @@ struct VqArgs {
   int n_cb, K, w, feat_dim;
   int n_tiles, n_stripes;
   int stripes_per_xcd;  // > 0: the column tiles of a stripe share one XCD (see the kernel)
+  int dense_store;      // sparse rows: results go through LDS so that every store instruction is dense
 };
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -293,8 +294,9 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   extern __shared__ __align__(16) unsigned char smem[];
   float* s_cb = reinterpret_cast<float*>(smem);
   const int wave = uni((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
-  unsigned char* s_codes = smem + (size_t)a.K * 128 * 4 + (size_t)wave * kWEdges * BT;
-  int* s_ptr = reinterpret_cast<int*>(smem + (size_t)a.K * 128 * 4 + (size_t)kWaves * kWEdges * BT) + wave * 2 * kWPtr;
+  constexpr int kStage = kWEdges * BT > 1024 ? kWEdges * BT : 1024;   // code bytes of a mini-block, or 64 float4
+  unsigned char* s_codes = smem + (size_t)a.K * 128 * 4 + (size_t)wave * kStage;
+  int* s_ptr = reinterpret_cast<int*>(smem + (size_t)a.K * 128 * 4 + (size_t)kWaves * kStage) + wave * 2 * kWPtr;
 
   int tile, stripe;
   if (a.stripes_per_xcd > 0) {
@@ -405,7 +407,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       Ireg = (int64_t)*src;
     }
     // compute mini-block g
-    if (g >= 0 && col_on) {
+    if (g >= 0) {
       const int64_t c = g / kMini;
       const int m = (int)(g - c * kMini);
       const int* buf = s_ptr + (int)(c & 1) * kWPtr + m * RPM;
@@ -413,18 +415,14 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       const int64_t left = row_end - row0;
       const int nr = (int)(left < RPM ? left : RPM);
       const bool staged = ne0 <= kWEdges;
-      float* orow = out + row0 * (int64_t)a.feat_dim + tile * 128 + col0;
       // RPM < 4 (H == 2 only): the 4 / RPM lane groups ("slots") of a pass share a row, slot s of
       // them takes the row's edges s, s + SPR, ... and the partial sums are added across the slots
       constexpr int SPR = kRowsPerPass / (RPM < kRowsPerPass ? RPM : kRowsPerPass);
       constexpr int kPasses = RPM * SPR / kRowsPerPass;
-#pragma unroll
-      for (int pass = 0; pass < kPasses; ++pass) {
-        const int slot = pass * kRowsPerPass + half;
-        const int row = slot / SPR, sub = slot % SPR;
-        if (row >= nr) continue;
+      // sum of the codebook entries of this slot's share of row `row` (all of it when SPR == 1),
+      // in edge order; returns the row's edge count
+      auto row_sum = [&](int row, int sub, float (&acc)[H][4]) -> int {
         int rb = buf[row] - eb0, re = buf[row + 1] - eb0;
-        float acc[H][4];
 #pragma unroll
         for (int h = 0; h < H; ++h) acc[h][0] = acc[h][1] = acc[h][2] = acc[h][3] = 0.f;
         int n;
@@ -474,16 +472,9 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
             }
           }
         }
-        if (SPR > 1) {
-#pragma unroll
-          for (int h = 0; h < H; ++h)
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-              acc[h][t] += __shfl_xor(acc[h][t], kLanesPerRow);
-              if (SPR > 2) acc[h][t] += __shfl_xor(acc[h][t], 2 * kLanesPerRow);
-            }
-          if (sub != 0) continue;
-        }
+        return n;
+      };
+      auto mean = [&](int n, float (&acc)[H][4]) {
         if (n > 1) {
           const float d = (float)n;
           float r = __builtin_amdgcn_rcpf(d);
@@ -493,9 +484,62 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
 #pragma unroll
             for (int t = 0; t < 4; ++t) acc[h][t] = div_by(acc[h][t], d, r);
         }
+      };
+      if (H == 2 && SPR == 1 && kPasses == 1 && a.dense_store) {
+        // Four rows, sixteen lanes each.  A lane's result is 32 consecutive bytes, which as two
+        // stores would be 16 of every 32 bytes per instruction (half-written sectors on the way to
+        // memory).  The wave's 1 KB staging area, free once the edge loops are done, turns them
+        // around: the lanes of columns [64 p, 64 p + 64) write their two float4, every lane reads
+        // back the float4 of its own lane index, and each store instruction covers 256 contiguous
+        // bytes of every row.
+        const int row = half;
+        const bool active = col_on && row < nr;
+        float acc[H][4];
 #pragma unroll
-        for (int h = 0; h < H; ++h)
-          store_nt4(orow + (int64_t)row * a.feat_dim + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+        for (int h = 0; h < H; ++h) acc[h][0] = acc[h][1] = acc[h][2] = acc[h][3] = 0.f;
+        if (active) {
+          const int n = row_sum(row, 0, acc);
+          mean(n, acc);
+        }
+        float4* stg = reinterpret_cast<float4*>(s_codes);
+        float* obase = out + (row0 + row) * (int64_t)a.feat_dim + tile * 128;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          __builtin_amdgcn_wave_barrier();
+          if ((c4 >> 3) == p) {
+#pragma unroll
+            for (int h = 0; h < H; ++h)
+              stg[row * 16 + (c4 & 7) * 2 + h] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+          }
+          __builtin_amdgcn_wave_barrier();
+          const float4 v = stg[row * 16 + c4];
+          const int col = 64 * p + 4 * c4;
+          if (row < nr && col < tile_cols) store_nt4(obase + col, v.x, v.y, v.z, v.w);
+        }
+      } else if (col_on) {
+        float* orow = out + row0 * (int64_t)a.feat_dim + tile * 128 + col0;
+#pragma unroll
+        for (int pass = 0; pass < kPasses; ++pass) {
+          const int slot = pass * kRowsPerPass + half;
+          const int row = slot / SPR, sub = slot % SPR;
+          if (row >= nr) continue;
+          float acc[H][4];
+          const int n = row_sum(row, sub, acc);
+          if (SPR > 1) {
+#pragma unroll
+            for (int h = 0; h < H; ++h)
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                acc[h][t] += __shfl_xor(acc[h][t], kLanesPerRow);
+                if (SPR > 2) acc[h][t] += __shfl_xor(acc[h][t], 2 * kLanesPerRow);
+              }
+            if (sub != 0) continue;
+          }
+          mean(n, acc);
+#pragma unroll
+          for (int h = 0; h < H; ++h)
+            store_nt4(orow + (int64_t)row * a.feat_dim + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+        }
       }
     }
     eb0 = eb1; ne0 = ne1;
@@ -542,8 +586,11 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
   // mini-blocks up to 15 edges per row, and, with whole 8-column groups in every tile (one lane
   // per group, two float4 per edge), 2-row and 1-row mini-blocks up to 30 and 60 edges per row
   // (larger mini-blocks for sparse rows were tried and were slower than 4-row ones).
-  const size_t wlds = (size_t)a.K * 128 * 4 + (size_t)(kThreads / 64) * kWEdges * BT +
+  const size_t wlds = (size_t)a.K * 128 * 4 + (size_t)(kThreads / 64) * (kWEdges * BT > 1024 ? kWEdges * BT : 1024) +
                       (size_t)(kThreads / 64) * 2 * kWPtr * 4;
+  // with few edges per row the output dominates and its store pattern decides (fanout 2 at the C3
+  // shape: 845 -> 405 us); from about 8 edges per row the detour through LDS costs more than it saves
+  a.dense_store = avg_deg <= 8.0;
   if (a.feat_dim % 8 == 0) {
     if (avg_deg <= 15.0) return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
     if (avg_deg <= 30.0) return launch_wave<BT, 2, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
