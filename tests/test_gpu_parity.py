@@ -379,6 +379,21 @@ def test_fused_vq_shared_rows(fanout, rows):
     assert np.abs(got - exact).max() <= 1e-5 * np.abs(exact).max() + 1e-6
 
 
+@pytest.mark.parametrize("w,n_cb,feat_dim", [(8, 32, 200), (16, 16, 248), (32, 8, 160)])
+def test_fused_vq_sparse_rows_partial_tiles(w, n_cb, feat_dim):
+    # few edges per row: results are turned around in LDS before they are stored; the last column
+    # tile is partial, rows do not fill the last mini-block, some rows are empty
+    rng = np.random.default_rng(w + feat_dim)
+    N, rows = 4000, 2051
+    cb = rng.standard_normal((n_cb, 256, w)).astype(np.float32)
+    codes = rng.integers(0, 256, size=(N, n_cb), dtype=np.uint8)
+    indptr, indices = random_graph(rng, rows, N, 5)
+    got = host(capi.vq_decompress_spmm_csr(dev(codes), dev(cb), dev(indptr), dev(indices), feat_dim))
+    want = oc.vq_decompress_spmm_csr(codes, cb, indptr, indices, feat_dim)
+    assert got.shape == (rows, feat_dim)
+    assert np.array_equal(got, want)        # sequential edge order: bit-exact
+
+
 def test_fused_vq_int16_codes_big_codebook():
     rng = np.random.default_rng(5)
     cb = rng.standard_normal((2, 5000, 8)).astype(np.float32)   # 160 KB per slice: global path
