@@ -811,8 +811,10 @@ __global__ __launch_bounds__(256) void pairwise_kernel(const float* __restrict__
         float xv[8], yv[8];
         const float4 xa = *reinterpret_cast<const float4*>(&xs[c][ty * 8]);
         const float4 xb = *reinterpret_cast<const float4*>(&xs[c][ty * 8 + 4]);
-        const float4 ya = *reinterpret_cast<const float4*>(&ys[c][tx * 8]);
-        const float4 yb = *reinterpret_cast<const float4*>(&ys[c][tx * 8 + 4]);
+        // a thread's 8 y rows are two groups of 4, 64 apart, so that the 16 threads of a row of the
+        // tile store 256 contiguous bytes per instruction (8 consecutive ones would be 16 of every 32)
+        const float4 ya = *reinterpret_cast<const float4*>(&ys[c][tx * 4]);
+        const float4 yb = *reinterpret_cast<const float4*>(&ys[c][64 + tx * 4]);
         xv[0] = xa.x; xv[1] = xa.y; xv[2] = xa.z; xv[3] = xa.w; xv[4] = xb.x; xv[5] = xb.y; xv[6] = xb.z; xv[7] = xb.w;
         yv[0] = ya.x; yv[1] = ya.y; yv[2] = ya.z; yv[3] = ya.w; yv[4] = yb.x; yv[5] = yb.y; yv[6] = yb.z; yv[7] = yb.w;
         if (cosine) {
@@ -834,7 +836,7 @@ __global__ __launch_bounds__(256) void pairwise_kernel(const float* __restrict__
         }
       }
     }
-    const bool full = j0 + tx * 8 + 8 <= n && n % 4 == 0 && ((reinterpret_cast<uintptr_t>(dist) & 15) == 0);
+    const bool full = j0 + kTile <= n && n % 4 == 0 && ((reinterpret_cast<uintptr_t>(dist) & 15) == 0);
 #pragma unroll
     for (int a = 0; a < 8; ++a) {
       const int64_t i = i0 + ty * 8 + a;
@@ -849,14 +851,16 @@ __global__ __launch_bounds__(256) void pairwise_kernel(const float* __restrict__
           v[b] = 1.f - v[b] / den;
         }
       }
-      float* o = dist + i * n + j0 + tx * 8;
+      float* o = dist + i * n + j0 + tx * 4;       // columns j0 + 4 tx + (0..3) and + 64
       if (full) {
         store_nt4(o, v[0], v[1], v[2], v[3]);
-        store_nt4(o + 4, v[4], v[5], v[6], v[7]);
+        store_nt4(o + 64, v[4], v[5], v[6], v[7]);
       } else {
 #pragma unroll
-        for (int b = 0; b < 8; ++b)
-          if (j0 + tx * 8 + b < n) o[b] = v[b];
+        for (int b = 0; b < 8; ++b) {
+          const int col = tx * 4 + (b & 3) + (b >> 2) * 64;
+          if (j0 + col < n) dist[i * n + j0 + col] = v[b];
+        }
       }
     }
   }
