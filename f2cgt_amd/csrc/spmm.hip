@@ -355,7 +355,12 @@ struct HybridDec {
   int64_t n_sq, n_vq;
   int feat_dim, num_codebooks, K, w;
   const float* table;
+  bool in_lds;   // codebooks staged in LDS; larger ones are read through the caches
   __device__ void block_setup(unsigned char* smem, int, int) {
+    if (!in_lds) {
+      table = vq_codebooks;
+      return;
+    }
     float* l = reinterpret_cast<float*>(smem);
     const int total = num_codebooks * K * w;
     if ((total & 3) == 0) {
@@ -753,9 +758,10 @@ extern "C" int f2cgt_hybrid_decompress_spmm_csr(
   F2CGT_REQUIRE(param_stride >= feat_dim, F2CGT_E_INVALID, "%s: param_stride < feat_dim", what);
   F2CGT_REQUIRE(num_sq_rows >= 0 && num_vq_rows >= 0 && num_sq_rows + num_vq_rows > 0, F2CGT_E_INVALID,
                 "%s: both code tables are empty", what);
-  const int64_t lds = num_codebooks * K * width * 4;
-  F2CGT_REQUIRE(lds <= kLdsBudget, F2CGT_E_UNSUPPORTED, "%s: VQ codebook of %lld B exceeds the LDS budget",
-                what, (long long)lds);
+  F2CGT_REQUIRE(num_codebooks * K * width < (1ll << 28), F2CGT_E_UNSUPPORTED, "%s: VQ codebooks too large", what);
+  const int64_t cb_bytes = num_codebooks * K * width * 4;
+  const bool in_lds = cb_bytes <= kLdsBudget;
+  const int64_t lds = in_lds ? cb_bytes : 0;
   if (num_rows * feat_dim == 0) return 0;
   F2CGT_REQUIRE(row_map && sq_params && vq_codebooks, F2CGT_E_INVALID, "%s: null buffer", what);
   F2CGT_REQUIRE((num_sq_rows == 0 || sq_codes) && (num_vq_rows == 0 || vq_codes), F2CGT_E_INVALID,
@@ -771,13 +777,13 @@ extern "C" int f2cgt_hybrid_decompress_spmm_csr(
                           st, what);
   const bool a16 = aligned(out, 16) && aligned(vq_codebooks, 16);
   if (w % 4 == 0 && D >= 256 && aligned(sq_codes, 4) && a16) {
-    HybridDec<4> d{row_map, sq_codes, sq_params, param_stride, vq_codes, vq_codebooks, num_sq_rows, num_vq_rows, D, n_cb, k, w, nullptr};
+    HybridDec<4> d{row_map, sq_codes, sq_params, param_stride, vq_codes, vq_codebooks, num_sq_rows, num_vq_rows, D, n_cb, k, w, nullptr, in_lds};
     return run(d, indptr, indices, idx_dtype, out, num_rows, num_edges, num_src_rows, D, plan(num_rows, D, 1, 4, (size_t)lds), (size_t)lds, true, st, what);
   }
   if (w % 2 == 0 && aligned(sq_codes, 2) && a16) {
-    HybridDec<2> d{row_map, sq_codes, sq_params, param_stride, vq_codes, vq_codebooks, num_sq_rows, num_vq_rows, D, n_cb, k, w, nullptr};
+    HybridDec<2> d{row_map, sq_codes, sq_params, param_stride, vq_codes, vq_codebooks, num_sq_rows, num_vq_rows, D, n_cb, k, w, nullptr, in_lds};
     return run(d, indptr, indices, idx_dtype, out, num_rows, num_edges, num_src_rows, D, plan(num_rows, D, 1, 2, (size_t)lds), (size_t)lds, true, st, what);
   }
-  HybridDec<1> d{row_map, sq_codes, sq_params, param_stride, vq_codes, vq_codebooks, num_sq_rows, num_vq_rows, D, n_cb, k, w, nullptr};
+  HybridDec<1> d{row_map, sq_codes, sq_params, param_stride, vq_codes, vq_codebooks, num_sq_rows, num_vq_rows, D, n_cb, k, w, nullptr, in_lds};
   return run(d, indptr, indices, idx_dtype, out, num_rows, num_edges, num_src_rows, D, plan(num_rows, D, 1, 1, (size_t)lds), (size_t)lds, false, st, what);
 }

@@ -1,0 +1,150 @@
+"""Seeded random shapes through every fused operator and the streaming ones: the fast kernels are
+chosen by shape (column count, bits, degree, index type, alignment), so many small, odd shapes are
+what finds a path that a hand-picked list misses.  Same bars as the parity tests."""
+import numpy as np
+import pytest
+import torch
+
+import f2cgt_oracle as oc
+from f2cgt_amd import capi
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-5
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def graph(rng, rows, n_src, idx):
+    kind = rng.integers(0, 4)
+    if kind == 0:
+        deg = rng.integers(0, 4, size=rows)                          # sparse, with empty rows
+    elif kind == 1:
+        deg = np.full(rows, int(rng.integers(1, 40)))                # fixed fanout
+    elif kind == 2:
+        deg = np.minimum(rng.zipf(1.8, size=rows), 300)              # heavy tail
+    else:
+        deg = rng.integers(0, int(rng.integers(2, 90)), size=rows)
+    indptr = np.zeros(rows + 1, dtype=idx)
+    indptr[1:] = np.cumsum(deg)
+    indices = rng.integers(0, n_src, size=int(indptr[-1])).astype(idx)
+    return indptr, indices
+
+
+def close(got, want):
+    scale = float(np.abs(want).max()) if want.size else 1.0
+    return np.allclose(got, want, rtol=RTOL, atol=RTOL * scale)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_fused_affine_sq_random_shape(seed):
+    rng = np.random.default_rng(1000 + seed)
+    bits = int(rng.choice([1, 2, 4, 8]))
+    D = int(rng.choice([4, 8, 12, 20, 36, 64, 100, 128, 132, 256, 300]))
+    N, rows = int(rng.integers(50, 3000)), int(rng.integers(1, 1500))
+    idx = rng.choice([np.int32, np.int64])
+    x = rng.standard_normal((N, D)).astype(np.float32) * rng.uniform(0.1, 10)
+    params = oc.sq_affine_params(x, bits)
+    codes = oc.sq_affine_compress(x, params, bits)
+    indptr, indices = graph(rng, rows, N, idx)
+    got = host(capi.sq_affine_decompress_spmm_csr(dev(codes), dev(params), dev(indptr), dev(indices), bits, D))
+    want = oc.sq_affine_decompress_spmm_csr(codes, params, indptr.astype(np.int64), indices.astype(np.int64), bits, D)
+    assert got.shape == want.shape
+    assert close(got, want)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_fused_log_sq_random_shape(seed):
+    rng = np.random.default_rng(2000 + seed)
+    bits = int(rng.choice([1, 2, 4, 8, 16]))
+    per = max(1, 8 // bits)
+    D = int(rng.choice([8, 16, 24, 40, 64, 100, 128, 200]))
+    slices = [s for s in (8, 16, 40, 64, D) if s % per == 0 and s <= D]
+    cs = int(rng.choice(slices))
+    N, rows = int(rng.integers(50, 2500)), int(rng.integers(1, 1200))
+    idx = rng.choice([np.int32, np.int64])
+    x = rng.uniform(-3, 3, size=(N, D)).astype(np.float32)
+    cbs = np.stack([oc.sq_codebook(x[:, s:s + cs]) for s in range(0, D, cs)])
+    store = oc.sq_codes_to_storage(oc.sq_compress(x, cbs, bits, cs), bits)
+    indptr, indices = graph(rng, rows, N, idx)
+    got = host(capi.sq_decompress_spmm_csr(dev(store), dev(cbs), dev(indptr), dev(indices), bits, cs, D))
+    raw = store.view(np.uint8) if store.dtype == np.int8 and bits < 8 else store
+    want = oc.sq_decompress_spmm_csr(raw, cbs, indptr.astype(np.int64), indices.astype(np.int64), bits, cs, D)
+    assert close(got, want)
+    # and the standalone decode of the same table, bit for bit
+    dec = host(capi.sq_decompress(dev(store), dev(cbs), bits, cs, D))
+    assert np.array_equal(dec, oc.sq_decompress(raw, cbs, bits, cs, D))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_fused_vq_random_shape(seed):
+    rng = np.random.default_rng(3000 + seed)
+    w = int(rng.choice([4, 8, 16, 32]))
+    n_cb = int(rng.choice([1, 2, 4, 8, 16, 24]))
+    K = int(rng.choice([16, 100, 256]))
+    full = n_cb * w
+    D = int(rng.choice([full, max(4, full - 4), max(4, full - w // 2)]))
+    D = max(4, D - D % 4)
+    N, rows = int(rng.integers(50, 3000)), int(rng.integers(1, 1500))
+    idx = rng.choice([np.int32, np.int64])
+    cb = rng.standard_normal((n_cb, K, w)).astype(np.float32)
+    codes = rng.integers(0, K, size=(N, n_cb), dtype=np.uint8)
+    indptr, indices = graph(rng, rows, N, idx)
+    got = host(capi.vq_decompress_spmm_csr(dev(codes), dev(cb), dev(indptr), dev(indices), D))
+    want = oc.vq_decompress_spmm_csr(codes, cb, indptr.astype(np.int64), indices.astype(np.int64), D)
+    assert close(got, want)
+    dec = host(capi.vq_decompress(dev(codes), dev(cb), D))
+    assert np.array_equal(dec, oc.vq_decompress(codes, cb, D))
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_hybrid_random_shape(seed):
+    rng = np.random.default_rng(4000 + seed)
+    w = int(rng.choice([8, 16, 32]))
+    D = int(rng.choice([32, 64, 128, 256]))
+    n_cb = D // w
+    N, rows = int(rng.integers(100, 3000)), int(rng.integers(1, 1200))
+    idx = rng.choice([np.int32, np.int64])
+    n_sq = int(rng.integers(1, N))
+    n_vq = N - n_sq
+    x = rng.standard_normal((n_sq, D)).astype(np.float32)
+    params = oc.sq_affine_params(x, 8)
+    sq = oc.sq_affine_compress(x, params, 8)
+    cb = rng.standard_normal((n_cb, 256, w)).astype(np.float32)
+    vq = rng.integers(0, 256, size=(max(n_vq, 1), n_cb), dtype=np.uint8)
+    perm = rng.permutation(N)
+    row_map = np.empty(N, dtype=np.int32)
+    row_map[perm[:n_sq]] = np.arange(n_sq, dtype=np.int32)
+    row_map[perm[n_sq:]] = -np.arange(n_vq, dtype=np.int32) - 1
+    indptr, indices = graph(rng, rows, N, idx)
+    got = host(capi.hybrid_decompress_spmm_csr(dev(row_map), dev(sq), dev(params), dev(vq), dev(cb), dev(indptr),
+                                               dev(indices), D))
+    want = oc.hybrid_decompress_spmm_csr(row_map, sq, params, vq, cb, indptr.astype(np.int64),
+                                         indices.astype(np.int64), D)
+    assert close(got, want)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_pack_and_sq_encode_random_shape(seed):
+    rng = np.random.default_rng(5000 + seed)
+    bits = int(rng.choice([1, 2, 4]))
+    rows, U = int(rng.integers(1, 700)), int(rng.integers(1, 300))
+    codes = rng.integers(0, 1 << bits, size=(rows, U), dtype=np.uint8)
+    packed = host(capi.packbits(dev(codes), bits))
+    assert np.array_equal(packed, oc.packbits(codes, bits))
+    assert np.array_equal(host(capi.unpackbits(dev(packed), bits, U)), codes)
+    ebits = int(rng.choice([1, 2, 4, 8, 16]))
+    per = max(1, 8 // ebits)
+    D = int(rng.choice([4, 13, 32, 100, 130]))
+    cs = int(rng.choice([c for c in (8, 16, 64, 256) if c % per == 0]))
+    x = rng.uniform(-2, 2, size=(rows, D)).astype(np.float32)
+    cbs = np.stack([oc.sq_codebook(x[:, s:s + cs]) for s in range(0, D, cs)])
+    want = oc.sq_codes_to_storage(oc.sq_compress(x, cbs, ebits, cs), ebits)
+    got = host(capi.sq_encode(dev(x), dev(cbs), ebits, cs))
+    assert np.array_equal(got.view(want.dtype) if got.dtype != want.dtype else got, want)
