@@ -28,7 +28,7 @@ namespace {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 // Absolute part of the near-tie bound: the matrix core flushes products (and, for the split form,
-// piece products 2^-9 and 2^-18 of the full one) that fall below the smallest normal fp32 number,
+// piece products 2^-8 and 2^-16 of the full one) that fall below the smallest normal fp32 number,
 // which the relative bound does not see.  A few hundred such terms stay below this.
 constexpr float kTinyGap = 1e-33f;
 
@@ -294,7 +294,7 @@ __global__ __launch_bounds__(256) void predict_mfma_kernel(const float* __restri
 // The same scores at the bf16 matrix rate.  An fp32 value is the exact sum of three bf16 pieces
 // (round to nearest, then the residual, then its residual: 3 x 8 significand bits plus the signs
 // cover 24), a product of two pieces is exact in fp32, and of the nine piece products of x * c the
-// three of relative size <= 2^-26 are dropped, so six v_mfma_f32_32x32x16_bf16 per 16 dimensions
+// three of relative size <= 2^-24 are dropped, so six v_mfma_f32_32x32x16_bf16 per 16 dimensions
 // give x . c to fp32 accuracy at a sixth of the bf16 rate, 2.7 times the fp32 MFMA rate, and, unlike
 // fp32 MFMA, with the vector ALUs free for the arg-min update while the matrix core runs.  The
 // centre pieces sit in LDS in operand order ([piece][tile][step][lane] x 16 B, one ds_read_b128 per
@@ -331,8 +331,8 @@ __device__ int exact_argmin_row_l2_pieces(const float* __restrict__ xrow, float*
 #pragma unroll
     for (int e = 0; e < 8; ++e) cv[e] = ((float)p0[e] + (float)p1[e]) + (float)p2[e];
   };
-  // first pass: distance from the leading pieces only (relative error of a centre value 2^-9, of
-  // a distance well below 2^-3 of itself plus 2^-3 of the smallest one), one operand per chunk
+  // first pass: distance from the leading pieces only (relative error of a centre value 2^-8),
+  // one operand per chunk
   auto dist_lead = [&](int c) -> float {
     float d = 0.f;
 #pragma nounroll
@@ -366,9 +366,11 @@ __device__ int exact_argmin_row_l2_pieces(const float* __restrict__ xrow, float*
     }
     return d;
   };
-  // With c' the leading pieces, |c - c'| <= 2^-9 |c| per component, so
-  // | sqrt(d) - sqrt(d') | <= 2^-9 |c| <= 2^-9 (|x| + sqrt(d)): a centre can only be the minimum if
-  // sqrt(d') <= (sqrt(dmin') + 2^-8 |x|) * (1 + 2^-7) (slack for the fp32 sums included).
+  // With c' the leading pieces (8 significant bits, round to nearest), |c - c'| <= 2^-8 |c| per
+  // component, so | sqrt(d) - sqrt(d') | <= 2^-8 |c| <= 2^-8 (|x| + sqrt(d)): the centre c0 with the
+  // smallest d' has sqrt(d0) <= (sqrt(dmin') + 2^-8 |x|) / (1 - 2^-8), the true minimum is no
+  // farther, and so its own sqrt(d') <= (sqrt(dmin') + 2^-7 |x|) * (1 + 2^-6) (slack for the fp32
+  // sums included).
   constexpr int kKeep = 4;            // first-pass distances kept in registers (all of them up to 256 centres)
   float dkeep[kKeep] = {0.f, 0.f, 0.f, 0.f};
   float dmin = INFINITY;
@@ -410,7 +412,7 @@ __device__ int exact_argmin_row_l2_pieces(const float* __restrict__ xrow, float*
     dmin = fminf(dmin, __shfl_xor(dmin, off));
     xnorm2 += __shfl_xor(xnorm2, off);
   }
-  const float reach = (sqrtf(dmin) + 0.00390625f * sqrtf(xnorm2)) * 1.0078125f;
+  const float reach = (sqrtf(dmin) + 0.0078125f * sqrtf(xnorm2)) * 1.015625f;
   const float lead_limit = reach * reach * 1.0001f + 1e-37f;
   // second pass: full fp32 distance of the survivors, then the exact fp64 one of those that can
   // still be the minimum (relative error of the fp32 sum <= (k + 3) 2^-24, all terms positive)
@@ -458,8 +460,8 @@ __device__ int exact_argmin_row_l2_pieces(const float* __restrict__ xrow, float*
 }
 
 // Exact cosine assignment of one row by a whole wave.  The LDS pieces hold the centres divided by
-// their norms; with c' their leading pieces, |x . c/|c| - x . c'| <= 2^-9 |x| (1 + 2^-20), so only
-// centres whose leading-piece dot product is within 2^-7 |x| of the largest can have the smallest
+// their norms; with c' their leading pieces, |x . c/|c| - x . c'| <= 2^-8 |x| (1 + 2^-20), so only
+// centres whose leading-piece dot product is within 2^-6 |x| of the largest can have the smallest
 // distance; those are evaluated exactly, in fp64 from the centres in HBM, by the formula of
 // exact_argmin_row.  Needs every centre to have a direction (|c|^2 > 1e-12).
 template <int S>
@@ -488,7 +490,7 @@ __device__ int exact_argmin_row_cosine_pieces(const float* __restrict__ xrow, fl
   for (int c = lane; c < n; c += kWave) smax = fmaxf(smax, dot_lead(c));
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) smax = fmaxf(smax, __shfl_xor(smax, off));
-  const float floor_s = smax - 0.0078125f * sqrtf(xnorm2) - 1e-30f;
+  const float floor_s = smax - 0.015625f * sqrtf(xnorm2) - 1e-30f;
   double xn = 0.0;
   for (int t = 0; t < k; ++t) xn += (double)xrow[t] * (double)xrow[t];
   double bestv = DBL_MAX;
@@ -620,9 +622,10 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
   const int64_t n_groups = (m + kGroupRows - 1) / kGroupRows;
   // Error bound of one score in units of 2^-24 (|x|^2 + max |c|^2), which is >= 2 |x||c| = P and
   // >= |c|^2: each of the S leading instructions cuts its 17 addends at 2^-22 of the largest
-  // (<= P): 68 S; the small pairs together stay below 4; the bias sum k + 1; its addition 2; the
-  // dropped pairs 1.  Doubled for the two scores of a gap.
-  const float unit = 5.9604645e-8f * (float)(2 * (68 * S + k + 8));
+  // (<= P): 68 S; the small pairs (2^-8 P and below) together stay below 4; the bias sum k + 1;
+  // its addition 2; the dropped pairs (2^-24 P each way) 2; 3 spare.  Doubled for the two scores
+  // of a gap.
+  const float unit = 5.9604645e-8f * (float)(2 * (68 * S + k + 12));
   const float xscale = cosine ? -1.f : -2.f;
   const bool vec4 = (k % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
   // A workgroup owns a contiguous share of the row groups and its four waves draw from it through

@@ -361,6 +361,8 @@ def kmeans_predict(x: np.ndarray, centers: np.ndarray, metric: str):
     only specified outside the mask."""
     d = pairwise_distance(x, centers, metric, dtype=np.float64)
     labels = d.argmin(axis=1)
+    if d.shape[1] < 2:
+        return labels.astype(np.int64), np.zeros(d.shape[0], dtype=bool)
     part = np.partition(d, 1, axis=1)[:, :2]
     gap = part[:, 1] - part[:, 0]
     scale = np.maximum(np.abs(part[:, 1]), 1e-30)

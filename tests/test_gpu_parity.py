@@ -612,6 +612,22 @@ def test_kmeans_predict_extreme_magnitudes(scale):
     assert np.array_equal(got[~near], want[~near])
 
 
+@pytest.mark.parametrize("k,n", [(1, 256), (1, 700), (2, 300), (3, 256)])
+def test_kmeans_predict_few_dimensions_many_close_centres(k, n):
+    # points and centres packed on a short segment away from the origin: distances of 1e-5 next to
+    # norms of 4, so every row takes the exact path and its candidate filter (leading bf16 pieces of
+    # the centres, off by up to 2^-8 of their size) has to keep the true minimum among many
+    rng = np.random.default_rng(24 + k + n)
+    x = (rng.standard_normal((4000, k)) + 2.0).astype(np.float32)
+    c = (rng.standard_normal((n, k)) + 2.0).astype(np.float32)
+    want, near = oc.kmeans_predict(x, c, "l2")
+    got = host(capi.kmeans_predict(dev(x), dev(c), "l2"))
+    assert np.array_equal(got[~near], want[~near])
+    wantc, nearc = oc.kmeans_predict(x, c, "cosine")
+    gotc = host(capi.kmeans_predict(dev(x), dev(c), "cosine"))
+    assert np.array_equal(gotc[~nearc], wantc[~nearc])
+
+
 def test_kmeans_predict_cosine_with_a_centre_without_direction():
     rng = np.random.default_rng(22)
     x = rng.standard_normal((3000, 32)).astype(np.float32)

@@ -148,3 +148,25 @@ def test_pack_and_sq_encode_random_shape(seed):
     want = oc.sq_codes_to_storage(oc.sq_compress(x, cbs, ebits, cs), ebits)
     got = host(capi.sq_encode(dev(x), dev(cbs), ebits, cs))
     assert np.array_equal(got.view(want.dtype) if got.dtype != want.dtype else got, want)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_encode_random_shape(seed):
+    rng = np.random.default_rng(6000 + seed)
+    metric = str(rng.choice(["l2", "cosine"]))
+    m = int(rng.integers(1, 5000))
+    n = int(rng.choice([1, 2, 7, 33, 64, 100, 256, 300, 700]))
+    k = int(rng.choice([1, 3, 8, 16, 24, 32, 40, 64, 72, 130]))
+    shift = float(rng.choice([0.0, 0.0, 2.0, 30.0]))          # an offset makes the expanded form cancel
+    x = (rng.standard_normal((m, k)) + shift).astype(np.float32)
+    c = (rng.standard_normal((n, k)) + shift).astype(np.float32)
+    want, near = oc.kmeans_predict(x, c, metric)
+    got = host(capi.kmeans_predict(dev(x), dev(c), metric))
+    assert got.shape == (m,)
+    assert np.array_equal(got[~near], want[~near])
+    if n <= 256:
+        got8 = host(capi.kmeans_predict(dev(x), dev(c), metric, u8=True))
+        assert np.array_equal(got8.astype(np.int64), got)
+    d = host(capi.pairwise_distance(dev(x), dev(c), metric))
+    ref = oc.pairwise_distance(x, c, metric, dtype=np.float64)
+    assert np.allclose(d, ref, rtol=1e-5, atol=1e-5 * max(1.0, float(np.abs(ref).max())))
