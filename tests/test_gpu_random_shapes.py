@@ -22,8 +22,13 @@ def host(t):
 
 
 def graph(rng, rows, n_src, idx):
-    kind = rng.integers(0, 4)
-    if kind == 0:
+    kind = rng.integers(0, 6)
+    if kind == 4:
+        deg = np.zeros(rows, dtype=np.int64)                         # no edges at all
+    elif kind == 5:
+        deg = rng.integers(0, 3, size=rows)                          # a few very long rows among short ones
+        deg[rng.integers(0, rows, size=min(3, rows))] = int(rng.integers(300, 2500))
+    elif kind == 0:
         deg = rng.integers(0, 4, size=rows)                          # sparse, with empty rows
     elif kind == 1:
         deg = np.full(rows, int(rng.integers(1, 40)))                # fixed fanout
@@ -42,6 +47,18 @@ def close(got, want):
     return np.allclose(got, want, rtol=RTOL, atol=RTOL * scale)
 
 
+def agg_ok(got, want32, decoded, indptr, indices):
+    """Aggregation bar: within 1e-5 of the reference's sequential fp32 sum, or, where that sum
+    itself has drifted further from the exact mean (rows of thousands of edges), at least as close
+    to the fp64 mean of the same decoded fp32 values as the sequential fp32 sum is."""
+    if close(got, want32):
+        return True
+    exact = oc.spmm_csr(decoded.astype(np.float64), indptr.astype(np.int64), indices.astype(np.int64))
+    scale = float(np.abs(exact).max()) if exact.size else 1.0
+    bound = np.maximum(np.abs(want32 - exact), RTOL * np.abs(exact) + 1e-6 * scale)
+    return bool(np.all(np.abs(got - exact) <= bound))
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_fused_affine_sq_random_shape(seed):
     rng = np.random.default_rng(1000 + seed)
@@ -56,7 +73,7 @@ def test_fused_affine_sq_random_shape(seed):
     got = host(capi.sq_affine_decompress_spmm_csr(dev(codes), dev(params), dev(indptr), dev(indices), bits, D))
     want = oc.sq_affine_decompress_spmm_csr(codes, params, indptr.astype(np.int64), indices.astype(np.int64), bits, D)
     assert got.shape == want.shape
-    assert close(got, want)
+    assert agg_ok(got, want, oc.sq_affine_decompress(codes, params, bits, D), indptr, indices)
 
 
 @pytest.mark.parametrize("seed", range(24))
@@ -76,7 +93,7 @@ def test_fused_log_sq_random_shape(seed):
     got = host(capi.sq_decompress_spmm_csr(dev(store), dev(cbs), dev(indptr), dev(indices), bits, cs, D))
     raw = store.view(np.uint8) if store.dtype == np.int8 and bits < 8 else store
     want = oc.sq_decompress_spmm_csr(raw, cbs, indptr.astype(np.int64), indices.astype(np.int64), bits, cs, D)
-    assert close(got, want)
+    assert agg_ok(got, want, oc.sq_decompress_per_byte_codebook(raw, cbs, bits, cs, D), indptr, indices)
     # and the standalone decode of the same table, bit for bit
     dec = host(capi.sq_decompress(dev(store), dev(cbs), bits, cs, D))
     assert np.array_equal(dec, oc.sq_decompress(raw, cbs, bits, cs, D))
@@ -98,7 +115,7 @@ def test_fused_vq_random_shape(seed):
     indptr, indices = graph(rng, rows, N, idx)
     got = host(capi.vq_decompress_spmm_csr(dev(codes), dev(cb), dev(indptr), dev(indices), D))
     want = oc.vq_decompress_spmm_csr(codes, cb, indptr.astype(np.int64), indices.astype(np.int64), D)
-    assert close(got, want)
+    assert agg_ok(got, want, oc.vq_decompress(codes, cb, D), indptr, indices)
     dec = host(capi.vq_decompress(dev(codes), dev(cb), D))
     assert np.array_equal(dec, oc.vq_decompress(codes, cb, D))
 
@@ -127,7 +144,7 @@ def test_hybrid_random_shape(seed):
                                                dev(indices), D))
     want = oc.hybrid_decompress_spmm_csr(row_map, sq, params, vq, cb, indptr.astype(np.int64),
                                          indices.astype(np.int64), D)
-    assert close(got, want)
+    assert agg_ok(got, want, oc.hybrid_decompress(row_map, sq, params, vq, cb, D, np.arange(N)), indptr, indices)
 
 
 @pytest.mark.parametrize("seed", range(16))
