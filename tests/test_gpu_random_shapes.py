@@ -187,3 +187,45 @@ def test_encode_random_shape(seed):
     d = host(capi.pairwise_distance(dev(x), dev(c), metric))
     ref = oc.pairwise_distance(x, c, metric, dtype=np.float64)
     assert np.allclose(d, ref, rtol=1e-5, atol=1e-5 * max(1.0, float(np.abs(ref).max())))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_module_dtype_surface_random(seed):
+    """The F2CGTLib module with the reference's accepted dtypes (src/common.h:17-104): index tensors of
+    any integer width, fp16 / fp64 features for spmm_csr, fp16 codebooks and int16 codes for vq_decompress."""
+    import f2cgt_amd
+    lib = f2cgt_amd.load()
+    rng = np.random.default_rng(7000 + seed)
+    idt = [torch.int8, torch.uint8, torch.int16, torch.int32, torch.int64][seed % 5]
+    cap = {torch.int8: 127, torch.uint8: 255, torch.int16: 32767}.get(idt, 1 << 20)
+    n_src = int(min(cap, rng.integers(20, 2000)))
+    D = int(rng.choice([4, 16, 60, 128]))
+    # rows and edges limited so that every offset fits the index type
+    rows = int(rng.integers(1, 40))
+    deg = rng.integers(0, 4, size=rows)
+    while deg.sum() > cap:
+        deg = deg // 2
+    indptr = np.zeros(rows + 1, dtype=np.int64)
+    indptr[1:] = np.cumsum(deg)
+    indices = rng.integers(0, n_src, size=int(indptr[-1]))
+    ip, ix = torch.from_numpy(indptr).to(idt).cuda(), torch.from_numpy(indices).to(idt).cuda()
+    for ft in (torch.float32, torch.float16, torch.float64):
+        feat = torch.from_numpy(rng.standard_normal((n_src, D)).astype(np.float32)).to(ft).cuda()
+        out = lib.spmm_csr(feat, ip, ix)
+        assert out.dtype == ft and tuple(out.shape) == (rows, D)
+        want = oc.spmm_csr(feat.cpu().double().numpy(), indptr, indices)
+        tol = 2e-3 if ft == torch.float16 else 1e-5
+        assert np.allclose(out.cpu().double().numpy(), want, rtol=tol, atol=tol * max(1.0, float(np.abs(want).max())))
+    w, n_cb, K = 8, (D + 7) // 8, int(rng.choice([50, 256, 1000]))
+    if D >= 8:
+        cb = rng.standard_normal((n_cb, K, w)).astype(np.float32)
+        cdt = torch.uint8 if K <= 256 else torch.int16
+        codes = torch.from_numpy(rng.integers(0, K, size=(n_src, n_cb))).to(cdt).cuda()
+        for cbt in (torch.float32, torch.float16):
+            cbd = torch.from_numpy(cb).to(cbt).cuda()
+            dec = lib.vq_decompress(codes, cbd, D)
+            want = oc.vq_decompress(codes.cpu().numpy().astype(np.int64), cbd.float().cpu().numpy(), D)
+            assert np.array_equal(dec.float().cpu().numpy(), want)
+        fused = lib.vq_decompress_spmm_csr(codes, torch.from_numpy(cb).cuda(), ip, ix, D)
+        wantf = oc.vq_decompress_spmm_csr(codes.cpu().numpy().astype(np.int64), cb, indptr, indices, D)
+        assert close(fused.cpu().numpy(), wantf)
