@@ -32,11 +32,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # what the same counter reads for a plain copy of known size; see profiles/).  Keyed by
 # (workload name, index dtype).  Missing = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1_sq8_affine", "int64"): 18288715,
-    ("c2_sq4_affine", "int64"): 134110465,
-    ("c3_vq_16x8", "int64"): 506924358,
-    ("c4_hybrid", "int64"): 1004036407,
-    ("c5_vq_24x32", "int64"): 2195298735,
+    ("c1_sq8_affine", "int64"): 18275409,
+    ("c2_sq4_affine", "int64"): 134237487,
+    ("c3_vq_16x8", "int64"): 506816011,
+    ("c4_hybrid", "int64"): 1004036160,
+    ("c5_vq_24x32", "int64"): 2171366722,
 }
 
 
