@@ -1,6 +1,11 @@
 """Seeded random shapes through every fused operator and the streaming ones: the fast kernels are
 chosen by shape (column count, bits, degree, index type, alignment), so many small, odd shapes are
-what finds a path that a hand-picked list misses.  Same bars as the parity tests."""
+what finds a path that a hand-picked list misses.  Same bars as the parity tests.
+
+F2CGT_FUZZ_SEED0 (first seed, default 0) and F2CGT_FUZZ_MULT (multiplier of the number of seeds per
+test, default 1) widen the sweep for a one-off run; the defaults are what the suite runs."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -10,6 +15,12 @@ from f2cgt_amd import capi
 
 pytestmark = pytest.mark.gpu
 RTOL = 1e-5
+SEED0 = int(os.environ.get("F2CGT_FUZZ_SEED0", "0"))
+MULT = int(os.environ.get("F2CGT_FUZZ_MULT", "1"))
+
+
+def seeds(n):
+    return range(SEED0, SEED0 + n * MULT)
 
 
 def dev(a):
@@ -59,7 +70,7 @@ def agg_ok(got, want32, decoded, indptr, indices):
     return bool(np.all(np.abs(got - exact) <= bound))
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", seeds(24))
 def test_fused_affine_sq_random_shape(seed):
     rng = np.random.default_rng(1000 + seed)
     bits = int(rng.choice([1, 2, 4, 8]))
@@ -76,7 +87,7 @@ def test_fused_affine_sq_random_shape(seed):
     assert agg_ok(got, want, oc.sq_affine_decompress(codes, params, bits, D), indptr, indices)
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", seeds(24))
 def test_fused_log_sq_random_shape(seed):
     rng = np.random.default_rng(2000 + seed)
     bits = int(rng.choice([1, 2, 4, 8, 16]))
@@ -99,7 +110,7 @@ def test_fused_log_sq_random_shape(seed):
     assert np.array_equal(dec, oc.sq_decompress(raw, cbs, bits, cs, D))
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", seeds(24))
 def test_fused_vq_random_shape(seed):
     rng = np.random.default_rng(3000 + seed)
     w = int(rng.choice([4, 8, 16, 32]))
@@ -120,7 +131,7 @@ def test_fused_vq_random_shape(seed):
     assert np.array_equal(dec, oc.vq_decompress(codes, cb, D))
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", seeds(16))
 def test_hybrid_random_shape(seed):
     rng = np.random.default_rng(4000 + seed)
     w = int(rng.choice([8, 16, 32]))
@@ -147,7 +158,7 @@ def test_hybrid_random_shape(seed):
     assert agg_ok(got, want, oc.hybrid_decompress(row_map, sq, params, vq, cb, D, np.arange(N)), indptr, indices)
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", seeds(16))
 def test_pack_and_sq_encode_random_shape(seed):
     rng = np.random.default_rng(5000 + seed)
     bits = int(rng.choice([1, 2, 4]))
@@ -167,7 +178,7 @@ def test_pack_and_sq_encode_random_shape(seed):
     assert np.array_equal(got.view(want.dtype) if got.dtype != want.dtype else got, want)
 
 
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", seeds(40))
 def test_encode_random_shape(seed):
     rng = np.random.default_rng(6000 + seed)
     metric = str(rng.choice(["l2", "cosine"]))
@@ -189,7 +200,7 @@ def test_encode_random_shape(seed):
     assert np.allclose(d, ref, rtol=1e-5, atol=1e-5 * max(1.0, float(np.abs(ref).max())))
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", seeds(12))
 def test_module_dtype_surface_random(seed):
     """The F2CGTLib module with the reference's accepted dtypes (src/common.h:17-104): index tensors of
     any integer width, fp16 / fp64 features for spmm_csr, fp16 codebooks and int16 codes for vq_decompress."""
