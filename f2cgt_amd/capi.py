@@ -34,6 +34,7 @@ SIGNATURES = {
     "f2cgt_sq_affine_decompress_spmm_csr": ([P, P, L, P, P, I, P, L, L, L, L, L, I, P], c_int),
     "f2cgt_hybrid_decompress_spmm_csr":
         ([P, P, P, L, P, P, P, P, I, P, L, L, L, L, L, L, L, L, L, P], c_int),
+    "f2cgt_fetch_rows": ([P, P, P, P, I, P, L, L, L, L, P], c_int),
     "f2cgt_pairwise_distance": ([P, P, P, L, L, L, I, P], c_int),
     "f2cgt_kmeans_predict": ([P, P, P, P, L, L, L, I, P], c_int),
 }
@@ -204,6 +205,19 @@ def hybrid_decompress_spmm_csr(row_map, sq_codes, sq_params, vq_codes, vq_codebo
         _ptr(vq_codebooks), _ptr(indptr), _ptr(indices), _tag(indptr), _ptr(out), rows, indices.numel(),
         row_map.numel(), sq_codes.shape[0], vq_codes.shape[0], feat_dim, vq_codebooks.shape[0],
         vq_codebooks.shape[1], vq_codebooks.shape[2], _stream()), "hybrid_decompress_spmm_csr")
+    return out
+
+
+def fetch_rows(table, index, hot=None, slot_map=None, out=None):
+    """out[i] = hot[slot_map[index[i]]] where that slot is >= 0, else table[index[i]].  `table` is
+    any contiguous 2-D tensor on the device or in pinned host memory; rows are moved as bytes."""
+    import torch
+    row_bytes = table.shape[1] * table.element_size()
+    if out is None:
+        out = torch.empty((index.numel(), table.shape[1]), dtype=table.dtype, device=index.device)
+    _check(lib().f2cgt_fetch_rows(_ptr(table), _ptr(hot), _ptr(slot_map), _ptr(index), _tag(index), _ptr(out),
+                                  index.numel(), row_bytes, table.shape[0],
+                                  0 if hot is None else hot.shape[0], _stream()), "fetch_rows")
     return out
 
 

@@ -427,6 +427,42 @@ torch::Tensor kmeans_predict(torch::Tensor x, torch::Tensor centers, std::string
   return kmeans_predict_impl(x, centers, metric, false);
 }
 
+// Row fetch of the feature cache (examples/tensor_cache.py:49-58).  `table` is a device tensor
+// or a pinned host tensor (mapped into the device address space); `hot` and `slot_map` are the
+// device-resident cache of hot rows and the id -> cache slot array (-1 = not cached).
+torch::Tensor fetch_rows(torch::Tensor table, torch::Tensor index, c10::optional<torch::Tensor> hot,
+                         c10::optional<torch::Tensor> slot_map) {
+  TORCH_CHECK(table.defined() && table.dim() == 2 && table.is_contiguous(), "table must be a contiguous 2-D tensor");
+  TORCH_CHECK(table.device().is_cuda() || table.is_pinned(),
+              "table must be on the GPU or in pinned host memory");
+  index = dev_contig(index, "index");
+  TORCH_CHECK(index.dim() == 1, "index must be 1-D");
+  auto st = index.scalar_type();
+  TORCH_CHECK(st == torch::kInt64 || st == torch::kInt32, "index must be int32 or int64");
+  TORCH_CHECK(hot.has_value() == slot_map.has_value(), "hot and slot_map come together");
+  torch::Tensor hot_t, slot_t;
+  int64_t num_hot = 0;
+  if (hot.has_value()) {
+    hot_t = dev_contig(*hot, "hot");
+    slot_t = dev_contig(*slot_map, "slot_map");
+    TORCH_CHECK(hot_t.dim() == 2 && hot_t.size(1) == table.size(1) && hot_t.scalar_type() == table.scalar_type(),
+                "hot must have the row shape and dtype of table");
+    TORCH_CHECK(slot_t.scalar_type() == torch::kInt32 && slot_t.dim() == 1 && slot_t.numel() == table.size(0),
+                "slot_map must be int32 with one entry per row of table");
+    num_hot = hot_t.size(0);
+  }
+  TORCH_CHECK(index.numel() == 0 || table.size(0) > 0, "rows requested from an empty table");
+  c10::DeviceGuard guard(index.device());
+  auto out = torch::empty({index.numel(), table.size(1)}, table.options().device(index.device()).pinned_memory(false));
+  const int64_t row_bytes = table.size(1) * (int64_t)table.element_size();
+  check_rc(f2cgt_fetch_rows(table.data_ptr(), num_hot ? hot_t.data_ptr() : nullptr,
+                            num_hot ? slot_t.data_ptr<int32_t>() : nullptr, index.data_ptr(),
+                            st == torch::kInt64 ? F2CGT_DT_I64 : F2CGT_DT_I32, out.data_ptr(), index.numel(),
+                            row_bytes, table.size(0), num_hot, current_stream()),
+           "fetch_rows");
+  return out;
+}
+
 torch::Tensor vq_encode(torch::Tensor x, torch::Tensor centers, std::string metric) {
   return kmeans_predict_impl(x, centers, metric, true);
 }
@@ -462,7 +498,9 @@ PYBIND11_MODULE(F2CGTLib, m) {
       .def("sq_encode", &sq_encode, py::arg("src"), py::arg("codebooks"), py::arg("target_bits"),
            py::arg("column_slice"))
       .def("kmeans_predict", &kmeans_predict, py::arg("x"), py::arg("centers"), py::arg("metric"))
-      .def("vq_encode", &vq_encode, py::arg("x"), py::arg("centers"), py::arg("metric"));
+      .def("vq_encode", &vq_encode, py::arg("x"), py::arg("centers"), py::arg("metric"))
+      .def("fetch_rows", &fetch_rows, py::arg("table"), py::arg("index"), py::arg("hot") = py::none(),
+           py::arg("slot_map") = py::none());
   py::class_<KMeans>(m, "KMeans")
       .def(py::init<int64_t, int64_t, std::string, int, double, int, double, int, int, bool>(),
            py::arg("n_cluster"), py::arg("feat_dim"), py::arg("metric"), py::arg("max_iter") = 300,

@@ -4,6 +4,8 @@ place of DGL blocks, ShmTensor and torch.distributed (one process, one GPU):
   * the offline encode pipeline: `sq_metadata`, `sq_compress`, `vq_metadata`, `vq_compress`
     (examples/process_compress.py:16-68, 71-144, 147-292), `run` that writes the artefact files
     (`:295-388`) and `load_compress_data` that reads them back (examples/load_dataset.py:63-85);
+  * `TensorCache` (examples/tensor_cache.py:36-110): a table of rows on the device or in pinned
+    host memory, with an optional device-resident copy of its hottest rows, indexed by global id;
   * `CompressionManager` (examples/compress.py:8-106): keeps the code tables and codebooks,
     serves seed rows (first level) and neighbour rows (second level);
   * `MySAGEConv` (examples/conv.py:9-76): GraphSAGE mean layer whose neighbour aggregation is the
@@ -214,6 +216,67 @@ def load_compress_data(root):
 
 
 # ---- runtime callers -------------------------------------------------------------------------------
+class TensorCache:
+    """examples/tensor_cache.py:36-110 without ShmTensor.
+
+    `data` is a 2-D table of rows (code rows or plain features).  A host table is copied once
+    into pinned memory that the device can address (the reference pins the shared-memory table in
+    place; registering existing memory is not available here), and `cache[index]` reads its rows
+    over the host link; `create_cache(capacity, hotness)` moves the whole table to the device
+    when it fits in `capacity` bytes and otherwise keeps a device copy of the hottest rows plus a
+    dense int32 array id -> cache slot (-1 = not cached) where the reference keeps a GPU hash
+    map.  The array costs 4 bytes per table row and is charged to the capacity.
+    `index` is a device tensor of int32/int64 ids; the result is a new device tensor."""
+
+    def __init__(self, data):
+        if data.dim() != 2:
+            raise ValueError("TensorCache holds a 2-D table of rows")
+        if data.device.type == "cpu":
+            pinned = torch.empty(data.shape, dtype=data.dtype, pin_memory=True)
+            pinned.copy_(data)
+            data = pinned
+        self.data = data.contiguous()
+        self.gpu_data = None
+        self.slot_map = None
+        self.has_cache = False
+
+    def __getitem__(self, index):
+        capi = _capi()
+        if index.dtype not in (torch.int32, torch.int64):
+            index = index.long()
+        if self.has_cache:
+            return capi.fetch_rows(self.data, index, self.gpu_data, self.slot_map)
+        return capi.fetch_rows(self.data, index)
+
+    def create_cache(self, cache_capacity, hotness):
+        if cache_capacity <= 0:
+            return
+        full_size = self.data.numel() * self.data.element_size()
+        if full_size <= cache_capacity:
+            self.data = self.data.cuda()
+            return
+        row_bytes = self.data.shape[1] * self.data.element_size()
+        cache_num = int((cache_capacity - 4 * self.data.shape[0]) // row_bytes)
+        if cache_num <= 0:
+            return
+        _, candidates = torch.sort(hotness, descending=True)
+        candidates = candidates[:cache_num]
+        self.gpu_data = self.data[candidates.to(self.data.device)].cuda()
+        self.slot_map = torch.full((self.data.shape[0],), -1, dtype=torch.int32, device="cuda")
+        self.slot_map[candidates.cuda().long()] = torch.arange(candidates.numel(), dtype=torch.int32, device="cuda")
+        self.has_cache = True
+
+    def clear_cache(self):
+        self.has_cache = False
+        self.gpu_data = None
+        self.slot_map = None
+
+    def compute_weight_size(self, hotness):
+        full_size = self.data.numel() * self.data.element_size()
+        item_size = self.data.element_size() * self.data.shape[1] * torch.mean(hotness[hotness > 0]).item()
+        return full_size, item_size
+
+
 class CompressionManager:
     """examples/compress.py:8-106 on plain tensors.
 
@@ -222,23 +285,30 @@ class CompressionManager:
     `configs` (per level (column_slice, target_bits)), `codebooks` (per level), `compression_data`
     (code table of the last level, [N, src_dim]), and for two levels `seeds_compression_data`
     (code table of the seed rows) with `seeds` (their global ids).
+
+    The code tables sit behind `TensorCache`.  `device_resident=True` (the default: the largest
+    table of the benchmark configurations is 5.76 GB against 288 GB of device memory) moves them
+    to the device at construction, the reference's whole-table cache
+    (examples/tensor_cache.py:66-70); `False` leaves host tables in pinned host memory until
+    `manager.data.create_cache(capacity, hotness)` is called, as the reference does.
     """
 
-    def __init__(self, compress_data, fusion=False):
+    def __init__(self, compress_data, fusion=False, device_resident=True):
         self.meta = compress_data
         self.methods = compress_data["methods"]
         self.feat_dim = compress_data["feat_dim"]
         self.configs = compress_data["configs"]
         self.codebooks = [c.cuda() for c in compress_data["codebooks"]]
-        self.data = compress_data["compression_data"].cuda()
+        place = (lambda t: t.cuda()) if device_resident else (lambda t: t)
+        self.data = TensorCache(place(compress_data["compression_data"]))
         self.seeds_data = None
         self.is_two_level = len(self.methods) >= 2
         self.is_fusion = fusion
         if self.is_two_level:
-            self.seeds_data = compress_data["seeds_compression_data"].cuda()
+            self.seeds_data = TensorCache(place(compress_data["seeds_compression_data"]))
             keys = compress_data["seeds"].long().cuda()
             # global id -> row of the seed table (the reference keeps a GPU hash map)
-            self.seed_slot = torch.full((self.data.shape[0],), -1, dtype=torch.int32, device="cuda")
+            self.seed_slot = torch.full((self.data.data.shape[0],), -1, dtype=torch.int32, device="cuda")
             self.seed_slot[keys] = torch.arange(keys.numel(), dtype=torch.int32, device="cuda")
 
     def _decompress(self, level, data):
@@ -254,10 +324,10 @@ class CompressionManager:
         slots = self.seed_slot[seeds_key.long()].long()
         if bool((slots < 0).any()):
             raise KeyError("a requested id is not a seed row")
-        return self._decompress(0, self.seeds_data[slots].contiguous())
+        return self._decompress(0, self.seeds_data[slots])
 
     def get_all_data(self, keys):
-        data = self.data[keys.long()].contiguous()
+        data = self.data[keys]
         if self.is_fusion:
             return data
         return self._decompress(1 if self.is_two_level else 0, data)

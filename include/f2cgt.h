@@ -166,6 +166,21 @@ int f2cgt_hybrid_decompress_spmm_csr(const int32_t* row_map, const uint8_t* sq_c
                                      int64_t num_codebooks, int64_t K, int64_t width,
                                      void* stream);
 
+/* ---- row fetch in front of the operators -------------------------------------- */
+
+/* Replaces TensorCache.__getitem__, examples/tensor_cache.py:49-58: shmtensor.capi.uva_fetch
+ * (slot_map NULL) and shmtensor.capi.cache_fetch (hot table + id -> slot map; the reference
+ * keeps a GPU hash map, examples/tensor_cache.py:80-86, here a dense int32 array).
+ * Tables hold opaque rows of row_bytes bytes each (code rows or plain feature rows).
+ * out[i, :] = hot[slot_map[id], :] if slot_map && 0 <= slot_map[id] < num_hot_rows
+ *            else table[id, :],   id = index[i] clamped to [0, num_rows).
+ * `table` may be pinned host memory mapped into the device address space (its rows then
+ * cross the host link); hot, slot_map [num_rows], index [num_index] and out
+ * [num_index, row_bytes] are device buffers.  No alignment is required of any of them. */
+int f2cgt_fetch_rows(const void* table, const void* hot, const int32_t* slot_map,
+                     const void* index, int idx_dtype, void* out, int64_t num_index,
+                     int64_t row_bytes, int64_t num_rows, int64_t num_hot_rows, void* stream);
+
 /* ---- VQ encode ---------------------------------------------------------------- */
 
 /* Replaces pairwise_distance(), src/kmeans.cu:102-118 (raft L2Unexpanded /

@@ -24,6 +24,8 @@ What pins each function (tests/test_oracle_*.py):
   fused ops             == spmm_csr(decompress(.)) bit for bit
                         (tests/test_fusion_decompress_spmm.py:27-33,113-120).
   pairwise_distance     torch.cdist**2 / 1-cosine_similarity, fp64 brute force.
+  fetch_rows            torch.index_select on the full table; a cache of any subset of
+                        rows must not change the result.
   sq_affine_*, hybrid   closed forms stated by the benchmark configuration.
 
 PARITY UNPINNED (nothing in the reference or in this container fixes them):
@@ -329,6 +331,23 @@ def hybrid_decompress_spmm_csr(row_map, sq_codes, sq_params, vq_codes, vq_codebo
     table = hybrid_decompress(row_map, sq_codes, sq_params, vq_codes, vq_codebooks,
                               feat_dim, uniq)
     return spmm_csr(table, indptr, inv)
+
+
+# --------------------------------------------------------------------------- #
+# Row fetch in front of the operators (examples/tensor_cache.py:49-58)
+# --------------------------------------------------------------------------- #
+def fetch_rows(table: np.ndarray, index: np.ndarray, hot: np.ndarray = None,
+               slot_map: np.ndarray = None) -> np.ndarray:
+    """TensorCache.__getitem__: row `index[i]` of the table, taken from the cache of hot rows
+    where the id has a slot (shmtensor cache_fetch) and from the table itself otherwise
+    (uva_fetch).  The cache holds copies (`gpu_data = data[cache_candidates]`,
+    examples/tensor_cache.py:79), so the result equals `table[index]` whenever it does."""
+    index = np.asarray(index).astype(np.int64)
+    out = np.empty((index.size,) + table.shape[1:], dtype=table.dtype)
+    for i, key in enumerate(index):
+        slot = -1 if slot_map is None else int(slot_map[key])
+        out[i] = hot[slot] if slot >= 0 else table[key]
+    return out
 
 
 # --------------------------------------------------------------------------- #
