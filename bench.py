@@ -214,6 +214,33 @@ def _others(idx):
     vq = torch.randint(0, 256, (n, 16), dtype=torch.uint8, device="cuda")
     _, ms = _time_steps(lambda: capi.vq_decompress(vq, cb, 128), 20, 3)
     res["vq_decompress_16x8_2.4M"] = {"launch_us": ms * 1e3, "GBps": n * (16 + 512) / (ms * 1e-3) / 1e9}
+    del vq, codes
+    # the row fetch in front of the operators: uniform random ids (no reuse to speak of), device
+    # tables; bytes = ids + rows read + rows written (+ the slot array with a cache of hot rows)
+    m = 4_000_000
+    ids = torch.randint(0, n, (m,), device="cuda")
+
+    def fetch_case(name, table, hot=None, slot=None, count=m):
+        idx = ids[:count]
+        out = torch.empty((count, table.shape[1]), dtype=table.dtype, device="cuda")
+        _, t = _time_steps(lambda: capi.fetch_rows(table, idx, hot, slot, out=out), 20, 3)
+        rb = table.shape[1] * table.element_size()
+        nbytes = count * (8 + 2 * rb + (4 if slot is not None else 0))
+        res[name] = {"launch_us": t * 1e3, "rows_per_s": count / (t * 1e-3), "GBps": nbytes / (t * 1e-3) / 1e9}
+
+    fetch_case("fetch_rows_16B_4M_of_2.4M", torch.randint(0, 256, (n, 16), dtype=torch.uint8, device="cuda"))
+    fetch_case("fetch_rows_50B_4M_of_2.4M", packed)
+    hot_ids = torch.randperm(n, device="cuda")[:n // 4]
+    slot = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    slot[hot_ids] = torch.arange(hot_ids.numel(), dtype=torch.int32, device="cuda")
+    fetch_case("fetch_rows_50B_4M_quarter_cached", packed, packed[hot_ids].contiguous(), slot)
+    feats = torch.randn((n, d), device="cuda")
+    fetch_case("fetch_rows_400B_4M_of_2.4M", feats)
+    host_table = torch.empty((n, 50), dtype=torch.uint8, pin_memory=True)
+    host_table.copy_(packed)
+    fetch_case("fetch_rows_50B_pinned_host_1M", host_table, count=1_000_000)
+    fetch_case("fetch_rows_50B_pinned_host_1M_quarter_cached", host_table, packed[hot_ids].contiguous(), slot,
+               count=1_000_000)
     return res
 
 

@@ -8,18 +8,17 @@
 // (no slot map) and shmtensor.capi.cache_fetch (hot table + id -> slot hash map; here the map is a
 // dense int32 array indexed by the id, one dependent load instead of a probe sequence).
 //
-// A group of 1..64 lanes owns a row and moves it in pieces of V bytes.  V = 16 when the row
-// pitch and every base address are multiples of 16; otherwise the pieces are 8 (4, 2, 1 for rows
-// shorter than that) bytes at byte granularity -- the hardware serves unaligned global accesses --
-// and the last piece of a row is moved back so that it ends with the row (the overlap is written
-// twice with the same bytes).  Every lane issues the loads of four rows before the first store.
+// A group of 1..64 lanes owns a row and moves it in pieces of V = 16 bytes (8, 4, 2, 1 for rows
+// shorter than that) at byte granularity -- the hardware serves unaligned global accesses -- and
+// the last piece of a row is moved back so that it ends with the row (the overlap is written
+// twice with the same bytes).  Every lane issues the loads of U rows (8 for rows of up to four
+// pieces, else 4) before the first store.
 #include "common.hpp"
 
 namespace f2cgt {
 namespace {
 
 constexpr int kFetchThreads = 256;
-constexpr int kFetchUnroll = 4;
 
 struct FetchArgs {
   const uint8_t* table;
@@ -39,7 +38,7 @@ template <> struct piece_type<4> { typedef uint32_t type; };
 template <> struct piece_type<2> { typedef uint16_t type; };
 template <> struct piece_type<1> { typedef uint8_t type; };
 
-template <int V, typename Idx>
+template <int V, int kFetchUnroll, typename Idx>
 __global__ __launch_bounds__(kFetchThreads) void fetch_rows_kernel(FetchArgs a, const Idx* __restrict__ index) {
   using P = typename piece_type<V>::type;
   const int rows_per_pass = kFetchThreads >> a.group_shift;
@@ -78,23 +77,29 @@ __global__ __launch_bounds__(kFetchThreads) void fetch_rows_kernel(FetchArgs a, 
   }
 }
 
+template <int V, int U>
+int launch_fetch(FetchArgs a, const void* index, int idx_dtype, hipStream_t st) {
+  const int64_t rows_per_block = (int64_t)(kFetchThreads >> a.group_shift) * U;
+  const int64_t blocks = ceil_div(a.n, rows_per_block);
+  F2CGT_REQUIRE(blocks <= 0x7fffffff, F2CGT_E_UNSUPPORTED, "fetch_rows: %lld rows need more than 2^31 workgroups",
+                (long long)a.n);
+  if (idx_dtype == F2CGT_DT_I64)
+    fetch_rows_kernel<V, U, int64_t><<<dim3((unsigned)blocks), dim3(kFetchThreads), 0, st>>>(
+        a, static_cast<const int64_t*>(index));
+  else
+    fetch_rows_kernel<V, U, int32_t><<<dim3((unsigned)blocks), dim3(kFetchThreads), 0, st>>>(
+        a, static_cast<const int32_t*>(index));
+  return launch_status("fetch_rows");
+}
+
 template <int V>
 int launch_fetch(FetchArgs a, const void* index, int idx_dtype, hipStream_t st) {
   a.pieces = (int)ceil_div(a.row_bytes, V);
   a.group = a.pieces >= 64 ? 64 : pow2_ceil(a.pieces);
   a.group_shift = 0;
   while ((1 << a.group_shift) < a.group) ++a.group_shift;
-  const int64_t rows_per_block = (int64_t)(kFetchThreads >> a.group_shift) * kFetchUnroll;
-  const int64_t blocks = ceil_div(a.n, rows_per_block);
-  F2CGT_REQUIRE(blocks <= 0x7fffffff, F2CGT_E_UNSUPPORTED, "fetch_rows: %lld rows need more than 2^31 workgroups",
-                (long long)a.n);
-  if (idx_dtype == F2CGT_DT_I64)
-    fetch_rows_kernel<V, int64_t><<<dim3((unsigned)blocks), dim3(kFetchThreads), 0, st>>>(
-        a, static_cast<const int64_t*>(index));
-  else
-    fetch_rows_kernel<V, int32_t><<<dim3((unsigned)blocks), dim3(kFetchThreads), 0, st>>>(
-        a, static_cast<const int32_t*>(index));
-  return launch_status("fetch_rows");
+  if (a.pieces <= 4) return launch_fetch<V, 8>(a, index, idx_dtype, st);
+  return launch_fetch<V, 4>(a, index, idx_dtype, st);
 }
 
 }  // namespace
@@ -125,8 +130,7 @@ extern "C" int f2cgt_fetch_rows(const void* table, const void* hot, const int32_
   a.num_hot = num_hot_rows;
   a.pieces = a.group = a.group_shift = 0;
   hipStream_t st = as_stream(stream);
-  const bool a16 = row_bytes % 16 == 0 && aligned(table, 16) && aligned(out, 16) && (a.slot == nullptr || aligned(hot, 16));
-  if (a16) return launch_fetch<16>(a, index, idx_dtype, st);
+  if (row_bytes >= 16) return launch_fetch<16>(a, index, idx_dtype, st);
   if (row_bytes >= 8) return launch_fetch<8>(a, index, idx_dtype, st);
   if (row_bytes >= 4) return launch_fetch<4>(a, index, idx_dtype, st);
   if (row_bytes >= 2) return launch_fetch<2>(a, index, idx_dtype, st);

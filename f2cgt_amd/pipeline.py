@@ -332,6 +332,23 @@ class CompressionManager:
             return data
         return self._decompress(1 if self.is_two_level else 0, data)
 
+    def aggregate_global(self, indptr, indices, input_nodes):
+        """Mean aggregation of a sampled block straight from the device-resident code table:
+        `indices` are positions in `input_nodes` (the block's source ids), which are composed
+        into global ids so that the fused operator reads the table rows itself and the gathered
+        copy of `get_all_data` is never written.  Same result as
+        `fused_op(get_all_data(input_nodes), ..., indptr, indices)`."""
+        if not self.data.data.is_cuda:
+            raise RuntimeError("aggregate_global needs the code table on the device")
+        capi = _capi()
+        level = 1 if self.is_two_level else 0
+        global_ids = input_nodes.to(indices.dtype)[indices.long()]
+        if self.methods[level] == "vq":
+            return capi.vq_decompress_spmm_csr(self.data.data, self.codebooks[level], indptr, global_ids,
+                                               self.feat_dim)
+        return capi.sq_decompress_spmm_csr(self.data.data, self.codebooks[level], indptr, global_ids,
+                                           self.configs[level][1], self.configs[level][0], self.feat_dim)
+
     def reorganize_seeds_data(self, seeds_feature, all_feature, num_dst):
         if not self.is_fusion:
             if seeds_feature is None:

@@ -173,6 +173,37 @@ def test_manager_with_host_resident_tables_matches_device_resident():
     assert torch.equal(a, b) and torch.equal(a.cpu(), table.cpu()[keys.cpu()])
 
 
+@pytest.mark.parametrize("method", ["sq", "vq"])
+def test_aggregation_by_global_id_equals_fetch_then_fused(method):
+    import f2cgt_amd
+    from f2cgt_amd import pipeline
+    lib = f2cgt_amd.load()
+    rng = np.random.default_rng(13)
+    n, d = 4000, 64
+    x = torch.from_numpy(rng.standard_normal((n, d)).astype(np.float32))
+    torch.manual_seed(4)
+    if method == "sq":
+        table, cbs = pipeline.sq_compress(x, 4, 32, sample_index=torch.arange(n))
+        configs = [(32, 4)]
+    else:
+        table, cbs = pipeline.vq_compress(x, 256, 8, sample_index=torch.arange(n))
+        configs = [(8, 256)]
+    sm = pipeline.CompressionManager({"methods": [method], "feat_dim": d, "configs": configs, "codebooks": [cbs],
+                                      "compression_data": table}, fusion=True)
+    input_nodes = dev(rng.permutation(n)[:900])
+    deg = rng.integers(0, 12, size=300)
+    indptr = np.zeros(301, dtype=np.int64)
+    indptr[1:] = np.cumsum(deg)
+    indices = rng.integers(0, 900, size=int(indptr[-1]))
+    ip, ix = dev(indptr), dev(indices)
+    rows = sm.get_all_data(input_nodes)
+    if method == "vq":
+        two_step = lib.vq_decompress_spmm_csr(rows, sm.codebooks[0], ip, ix, d)
+    else:
+        two_step = lib.sq_decompress_spmm_csr(rows, sm.codebooks[0], ip, ix, 4, 32, d)
+    assert torch.equal(sm.aggregate_global(ip, ix, input_nodes), two_step)
+
+
 def test_module_fetch_rows():
     import f2cgt_amd
     lib = f2cgt_amd.load()
