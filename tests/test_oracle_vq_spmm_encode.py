@@ -179,3 +179,20 @@ def test_golden_fixtures_reproduce(golden):
                           g["hy_fused"])
     for metric in ("l2", "cosine"):
         assert np.array_equal(oc.kmeans_predict(g["enc_x"], g["enc_c"], metric)[0], g["enc_labels_" + metric])
+
+
+# ---- row fetch of the feature cache --------------------------------------------------------
+def test_fetch_rows_is_index_select_and_a_cache_of_copies_changes_nothing():
+    rng = np.random.default_rng(21)
+    table = rng.integers(0, 256, size=(500, 7), dtype=np.uint8)
+    index = rng.integers(0, 500, size=300)
+    want = torch.index_select(torch.from_numpy(table), 0, torch.from_numpy(index)).numpy()
+    assert np.array_equal(oc.fetch_rows(table, index), want)
+    hot_ids = rng.permutation(500)[:120]
+    slot_map = np.full(500, -1, dtype=np.int32)
+    slot_map[hot_ids] = np.arange(120, dtype=np.int32)
+    assert np.array_equal(oc.fetch_rows(table, index, table[hot_ids], slot_map), want)
+    # rows that have a slot come from the cache, the others from the table
+    marked = oc.fetch_rows(table, index, np.zeros((120, 7), dtype=np.uint8), slot_map)
+    cached = slot_map[index] >= 0
+    assert not marked[cached].any() and np.array_equal(marked[~cached], want[~cached])
