@@ -139,3 +139,18 @@ def test_full_size_encode():
     # idempotence: assigning the centres to themselves gives the identity
     ident = capi.kmeans_predict(enc["centers"], enc["centers"], "l2")
     assert torch.equal(ident.cpu(), torch.arange(enc["n"]))
+
+
+@pytest.mark.parametrize("name", ["c2", "c3", "c5"])
+def test_full_size_fetch_then_fused_equals_fused_on_global_ids(name):
+    """The reference's flow (fetch the code rows of the block's source nodes, run the fused
+    operator on local indices) against the fused operator on global ids, at full size."""
+    wl = synth.WORKLOADS[name](device="cuda")
+    uniq, inv = torch.unique(wl["indices"], return_inverse=True)
+    rows = capi.fetch_rows(wl["codes"], uniq)
+    assert torch.equal(rows, wl["codes"][uniq])
+    if wl["kind"] == "vq":
+        local = capi.vq_decompress_spmm_csr(rows, wl["codebooks"], wl["indptr"], inv, wl["feat_dim"])
+    else:
+        local = capi.sq_affine_decompress_spmm_csr(rows, wl["params"], wl["indptr"], inv, wl["bits"], wl["feat_dim"])
+    assert torch.equal(local, _fused(wl))
