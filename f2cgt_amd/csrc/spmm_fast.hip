@@ -269,6 +269,7 @@ struct AccArgs {
   int fin_group;     // finalize: lanes per row (min(f4_per_row, block))
   int fin_slots;     // finalize: rows per pass
   uint32_t fin_magic;  // ceil(2^16 / fin_group)
+  int nt_out;        // output larger than the last-level cache: non-temporal stores
 };
 
 template <int TB, int BITS>
@@ -449,7 +450,8 @@ __device__ __forceinline__ void acc_finalize(const AccArgs& a, const FinParams& 
       if (rdeg == 0.f) v0 = v1 = v2 = v3 = 0.f;
       // plain stores: rows are not cache-line multiples in general, and the L2 merges the partial
       // lines that neighbouring waves write before they go to HBM
-      *reinterpret_cast<float4*>(o + (int64_t)r * a.feat_dim) = make_float4(v0, v1, v2, v3);
+      if (a.nt_out) store_nt4(o + (int64_t)r * a.feat_dim, v0, v1, v2, v3);
+      else *reinterpret_cast<float4*>(o + (int64_t)r * a.feat_dim) = make_float4(v0, v1, v2, v3);
     }
   }
 }
@@ -557,6 +559,7 @@ int launch_acc_tb(AccArgs a, size_t lds, int64_t grid, const void* indptr, const
   a.fin_group = a.f4_per_row < TB ? a.f4_per_row : TB;
   a.fin_slots = TB / a.fin_group;
   a.fin_magic = (uint32_t)((65536 + a.fin_group - 1) / a.fin_group);
+  a.nt_out = stream_output(a.R * (int64_t)a.feat_dim * 4) ? 1 : 0;
   if (idx_dtype == F2CGT_DT_I32)
     sq_affine_acc_kernel<TB, BITS, int32_t><<<(unsigned)grid, TB, lds, st>>>(
         a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
@@ -621,6 +624,7 @@ struct RowsArgs {
   int lanes, lane_shift;
   int f4_per_row, fin_group, fin_slots;
   uint32_t fin_magic;
+  int nt_out;            // output larger than the last-level cache: non-temporal stores
 };
 
 constexpr int kRowsBlock = 128;
@@ -813,7 +817,8 @@ __global__ __launch_bounds__(kRowsBlock) void sq_rows_kernel(RowsArgs a, const I
         rc = __fmaf_rn(__fmaf_rn(-d, rc, 1.f), rc, rc);
         s0 = mean_of(s0, d, rc); s1 = mean_of(s1, d, rc); s2 = mean_of(s2, d, rc); s3 = mean_of(s3, d, rc);
       }
-      *reinterpret_cast<float4*>(o + (int64_t)r * a.feat_dim) = make_float4(s0, s1, s2, s3);
+      if (a.nt_out) store_nt4(o + (int64_t)r * a.feat_dim, s0, s1, s2, s3);
+      else *reinterpret_cast<float4*>(o + (int64_t)r * a.feat_dim) = make_float4(s0, s1, s2, s3);
     }
   }
 }
@@ -832,6 +837,7 @@ int launch_sq_rows(RowsArgs a, const void* indptr, const void* indices, int idx_
   a.fin_group = a.f4_per_row < TB ? a.f4_per_row : TB;
   a.fin_slots = TB / a.fin_group;
   a.fin_magic = (uint32_t)((65536 + a.fin_group - 1) / a.fin_group);
+  a.nt_out = stream_output(a.R * (int64_t)a.feat_dim * 4) ? 1 : 0;
   const size_t lut_bytes = AFFINE ? 0 : (size_t)(((a.num_codebooks << BITS) + 3) & ~3) * 4;
   int cap = (int)((20 * 1024) / (a.pitch + 4));
   a.edge_cap = (cap > 2 * TB ? 2 * TB : (cap < 8 ? 8 : cap)) & ~1;  // even: keeps the staging 8-byte aligned
