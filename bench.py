@@ -32,11 +32,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # what the same counter reads for a plain copy of known size; see profiles/).  Keyed by
 # (workload name, index dtype).  Missing = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1_sq8_affine", "int64"): 18275409,
-    ("c2_sq4_affine", "int64"): 134237487,
-    ("c3_vq_16x8", "int64"): 506816011,
-    ("c4_hybrid", "int64"): 1004036160,
-    ("c5_vq_24x32", "int64"): 2171366722,
+    ("c1_sq8_affine", "int64"): 18292815,
+    ("c2_sq4_affine", "int64"): 134406614,
+    ("c3_vq_16x8", "int64"): 506241813,
+    ("c4_hybrid", "int64"): 1003842559,
+    ("c5_vq_24x32", "int64"): 2195351693,
 }
 
 
