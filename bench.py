@@ -33,10 +33,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # (workload name, index dtype).  Missing = not measured.
 MEASURED_TRAFFIC_BYTES = {
     ("c1_sq8_affine", "int64"): 18292815,
-    ("c2_sq4_affine", "int64"): 134406614,
-    ("c3_vq_16x8", "int64"): 506241813,
-    ("c4_hybrid", "int64"): 1003842559,
-    ("c5_vq_24x32", "int64"): 2195351693,
+    ("c2_sq4_affine", "int64"): 134402391,
+    ("c3_vq_16x8", "int64"): 506323232,
+    ("c4_hybrid", "int64"): 1004036197,
+    ("c5_vq_24x32", "int64"): 2185646058,
 }
 
 
