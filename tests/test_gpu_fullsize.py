@@ -154,3 +154,23 @@ def test_full_size_fetch_then_fused_equals_fused_on_global_ids(name):
     else:
         local = capi.sq_affine_decompress_spmm_csr(rows, wl["params"], wl["indptr"], inv, wl["bits"], wl["feat_dim"])
     assert torch.equal(local, _fused(wl))
+
+
+@pytest.mark.parametrize("form", ["affine", "log"])
+def test_outputs_beyond_the_last_level_cache_take_the_streaming_stores(form):
+    """Above 220 MB of output the row-block kernels switch to non-temporal stores; the result must
+    be what the same kernel writes with plain stores, which is how each half of the rows is run."""
+    wl = synth.c2_sq4_affine(device="cuda", R=800_000)              # 320 MB of output
+    indptr, indices, d = wl["indptr"], wl["indices"], wl["feat_dim"]
+    if form == "affine":
+        run = lambda ip, ix: capi.sq_affine_decompress_spmm_csr(wl["codes"], wl["params"], ip, ix, 4, d)
+    else:
+        logcb = torch.tensor([[0.01, 3.0, -6.643856, 1.5849625, 0.4]], device="cuda")
+        run = lambda ip, ix: capi.sq_decompress_spmm_csr(wl["codes"], logcb, ip, ix, 4, d, d)
+    full = run(indptr, indices)
+    half = wl["R"] // 2
+    e_half = int(indptr[half])
+    first = run(indptr[:half + 1].contiguous(), indices[:e_half].contiguous())
+    second = run((indptr[half:] - e_half).contiguous(), indices[e_half:].contiguous())
+    assert full.shape[0] * d * 4 > 220_000_000 > first.shape[0] * d * 4
+    assert torch.equal(full, torch.cat([first, second]))
