@@ -189,6 +189,13 @@ def _others(idx):
                                   "algorithmic_TFLOPps": tf, "executed_bf16_mfma_TFLOPps": 6 * tf,
                                   "frac_mfma_bf16_peak": 6 * tf / MFMA_BF16_PEAK_TFLOPS,
                                   "algorithmic_over_f32_mfma_peak": tf / MFMA_F32_PEAK_TFLOPS}
+    # the distance matrix itself (pairwise_distance): 9..64 dimensions go through the same split-bf16
+    # matrix-core evaluation as the assignment; the 1.02 GB matrix write is the bound
+    for metric in ("l2", "cosine"):
+        _, t = _time_steps(lambda: capi.pairwise_distance(enc["x"], enc["centers"], metric), 20, 3)
+        res["c5_pairwise_distance_" + metric] = {"launch_us": t * 1e3,
+                                                 "matrix_write_GBps": enc["m"] * enc["n"] * 4 / (t * 1e-3) / 1e9,
+                                                 "frac_hbm_peak": enc["m"] * enc["n"] * 4 / (t * 1e-3) / 1e9 / HBM_PEAK_GBS}
     # streaming ops at the C2 table shape
     n, d = 2_400_000, 100
     codes = torch.randint(0, 16, (n, d), dtype=torch.uint8, device="cuda")

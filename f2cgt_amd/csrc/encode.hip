@@ -517,12 +517,38 @@ __device__ int exact_argmin_row_cosine_pieces(const float* __restrict__ xrow, fl
   return besti;
 }
 
-template <int S, int NB>
+// One distance by the whole wave in fp64 (lane t takes dimensions t, t + 64, ...): the entries of
+// the distance matrix that the expanded form cannot give (x almost equal to y, vectors without a
+// direction for cosine).
+__device__ __noinline__ float exact_pair(const float* __restrict__ xr, const float* __restrict__ yr, int k,
+                                         bool cosine, int lane) {
+  double a = 0.0, b = 0.0, c = 0.0;
+  for (int t = lane; t < k; t += 64) {
+    const double xv = (double)xr[t], yv = (double)yr[t];
+    if (cosine) { a += xv * yv; b += xv * xv; c += yv * yv; }
+    else { const double d = xv - yv; a += d * d; }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    a += __shfl_xor(a, off);
+    b += __shfl_xor(b, off);
+    c += __shfl_xor(c, off);
+  }
+  if (!cosine) return (float)a;
+  double den = sqrt(b) * sqrt(c);
+  den = den > 1e-8 ? den : 1e-8;
+  return (float)(1.0 - a / den);
+}
+
+// PW = false: labels of the nearest centre (KMeans.predict).  PW = true: the distance matrix itself
+// (pairwise_distance), dist[row * ldd + centre], from the same scores.
+template <int S, int NB, bool PW>
 __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restrict__ x,
                                                             const float* __restrict__ centers,
                                                             int64_t* __restrict__ lab64,
                                                             uint8_t* __restrict__ lab8, int64_t m,
-                                                            int n, int k, int metric, int n_pad) {
+                                                            int n, int k, int metric, int n_pad,
+                                                            float* __restrict__ dist, int64_t ldd) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   const int n_ct = n_pad >> 5;                                   // 32-centre tiles
   bf16x8* ap = reinterpret_cast<bf16x8*>(smem_raw);              // [3][n_ct][S][64]
@@ -530,8 +556,10 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
   float* inv = bias + n_pad;                                     // [n_pad] 1 / |c| (cosine) or 1
   int* cmax_bits = reinterpret_cast<int*>(inv + n_pad);
   float* xs = reinterpret_cast<float*>(cmax_bits + 4) + (threadIdx.x >> 6) * 16 * S;   // one row of x per wave
+  constexpr int kTrPitch = 36;
+  float* tr = reinterpret_cast<float*>(cmax_bits + 4) + 4 * 16 * S + (threadIdx.x >> 6) * 32 * kTrPitch;   // PW only
   const bool cosine = metric == F2CGT_METRIC_COSINE;
-  if (threadIdx.x == 0) { cmax_bits[0] = 0; cmax_bits[1] = 0; cmax_bits[2] = 0; }
+  if (threadIdx.x == 0) { cmax_bits[0] = 0; cmax_bits[1] = 0; cmax_bits[2] = 0; cmax_bits[3] = 0x7f800000; }
   // Staging works on items (centre, chunk of 8 dimensions) = one half-operand, four items per
   // thread with their loads issued together: first the sums of squares of the chunks, then, once
   // the norms are known, the pieces.  Dimensions from k on and centres from n on read as zeros.
@@ -582,6 +610,7 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
     bias[jj] = jj >= n ? INFINITY : (cosine ? 0.f : cn);
     if (jj < n && !cosine) atomicMax(cmax_bits, __float_as_int(cn));
     if (jj < n && cosine && !(cn > 1e-12f)) atomicOr(cmax_bits + 1, 1);   // a centre without a direction
+    if (PW && jj < n && cosine) atomicMin(cmax_bits + 3, __float_as_int(cn));
   }
   __syncthreads();
   for (int i0 = threadIdx.x; i0 < n_items; i0 += blockDim.x * 4) {
@@ -614,6 +643,7 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
   __syncthreads();
   const float cmax = __int_as_float(cmax_bits[0]);
   const bool plain_cosine = cmax_bits[1] != 0;   // degenerate centres: no candidate filter for cosine
+  const float cmin_norm = sqrtf(__int_as_float(cmax_bits[3]));   // PW, cosine: smallest |c|
 
   const int lane = threadIdx.x & 63;
   const int j = lane & 31;
@@ -712,13 +742,86 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
           for (int b = 0; b < NB; ++b)
             acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[pc[term]][st], xp[b][st][px[term]], acc[b], 0, 0, 0);
         }
+      if constexpr (PW) {
+        // Distances of this 32-centre tile.  L2: |x|^2 + |c|^2 - 2 x.c loses what the two vectors have
+        // in common, so an entry below an eighth of |x|^2 + |c|^2 (three bits gone) is evaluated again
+        // as sum((x - c)^2); cosine needs that only for vectors without a direction.
+        const bool vst = (ldd % 4 == 0) && ((reinterpret_cast<uintptr_t>(dist) & 15) == 0);
 #pragma unroll
-      for (int b = 0; b < NB; ++b) {
+        for (int b = 0; b < NB; ++b) {
+          const bool valid = grp * kGroupRows + 32 * b + j < m;
+          float dv[16];
+          bool redo = false;
+          if (!cosine) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[b][v] += bz[v];
-        argmin_update(acc[b], ct * 32, best[b], second[b], bv[b], bct[b]);
+            for (int v = 0; v < 16; ++v) {
+              dv[v] = (acc[b][v] + bz[v]) + xn[b];
+              redo = redo || (dv[v] < 0.125f * (xn[b] + bz[v]));
+            }
+          } else {
+            const float nx = sqrtf(xn[b]);
+            const float rx = 1.f / (nx > 1e-30f ? nx : 1e-30f);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) dv[v] = __fmaf_rn(acc[b][v], rx, 1.f);
+            // the reference form clamps |x||c| at 1e-8 from below: rows that can reach the clamp
+            redo = plain_cosine || !(xn[b] > 1e-12f) || !(nx * cmin_norm > 2e-8f);
+          }
+          if (__ballot(valid && redo)) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const bool f = valid && (cosine ? redo : (dv[v] < 0.125f * (xn[b] + bz[v])));
+              uint64_t mk = __ballot(f);
+              while (mk) {
+                const int src = __ffsll((unsigned long long)mk) - 1;
+                mk &= mk - 1;
+                const int64_t rrow = grp * kGroupRows + 32 * b + (src & 31);
+                const int cc = ct * 32 + 8 * (v >> 2) + 4 * (src >> 5) + (v & 3);
+                if (cc < n) {
+                  const float ex = exact_pair(x + rrow * k, centers + (int64_t)cc * k, k, cosine, lane);
+                  if (lane == src) dv[v] = ex;
+                }
+              }
+            }
+          }
+          // A lane holds four 16-byte pieces of its row's 128-byte segment, every other one: stored
+          // from here, an instruction would write half of each 32-byte sector.  The wave's LDS tile
+          // (32 rows, pitch 36 floats: conflict-free both ways) turns the segment around so that
+          // eight lanes store the 128 contiguous bytes of a row and an instruction covers eight rows.
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            *reinterpret_cast<float4*>(tr + j * kTrPitch + 8 * q + 4 * g) =
+                make_float4(dv[4 * q], dv[4 * q + 1], dv[4 * q + 2], dv[4 * q + 3]);
+          __builtin_amdgcn_wave_barrier();
+          const int c0 = ct * 32 + 4 * (lane & 7);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int rr = 8 * i + (lane >> 3);
+            const float4 o4 = *reinterpret_cast<const float4*>(tr + rr * kTrPitch + 4 * (lane & 7));
+            const int64_t orow_i = grp * kGroupRows + 32 * b + rr;
+            if (orow_i < m) {
+              float* o = dist + orow_i * ldd + c0;
+              if (vst && c0 + 3 < n) {
+                store_nt4(o, o4.x, o4.y, o4.z, o4.w);
+              } else {
+                if (c0 < n) o[0] = o4.x;
+                if (c0 + 1 < n) o[1] = o4.y;
+                if (c0 + 2 < n) o[2] = o4.z;
+                if (c0 + 3 < n) o[3] = o4.w;
+              }
+            }
+          }
+        }
+      } else {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[b][v] += bz[v];
+          argmin_update(acc[b], ct * 32, best[b], second[b], bv[b], bct[b]);
+        }
       }
     }
+    if constexpr (PW) continue;
     int besti[NB];
     uint64_t todo[NB];
 #pragma unroll
@@ -899,10 +1002,10 @@ int launch_mfma(const float* x, const float* centers, int64_t* l64, uint8_t* l8,
   return launch_status("kmeans_predict");
 }
 
-template <int S, int NB>
+template <int S, int NB, bool PW = false>
 int launch_split(const float* x, const float* centers, int64_t* l64, uint8_t* l8, int64_t m, int n, int k,
-                 int metric, int n_pad, size_t lds, hipStream_t st) {
-  auto kern = predict_split_kernel<S, NB>;
+                 int metric, int n_pad, size_t lds, hipStream_t st, float* dist = nullptr, int64_t ldd = 0) {
+  auto kern = predict_split_kernel<S, NB, PW>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -921,8 +1024,8 @@ int launch_split(const float* x, const float* centers, int64_t* l64, uint8_t* l8
   }
   const int64_t need = ceil_div(ceil_div(m, 32 * NB), 4);
   const int64_t cap = (int64_t)num_cus() * cached_per_cu;
-  kern<<<(int)(need < cap ? need : cap), 256, lds, st>>>(x, centers, l64, l8, m, n, k, metric, n_pad);
-  return launch_status("kmeans_predict");
+  kern<<<(int)(need < cap ? need : cap), 256, lds, st>>>(x, centers, l64, l8, m, n, k, metric, n_pad, dist, ldd);
+  return launch_status(PW ? "pairwise_distance" : "kmeans_predict");
 }
 
 }  // namespace
@@ -938,6 +1041,33 @@ extern "C" int f2cgt_pairwise_distance(const float* x, const float* y, float* di
                 "pairwise_distance: unknown metric %d", metric);
   if (m * n == 0) return 0;
   F2CGT_REQUIRE(dist && (k == 0 || (x && y)), F2CGT_E_INVALID, "pairwise_distance: null buffer");
+  {  // matrix-core path: 9..64 dimensions; y goes through LDS in chunks of up to 96 KB of operands
+    const int steps = (int)ceil_div(k, 16);
+    if (k > 8 && steps <= 4) {
+      const int64_t per32 = (int64_t)3 * steps * 64 * 16 + 2 * 32 * 4;          // bytes per 32 rows of y
+      const int64_t turn = 4 * 32 * 36 * 4;                                     // the waves' output tiles
+      int64_t chunk = ((96 * 1024 - 16 - 4 * 16 * steps * 4 - turn) / per32) * 32;
+      chunk = chunk > 512 ? 512 : chunk;
+      for (int64_t c0 = 0; c0 < n; c0 += chunk) {
+        const int nn = (int)(n - c0 < chunk ? n - c0 : chunk);
+        const int n_pad32 = (int)ceil_div(nn, 32) * 32;
+        const size_t lds = (size_t)3 * (n_pad32 / 32) * steps * 64 * 16 + (size_t)2 * n_pad32 * 4 + 16 +
+                           (size_t)4 * 16 * steps * 4 + (size_t)turn;
+        const float* yc = y + c0 * k;
+        float* dc = dist + c0;
+        hipStream_t st = as_stream(stream);
+        int rc;
+        switch (steps) {
+          case 1: rc = launch_split<1, 2, true>(x, yc, nullptr, nullptr, m, nn, (int)k, metric, n_pad32, lds, st, dc, n); break;
+          case 2: rc = launch_split<2, 2, true>(x, yc, nullptr, nullptr, m, nn, (int)k, metric, n_pad32, lds, st, dc, n); break;
+          case 3: rc = launch_split<3, 2, true>(x, yc, nullptr, nullptr, m, nn, (int)k, metric, n_pad32, lds, st, dc, n); break;
+          default: rc = launch_split<4, 2, true>(x, yc, nullptr, nullptr, m, nn, (int)k, metric, n_pad32, lds, st, dc, n); break;
+        }
+        if (rc != 0) return rc;
+      }
+      return 0;
+    }
+  }
   const int64_t tiles = ceil_div(m, kTile) * ceil_div(n, kTile);
   const int64_t cap = (int64_t)num_cus() * 8;
   pairwise_kernel<<<(int)(tiles < cap ? tiles : cap), 256, 0, as_stream(stream)>>>(x, y, dist, m, n,

@@ -557,6 +557,57 @@ def test_pairwise_distance(metric, m, n, k):
 
 
 @pytest.mark.parametrize("metric", ["l2", "cosine"])
+@pytest.mark.parametrize("m,n,k", [(5000, 256, 32), (4097, 255, 9), (700, 37, 16), (1000, 1000, 17), (321, 600, 33),
+                                   (2000, 256, 48), (999, 230, 64), (500, 100, 65), (70, 3, 24), (1, 1, 32)])
+def test_pairwise_distance_matrix_core_shapes(metric, m, n, k):
+    """9 to 64 dimensions go through the matrix cores (y in chunks that fit LDS, vector or scalar
+    stores by the row pitch); the neighbours of that range take the vector-ALU kernel."""
+    rng = np.random.default_rng(m * 7 + n * 3 + k)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    y = rng.standard_normal((n, k)).astype(np.float32)
+    got = host(capi.pairwise_distance(dev(x), dev(y), metric))
+    want = oc.pairwise_distance(x, y, metric, dtype=np.float64)
+    assert got.shape == want.shape
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("k", [16, 32, 40, 64])
+def test_pairwise_l2_between_almost_equal_points(k):
+    """|x|^2 + |y|^2 - 2 x.y cancels when x is close to y; those entries must still be the sum of
+    squared differences, to its own relative accuracy (and exactly zero for x == y)."""
+    rng = np.random.default_rng(k)
+    y = (rng.standard_normal((300, k)) * 10).astype(np.float32)
+    x = y[rng.integers(0, 300, size=2000)].copy()
+    x[:500] += (rng.standard_normal((500, k)) * 1e-3).astype(np.float32)     # close
+    x[500:1000] += (rng.standard_normal((500, k)) * 1e-6).astype(np.float32)  # mostly identical after rounding
+    x[1500:] = (rng.standard_normal((500, k)) * 10).astype(np.float32)       # far
+    got = host(capi.pairwise_distance(dev(x), dev(y), "l2"))
+    want = oc.pairwise_distance(x, y, "l2", dtype=np.float64)
+    assert np.allclose(got, want, rtol=1e-5, atol=0.0)
+    same = (x[:, None, :] == y[None, :, :]).all(axis=2)
+    assert same.any() and not got[same].any()
+
+
+def test_pairwise_cosine_with_vectors_without_a_direction():
+    rng = np.random.default_rng(8)
+    k = 32
+    x = rng.standard_normal((400, k)).astype(np.float32)
+    y = rng.standard_normal((96, k)).astype(np.float32)
+    x[3] = 0
+    x[77] *= 1e-7            # |x||y| falls below the clamp of the denominator
+    x[200] *= 1e-4
+    y[5] = 0
+    y[40] *= 1e-6
+    got = host(capi.pairwise_distance(dev(x), dev(y), "cosine"))
+    want = oc.pairwise_distance(x, y, "cosine", dtype=np.float64)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+    # without degenerate centres only the rows near the clamp take the exact path
+    y2 = rng.standard_normal((96, k)).astype(np.float32)
+    got = host(capi.pairwise_distance(dev(x), dev(y2), "cosine"))
+    assert np.allclose(got, oc.pairwise_distance(x, y2, "cosine", dtype=np.float64), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("metric", ["l2", "cosine"])
 @pytest.mark.parametrize("m,n,k", [(20000, 256, 32), (5000, 256, 8), (3001, 100, 16), (777, 37, 5),
                                    (4000, 256, 64), (500, 1000, 24), (300, 50, 200)])
 def test_kmeans_predict_vs_oracle(metric, m, n, k):
