@@ -1,8 +1,14 @@
 // VQ encode: pairwise distance and nearest-centre assignment.
 //
-// pairwise_distance materialises the [m,n] matrix; it evaluates the unexpanded form
-// sum((x-y)^2) (or 1 - cos) with fused multiply-adds on the vector ALUs, so the numbers carry
-// no cancellation error, and at small k the vector ALUs rather than the matrix write bound it.
+// pairwise_distance materialises the [m,n] matrix.  With 9 to 64 dimensions the scores come from
+// the matrix cores, as in predict_split_kernel below (its PW mode): |x|^2 + |y|^2 - 2 x.y with x.y
+// from three bf16 pieces per value, after the mean of y has been subtracted from both (L2).  That
+// form loses what x and y have in common, so an entry below an eighth of |x|^2 + |y|^2 is
+// evaluated again as sum((x-y)^2) by its lane (cosine: rows and columns whose |x||y| can reach the
+// reference's 1e-8 clamp); the 128-byte row
+// segments of a tile are turned around through LDS so that a store instruction writes whole
+// lines, and the matrix write bounds the kernel.  Other dimensions take pairwise_kernel: the
+// unexpanded form with fused multiply-adds on the vector ALUs.
 //
 // kmeans_predict never writes the matrix.  A wave owns rows of x and walks the centres a tile
 // at a time on the matrix core: A = centre tile, B = x tile, so every lane holds 16 centre
@@ -517,31 +523,12 @@ __device__ int exact_argmin_row_cosine_pieces(const float* __restrict__ xrow, fl
   return besti;
 }
 
-// One distance by the whole wave in fp64 (lane t takes dimensions t, t + 64, ...): the entries of
-// the distance matrix that the expanded form cannot give (x almost equal to y, vectors without a
-// direction for cosine).
-__device__ __noinline__ float exact_pair(const float* __restrict__ xr, const float* __restrict__ yr, int k,
-                                         bool cosine, int lane) {
-  double a = 0.0, b = 0.0, c = 0.0;
-  for (int t = lane; t < k; t += 64) {
-    const double xv = (double)xr[t], yv = (double)yr[t];
-    if (cosine) { a += xv * yv; b += xv * xv; c += yv * yv; }
-    else { const double d = xv - yv; a += d * d; }
-  }
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    a += __shfl_xor(a, off);
-    b += __shfl_xor(b, off);
-    c += __shfl_xor(c, off);
-  }
-  if (!cosine) return (float)a;
-  double den = sqrt(b) * sqrt(c);
-  den = den > 1e-8 ? den : 1e-8;
-  return (float)(1.0 - a / den);
-}
-
 // PW = false: labels of the nearest centre (KMeans.predict).  PW = true: the distance matrix itself
-// (pairwise_distance), dist[row * ldd + centre], from the same scores.
+// (pairwise_distance), dist[row * ldd + centre], from the same scores.  The squared L2 distance
+// does not change when one vector is subtracted from both arguments, and fl(v - mu) carries a
+// relative error of 2^-24 of the difference itself, so the PW mode first subtracts the mean of the
+// centres from every x and centre: data far from the origin would otherwise lose most of the
+// expanded form's bits to cancellation.
 template <int S, int NB, bool PW>
 __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restrict__ x,
                                                             const float* __restrict__ centers,
@@ -564,6 +551,22 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
   // thread with their loads issued together: first the sums of squares of the chunks, then, once
   // the norms are known, the pieces.  Dimensions from k on and centres from n on read as zeros.
   const bool cvec = (k % 8 == 0) && ((reinterpret_cast<uintptr_t>(centers) & 15) == 0);
+  // PW, L2: mu[t] = mean of the centres in dimension t (zeros otherwise), in the x slots of the waves
+  float* mu = reinterpret_cast<float*>(cmax_bits + 4);           // [16 S]
+  const bool centred = PW && !cosine;
+  if (PW) {
+    float* psum = reinterpret_cast<float*>(smem_raw);            // [4][64], overwritten by the pieces later
+    const int t = threadIdx.x & 63, part = threadIdx.x >> 6;
+    float sum = 0.f;
+    if (centred && t < k)
+      for (int c = part; c < n; c += 4) sum += centers[(int64_t)c * k + t];
+    psum[part * 64 + t] = sum;
+    __syncthreads();
+    if (threadIdx.x < 16 * S)
+      mu[threadIdx.x] = ((psum[threadIdx.x] + psum[64 + threadIdx.x]) +
+                         (psum[128 + threadIdx.x] + psum[192 + threadIdx.x])) / (float)n;
+    __syncthreads();
+  }
   auto load8 = [&](int c, int ch, float (&v)[8]) {
     const bool in = c < n && 8 * ch < k;
     const float* cr = centers + (in ? (int64_t)c * k + 8 * ch : 0);
@@ -575,6 +578,10 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
     } else {
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = (in && 8 * ch + e < k) ? cr[e] : 0.f;
+    }
+    if (PW) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = (in && 8 * ch + e < k) ? v[e] - mu[8 * ch + e] : 0.f;
     }
   };
   constexpr int kChunks = 2 * S;
@@ -690,6 +697,10 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
 #pragma unroll
           for (int e = 0; e < 8; ++e) q[e] = (valid && kk0 + e < k) ? x[row * k + kk0 + e] : 0.f;
         }
+        if constexpr (PW) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) q[e] = (valid && kk0 + e < k) ? q[e] - mu[kk0 + e] : 0.f;
+        }
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           sum += q[e] * q[e];
@@ -743,9 +754,9 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
             acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[pc[term]][st], xp[b][st][px[term]], acc[b], 0, 0, 0);
         }
       if constexpr (PW) {
-        // Distances of this 32-centre tile.  L2: |x|^2 + |c|^2 - 2 x.c loses what the two vectors have
-        // in common, so an entry below an eighth of |x|^2 + |c|^2 (three bits gone) is evaluated again
-        // as sum((x - c)^2); cosine needs that only for vectors without a direction.
+        // Distances of this 32-centre tile.  L2: |x|^2 + |c|^2 - 2 x.c (of the centred vectors) loses
+        // what the two have in common, so an entry below an eighth of |x|^2 + |c|^2 (three bits gone)
+        // is evaluated again as sum((x - c)^2); cosine needs that only near the clamp of |x||c|.
         const bool vst = (ldd % 4 == 0) && ((reinterpret_cast<uintptr_t>(dist) & 15) == 0);
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
@@ -767,20 +778,50 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
             redo = plain_cosine || !(xn[b] > 1e-12f) || !(nx * cmin_norm > 2e-8f);
           }
           if (__ballot(valid && redo)) {
+            // every lane evaluates its own flagged entries in the unexpanded fp32 form, one per trip
+            // of a loop that exists once in the code (the entry's slot is a lane-varying index)
+            uint32_t fm = 0;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-              const bool f = valid && (cosine ? redo : (dv[v] < 0.125f * (xn[b] + bz[v])));
-              uint64_t mk = __ballot(f);
-              while (mk) {
-                const int src = __ffsll((unsigned long long)mk) - 1;
-                mk &= mk - 1;
-                const int64_t rrow = grp * kGroupRows + 32 * b + (src & 31);
-                const int cc = ct * 32 + 8 * (v >> 2) + 4 * (src >> 5) + (v & 3);
-                if (cc < n) {
-                  const float ex = exact_pair(x + rrow * k, centers + (int64_t)cc * k, k, cosine, lane);
-                  if (lane == src) dv[v] = ex;
+            for (int v = 0; v < 16; ++v)
+              if (valid && (cosine ? redo : (dv[v] < 0.125f * (xn[b] + bz[v])))) fm |= 1u << v;
+            const float* xr = x + (grp * kGroupRows + 32 * b + j) * k;
+#pragma nounroll
+            while (__ballot(fm != 0)) {
+              const int vl = fm ? __ffs((int)fm) - 1 : 0;
+              const int cc = ct * 32 + 8 * (vl >> 2) + 4 * g + (vl & 3);
+              const bool on = fm != 0 && cc < n;
+              fm &= fm - 1;
+              float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+              if (on) {
+                const float* yr = centers + (int64_t)cc * k;
+                auto term = [&](float xv, float yv) {
+                  if (cosine) {
+                    s0 = __fmaf_rn(xv, yv, s0);
+                    s1 = __fmaf_rn(xv, xv, s1);
+                    s2 = __fmaf_rn(yv, yv, s2);
+                  } else {
+                    const float d = xv - yv;
+                    s0 = __fmaf_rn(d, d, s0);
+                  }
+                };
+                if (vec4 && cvec) {        // eight dimensions per trip, their loads issued together
+                  for (int t = 0; t < k; t += 8) {
+                    const float4 xa = *reinterpret_cast<const float4*>(xr + t), xb = *reinterpret_cast<const float4*>(xr + t + 4);
+                    const float4 ya = *reinterpret_cast<const float4*>(yr + t), yb = *reinterpret_cast<const float4*>(yr + t + 4);
+                    term(xa.x, ya.x); term(xa.y, ya.y); term(xa.z, ya.z); term(xa.w, ya.w);
+                    term(xb.x, yb.x); term(xb.y, yb.y); term(xb.z, yb.z); term(xb.w, yb.w);
+                  }
+                } else {
+                  for (int t = 0; t < k; ++t) term(xr[t], yr[t]);
+                }
+                if (cosine) {
+                  float den = sqrtf(s1) * sqrtf(s2);
+                  den = den > 1e-8f ? den : 1e-8f;
+                  s0 = 1.f - s0 / den;
                 }
               }
+#pragma unroll
+              for (int v = 0; v < 16; ++v) dv[v] = (on && vl == v) ? s0 : dv[v];
             }
           }
           // A lane holds four 16-byte pieces of its row's 128-byte segment, every other one: stored
