@@ -94,6 +94,23 @@ def main():
         assert not near.any()
         out["enc_labels_" + metric] = labels
 
+    # a wider encode case (24 dimensions: the matrix-core path of the distance matrix)
+    wx = (rng.standard_normal((50, 24)) + 2.0).astype(np.float32)
+    wc = (rng.standard_normal((40, 24)) + 2.0).astype(np.float32)
+    out["enc24_x"], out["enc24_c"] = wx, wc
+    for metric in ("l2", "cosine"):
+        out["enc24_dist_" + metric] = oc.pairwise_distance(wx, wc, metric, dtype=np.float64)
+
+    # row fetch of the feature cache: 50-byte rows, a third of the ids cached with other bytes
+    ft = rng.integers(0, 256, size=(30, 50), dtype=np.uint8)
+    fi = rng.integers(0, 30, size=21).astype(np.int64)
+    fslot = np.full(30, -1, dtype=np.int32)
+    fslot[::3] = np.arange(10, dtype=np.int32)
+    fhot = rng.integers(0, 256, size=(10, 50), dtype=np.uint8)
+    out.update(fetch_table=ft, fetch_index=fi, fetch_slot=fslot, fetch_hot=fhot)
+    out["fetch_plain"] = oc.fetch_rows(ft, fi)
+    out["fetch_cached"] = oc.fetch_rows(ft, fi, fhot, fslot)
+
     path = os.path.join(HERE, "f2cgt_golden.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes,", len(out), "arrays")

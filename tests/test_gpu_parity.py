@@ -70,6 +70,11 @@ def test_golden_fixtures(golden):
         assert np.allclose(d, g["enc_dist_" + metric], rtol=1e-5, atol=1e-5)
         assert np.array_equal(host(capi.kmeans_predict(dev(g["enc_x"]), dev(g["enc_c"]), metric)),
                               g["enc_labels_" + metric])
+        d = host(capi.pairwise_distance(dev(g["enc24_x"]), dev(g["enc24_c"]), metric))
+        assert np.allclose(d, g["enc24_dist_" + metric], rtol=1e-5, atol=1e-6)
+    ft, fi = dev(g["fetch_table"]), dev(g["fetch_index"])
+    assert np.array_equal(host(capi.fetch_rows(ft, fi)), g["fetch_plain"])
+    assert np.array_equal(host(capi.fetch_rows(ft, fi, dev(g["fetch_hot"]), dev(g["fetch_slot"]))), g["fetch_cached"])
 
 
 # ---- packbits / unpackbits -------------------------------------------------------------------

@@ -179,6 +179,12 @@ def test_golden_fixtures_reproduce(golden):
                           g["hy_fused"])
     for metric in ("l2", "cosine"):
         assert np.array_equal(oc.kmeans_predict(g["enc_x"], g["enc_c"], metric)[0], g["enc_labels_" + metric])
+        assert np.array_equal(oc.pairwise_distance(g["enc24_x"], g["enc24_c"], metric, dtype=np.float64),
+                              g["enc24_dist_" + metric])
+    assert np.array_equal(oc.fetch_rows(g["fetch_table"], g["fetch_index"]), g["fetch_plain"])
+    assert np.array_equal(oc.fetch_rows(g["fetch_table"], g["fetch_index"], g["fetch_hot"], g["fetch_slot"]),
+                          g["fetch_cached"])
+    assert np.array_equal(g["fetch_plain"], g["fetch_table"][g["fetch_index"]])
 
 
 # ---- row fetch of the feature cache --------------------------------------------------------
