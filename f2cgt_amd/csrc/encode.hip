@@ -10,7 +10,10 @@
 // lines, and the matrix write bounds the kernel.  Other dimensions take pairwise_kernel: the
 // unexpanded form with fused multiply-adds on the vector ALUs.
 //
-// kmeans_predict never writes the matrix.  A wave owns rows of x and walks the centres a tile
+// kmeans_predict never writes the matrix.  For L2 it works, like pairwise_distance, on x - mu and
+// c - mu (mu = mean of the centres): a common offset of the data then costs nothing, and the rows
+// whose best two centres are closer than the rounding of that subtraction are decided from the
+// original arrays.  A wave owns rows of x and walks the centres a tile
 // at a time on the matrix core: A = centre tile, B = x tile, so every lane holds 16 centre
 // scores of ONE x row per tile and the running arg-min stays in registers.  Scores use the
 // expanded form (|c|^2 - 2 x.c, the row constant |x|^2 dropped); rows whose two best scores are
@@ -322,13 +325,19 @@ __device__ __forceinline__ void split3(float v, __bf16& p0, __bf16& p1, __bf16& 
 // fp32 centre, exactly); same result as exact_argmin_row on the array in HBM.  The unexpanded fp32
 // distance has relative error <= (k + 3) 2^-24 (all terms positive), so it decides which centres
 // can be the minimum at all; only those, usually two, are evaluated in fp64.
+// The pieces hold the centres minus mu and the row is compared as fl(x - mu): the decision is exact
+// for those rounded vectors, whose distances differ from the original ones by at most
+// 2^-22 (|x - mu|^2 + |c - mu|^2) each.  When the best two are closer than twice that, the original
+// row decides between them (fp64, from the arrays in HBM); with three or more that close the
+// function returns -1 - (its choice) and the caller evaluates every centre.
 template <int S>
 __device__ int exact_argmin_row_l2_pieces(const float* __restrict__ xrow, float* xs, const bf16x8* ap, int n, int n_ct,
-                                          int k, int lane) {
+                                          int k, int lane, const float* mu, float cmax,
+                                          const float* __restrict__ centers) {
   // the row goes through a wave-private LDS slot (16 S floats, zero padded) and the loops over the
   // 8-dimension chunks stay rolled: this rare path must not raise the kernel's register count
   const int piece_stride = n_ct * S * 64;                // operands per piece
-  if (lane < 16 * S) xs[lane] = lane < k ? xrow[lane] : 0.f;
+  if (lane < 16 * S) xs[lane] = lane < k ? xrow[lane] - mu[lane] : 0.f;
   __builtin_amdgcn_wave_barrier();                       // LDS operations of one wave execute in order
   // fp32 centre values of chunk ch (dimensions [8 ch, 8 ch + 8)) of centre c: one operand per piece
   auto centre8 = [&](int c, int ch, float (&cv)[8]) {
@@ -418,7 +427,11 @@ __device__ int exact_argmin_row_l2_pieces(const float* __restrict__ xrow, float*
     dmin = fminf(dmin, __shfl_xor(dmin, off));
     xnorm2 += __shfl_xor(xnorm2, off);
   }
-  const float reach = (sqrtf(dmin) + 0.0078125f * sqrtf(xnorm2)) * 1.015625f;
+  // centres whose exact distance is within `margin` of the smallest must reach the fp64 stage, so
+  // that everything left out is known to be farther than that (2^-21 = 4.77e-7; the constants
+  // leave room for the fp32 evaluation of the norms)
+  const float marginf = 5.2e-7f * (xnorm2 + cmax);
+  const float reach = (sqrtf(dmin) + 0.0078125f * sqrtf(xnorm2) + sqrtf(marginf)) * 1.015625f;
   const float lead_limit = reach * reach * 1.0001f + 1e-37f;
   // second pass: full fp32 distance of the survivors, then the exact fp64 one of those that can
   // still be the minimum (relative error of the fp32 sum <= (k + 3) 2^-24, all terms positive)
@@ -434,9 +447,9 @@ __device__ int exact_argmin_row_l2_pieces(const float* __restrict__ xrow, float*
     if (dist_lead(c) <= lead_limit) d32min = fminf(d32min, dist32(c));
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) d32min = fminf(d32min, __shfl_xor(d32min, off));
-  const float limit = d32min * (1.f + 1.1920929e-7f * (float)(k + 4)) + 1e-37f;
-  double bestv = DBL_MAX;
-  int besti = INT_MAX;
+  const float limit = d32min * (1.f + 1.1920929e-7f * (float)(k + 4)) + 1e-37f + marginf;
+  double bestv = DBL_MAX, nextv = DBL_MAX, thirdv = DBL_MAX;   // the three smallest exact distances
+  int besti = INT_MAX, nexti = INT_MAX;
   for (int c = lane, i = 0; c < n; c += kWave, ++i) {
     float d32 = dkeep[0];
 #pragma unroll
@@ -454,15 +467,47 @@ __device__ int exact_argmin_row_l2_pieces(const float* __restrict__ xrow, float*
         dd += df * df;
       }
     }
-    if (dd < bestv) { bestv = dd; besti = c; }
+    if (dd < bestv) { thirdv = nextv; nextv = bestv; nexti = besti; bestv = dd; besti = c; }
+    else if (dd < nextv) { thirdv = nextv; nextv = dd; nexti = c; }
+    else if (dd < thirdv) thirdv = dd;
+  }
+  // merge of two sorted triples (a lane's centres ascend, and ties go to the smaller index)
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const double ob = __shfl_xor(bestv, off), on = __shfl_xor(nextv, off), ot = __shfl_xor(thirdv, off);
+    const int oi = __shfl_xor(besti, off), oj = __shfl_xor(nexti, off);
+    double m1, m2, m3;
+    int i1, i2;
+    if (ob < bestv || (ob == bestv && oi < besti)) {       // the other triple leads
+      m1 = ob; i1 = oi;
+      if (on < bestv || (on == bestv && oj < besti)) { m2 = on; i2 = oj; m3 = ot < bestv ? ot : bestv; }
+      else { m2 = bestv; i2 = besti; m3 = on < nextv ? on : nextv; }
+    } else {
+      m1 = bestv; i1 = besti;
+      if (ob < nextv || (ob == nextv && oi < nexti)) { m2 = ob; i2 = oi; m3 = on < nextv ? on : nextv; }
+      else { m2 = nextv; i2 = nexti; m3 = ob < thirdv ? ob : thirdv; }
+    }
+    bestv = m1; besti = i1; nextv = m2; nexti = i2; thirdv = m3;
+  }
+  const double margin = 4.9e-7 * ((double)xnorm2 + (double)cmax);
+  if (nextv - bestv > margin) return besti;              // also the only candidate (nextv = DBL_MAX)
+  if (thirdv - bestv <= margin) return -1 - besti;       // three or more: the caller takes every centre
+  // exactly two centres can be the nearest one of the original row: decide between them there
+  double da = 0.0, db = 0.0;
+  for (int t = lane; t < k; t += kWave) {
+    const double xv = (double)xrow[t];
+    const double ea = xv - (double)centers[(int64_t)besti * k + t], eb = xv - (double)centers[(int64_t)nexti * k + t];
+    da += ea * ea;
+    db += eb * eb;
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
-    const double ov = __shfl_xor(bestv, off);
-    const int oi = __shfl_xor(besti, off);
-    if (ov < bestv || (ov == bestv && oi < besti)) { bestv = ov; besti = oi; }
+    da += __shfl_xor(da, off);
+    db += __shfl_xor(db, off);
   }
-  return besti;
+  const int lo = besti < nexti ? besti : nexti, hi = besti < nexti ? nexti : besti;
+  const double dlo = besti < nexti ? da : db, dhi = besti < nexti ? db : da;
+  return dhi < dlo ? hi : lo;
 }
 
 // Exact cosine assignment of one row by a whole wave.  The LDS pieces hold the centres divided by
@@ -526,9 +571,9 @@ __device__ int exact_argmin_row_cosine_pieces(const float* __restrict__ xrow, fl
 // PW = false: labels of the nearest centre (KMeans.predict).  PW = true: the distance matrix itself
 // (pairwise_distance), dist[row * ldd + centre], from the same scores.  The squared L2 distance
 // does not change when one vector is subtracted from both arguments, and fl(v - mu) carries a
-// relative error of 2^-24 of the difference itself, so the PW mode first subtracts the mean of the
-// centres from every x and centre: data far from the origin would otherwise lose most of the
-// expanded form's bits to cancellation.
+// relative error of 2^-24 of the difference itself, so for L2 both modes first subtract the mean of
+// the centres from every x and centre: data far from the origin would otherwise lose most of the
+// expanded form's bits to cancellation (and send most rows to the exact re-evaluation).
 template <int S, int NB, bool PW>
 __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restrict__ x,
                                                             const float* __restrict__ centers,
@@ -543,24 +588,53 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
   float* inv = bias + n_pad;                                     // [n_pad] 1 / |c| (cosine) or 1
   int* cmax_bits = reinterpret_cast<int*>(inv + n_pad);
   float* xs = reinterpret_cast<float*>(cmax_bits + 4) + (threadIdx.x >> 6) * 16 * S;   // one row of x per wave
+  float* mu = reinterpret_cast<float*>(cmax_bits + 4) + 4 * 16 * S;                    // [16 S]
   constexpr int kTrPitch = 36;
-  float* tr = reinterpret_cast<float*>(cmax_bits + 4) + 4 * 16 * S + (threadIdx.x >> 6) * 32 * kTrPitch;   // PW only
+  float* tr = mu + 16 * S + (threadIdx.x >> 6) * 32 * kTrPitch;                        // PW only
   const bool cosine = metric == F2CGT_METRIC_COSINE;
   if (threadIdx.x == 0) { cmax_bits[0] = 0; cmax_bits[1] = 0; cmax_bits[2] = 0; cmax_bits[3] = 0x7f800000; }
   // Staging works on items (centre, chunk of 8 dimensions) = one half-operand, four items per
   // thread with their loads issued together: first the sums of squares of the chunks, then, once
   // the norms are known, the pieces.  Dimensions from k on and centres from n on read as zeros.
   const bool cvec = (k % 8 == 0) && ((reinterpret_cast<uintptr_t>(centers) & 15) == 0);
-  // PW, L2: mu[t] = mean of the centres in dimension t (zeros otherwise), in the x slots of the waves
-  float* mu = reinterpret_cast<float*>(cmax_bits + 4);           // [16 S]
-  const bool centred = PW && !cosine;
-  if (PW) {
+  // L2: mu[t] = mean of the centres in dimension t, subtracted from every centre and every x (the
+  // distances do not change, the cancellation of the expanded form does); zeros for cosine
+  const bool centred = !cosine;
+  {
     float* psum = reinterpret_cast<float*>(smem_raw);            // [4][64], overwritten by the pieces later
-    const int t = threadIdx.x & 63, part = threadIdx.x >> 6;
-    float sum = 0.f;
-    if (centred && t < k)
-      for (int c = part; c < n; c += 4) sum += centers[(int64_t)c * k + t];
-    psum[part * 64 + t] = sum;
+    const int t = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    if (centred && cvec) {
+      // a lane sums a float4 column of every 16th row, eight loads in flight; the four row groups of
+      // a wave are added with shuffles
+      const int col = t & 15, part = threadIdx.x >> 4;
+      float4 a4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (4 * col < k) {
+        const float* base = centers + 4 * col;
+        int c = part;
+        for (; c + 16 * 7 < n; c += 16 * 8) {
+          float4 v[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(base + (int64_t)(c + 16 * u) * k);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) { a4.x += v[u].x; a4.y += v[u].y; a4.z += v[u].z; a4.w += v[u].w; }
+        }
+        for (; c < n; c += 16) {
+          const float4 v = *reinterpret_cast<const float4*>(base + (int64_t)c * k);
+          a4.x += v.x; a4.y += v.y; a4.z += v.z; a4.w += v.w;
+        }
+      }
+#pragma unroll
+      for (int off = 16; off <= 32; off <<= 1) {
+        a4.x += __shfl_xor(a4.x, off); a4.y += __shfl_xor(a4.y, off);
+        a4.z += __shfl_xor(a4.z, off); a4.w += __shfl_xor(a4.w, off);
+      }
+      if (t < 16) *reinterpret_cast<float4*>(psum + wv * 64 + 4 * t) = a4;
+    } else {
+      float sum = 0.f;
+      if (centred && t < k)
+        for (int c = wv; c < n; c += 4) sum += centers[(int64_t)c * k + t];
+      psum[wv * 64 + t] = sum;
+    }
     __syncthreads();
     if (threadIdx.x < 16 * S)
       mu[threadIdx.x] = ((psum[threadIdx.x] + psum[64 + threadIdx.x]) +
@@ -579,10 +653,8 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = (in && 8 * ch + e < k) ? cr[e] : 0.f;
     }
-    if (PW) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = (in && 8 * ch + e < k) ? v[e] - mu[8 * ch + e] : 0.f;
-    }
+    for (int e = 0; e < 8; ++e) v[e] = (in && 8 * ch + e < k) ? v[e] - mu[8 * ch + e] : 0.f;
   };
   constexpr int kChunks = 2 * S;
   const int n_items = n_pad * kChunks;
@@ -660,9 +732,9 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
   // Error bound of one score in units of 2^-24 (|x|^2 + max |c|^2), which is >= 2 |x||c| = P and
   // >= |c|^2: each of the S leading instructions cuts its 17 addends at 2^-22 of the largest
   // (<= P): 68 S; the small pairs (2^-8 P and below) together stay below 4; the bias sum k + 1;
-  // its addition 2; the dropped pairs (2^-24 P each way) 2; 3 spare.  Doubled for the two scores
-  // of a gap.
-  const float unit = 5.9604645e-8f * (float)(2 * (68 * S + k + 12));
+  // its addition 2; the dropped pairs (2^-24 P each way) 2; the rounding of x - mu and c - mu 4
+  // (L2: 2^-22 (|x|^2 + |c|^2)); 3 spare.  Doubled for the two scores of a gap.
+  const float unit = 5.9604645e-8f * (float)(2 * (68 * S + k + 16));
   const float xscale = cosine ? -1.f : -2.f;
   const bool vec4 = (k % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
   // A workgroup owns a contiguous share of the row groups and its four waves draw from it through
@@ -697,10 +769,8 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
 #pragma unroll
           for (int e = 0; e < 8; ++e) q[e] = (valid && kk0 + e < k) ? x[row * k + kk0 + e] : 0.f;
         }
-        if constexpr (PW) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) q[e] = (valid && kk0 + e < k) ? q[e] - mu[kk0 + e] : 0.f;
-        }
+        for (int e = 0; e < 8; ++e) q[e] = (valid && kk0 + e < k) ? q[e] - mu[kk0 + e] : 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           sum += q[e] * q[e];
@@ -897,7 +967,10 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
         td &= td - 1;
         const int64_t rrow = grp * kGroupRows + 32 * b + (src & 31);
         int exact;
-        if (!cosine) exact = exact_argmin_row_l2_pieces<S>(x + rrow * k, xs, ap, n, n_ct, k, lane);
+        if (!cosine) {
+          exact = exact_argmin_row_l2_pieces<S>(x + rrow * k, xs, ap, n, n_ct, k, lane, mu, cmax, centers);
+          if (exact < 0) exact = exact_argmin_row(x + rrow * k, centers, n, k, metric, lane);   // the original row decides
+        }
         else if (plain_cosine) exact = exact_argmin_row(x + rrow * k, centers, n, k, metric, lane);
         else exact = exact_argmin_row_cosine_pieces<S>(x + rrow * k, xs, ap, centers, n, n_ct, k, lane);
 #pragma unroll
@@ -1087,13 +1160,13 @@ extern "C" int f2cgt_pairwise_distance(const float* x, const float* y, float* di
     if (k > 8 && steps <= 4) {
       const int64_t per32 = (int64_t)3 * steps * 64 * 16 + 2 * 32 * 4;          // bytes per 32 rows of y
       const int64_t turn = 4 * 32 * 36 * 4;                                     // the waves' output tiles
-      int64_t chunk = ((96 * 1024 - 16 - 4 * 16 * steps * 4 - turn) / per32) * 32;
+      int64_t chunk = ((96 * 1024 - 16 - 5 * 16 * steps * 4 - turn) / per32) * 32;
       chunk = chunk > 512 ? 512 : chunk;
       for (int64_t c0 = 0; c0 < n; c0 += chunk) {
         const int nn = (int)(n - c0 < chunk ? n - c0 : chunk);
         const int n_pad32 = (int)ceil_div(nn, 32) * 32;
         const size_t lds = (size_t)3 * (n_pad32 / 32) * steps * 64 * 16 + (size_t)2 * n_pad32 * 4 + 16 +
-                           (size_t)4 * 16 * steps * 4 + (size_t)turn;
+                           (size_t)5 * 16 * steps * 4 + (size_t)turn;
         const float* yc = y + c0 * k;
         float* dc = dist + c0;
         hipStream_t st = as_stream(stream);
@@ -1134,7 +1207,7 @@ extern "C" int f2cgt_kmeans_predict(const float* x, const float* centers, int64_
     const int steps = (int)ceil_div(k, 16);
     const int n_pad32 = (int)ceil_div(n, 32) * 32;
     const size_t lds = (size_t)3 * (n_pad32 / 32) * steps * 64 * 16 + (size_t)2 * n_pad32 * 4 + 16 +
-                       (size_t)4 * 16 * steps * 4;
+                       (size_t)5 * 16 * steps * 4;
     if (steps <= 4 && lds <= 96 * 1024) {
       switch (steps) {
         case 1: return launch_split<1, 2>(x, centers, labels_i64, labels_u8, m, (int)n, (int)k, metric, n_pad32, lds, st);

@@ -684,6 +684,43 @@ def test_kmeans_predict_few_dimensions_many_close_centres(k, n):
     assert np.array_equal(gotc[~nearc], wantc[~nearc])
 
 
+@pytest.mark.parametrize("offset", [0.0, 1000.0])
+def test_kmeans_predict_l2_exact_ties_far_from_the_origin(offset):
+    """The L2 kernel works on x - mu and c - mu; ties and near-ties of the original rows must still
+    be decided as the original rows say: an exact tie goes to the first centre, a centre that is
+    closer by a few units in the last place wins."""
+    rng = np.random.default_rng(17)
+    k, m = 32, 32
+    p = (offset + rng.integers(-10, 11, size=(m, k))).astype(np.float32)
+    e = (rng.integers(0, 2, size=(m, k)) * 0.5 - 0.25).astype(np.float32)      # +-0.25, exact at this magnitude
+    c = np.empty((2 * m, k), dtype=np.float32)
+    c[0::2], c[1::2] = p + e, p - e
+    assert np.array_equal((c[0::2] - p), e) and np.array_equal((p - c[1::2]), e)
+    got = host(capi.kmeans_predict(dev(p), dev(c), "l2"))
+    assert np.array_equal(got, 2 * np.arange(m))                             # exact ties: the first
+    c2 = c.copy()
+    c2[1::2, 0] += np.sign(e[:, 0]) * np.float32(2.0 ** -13)                 # the second moves a hair closer
+    d = oc.pairwise_distance(p, c2, "l2", dtype=np.float64)
+    assert np.all(d[np.arange(m), 2 * np.arange(m) + 1] < d[np.arange(m), 2 * np.arange(m)])
+    got = host(capi.kmeans_predict(dev(p), dev(c2), "l2"))
+    assert np.array_equal(got, 2 * np.arange(m) + 1)
+    # three equidistant centres: the row is decided over every centre
+    c3 = np.concatenate([c, c[0:1]])
+    got = host(capi.kmeans_predict(dev(p), dev(c3), "l2"))
+    assert got[0] == 0 and np.array_equal(got[1:], 2 * np.arange(1, m))
+
+
+def test_kmeans_predict_l2_does_not_slow_down_far_from_the_origin():
+    """With the mean of the centres subtracted, a common offset no longer sends rows to the exact
+    re-evaluation; labels stay those of the fp64 distances."""
+    rng = np.random.default_rng(23)
+    x = (rng.standard_normal((20000, 32)) + 300.0).astype(np.float32)
+    c = (rng.standard_normal((256, 32)) + 300.0).astype(np.float32)
+    want, near = oc.kmeans_predict(x, c, "l2")
+    got = host(capi.kmeans_predict(dev(x), dev(c), "l2"))
+    assert np.array_equal(got[~near], want[~near])
+
+
 def test_kmeans_predict_cosine_with_a_centre_without_direction():
     rng = np.random.default_rng(22)
     x = rng.standard_normal((3000, 32)).astype(np.float32)
