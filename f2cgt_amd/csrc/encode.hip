@@ -598,16 +598,27 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
   // the norms are known, the pieces.  Dimensions from k on and centres from n on read as zeros.
   const bool cvec = (k % 8 == 0) && ((reinterpret_cast<uintptr_t>(centers) & 15) == 0);
   // L2: mu[t] = mean of the centres in dimension t, subtracted from every centre and every x (the
-  // distances do not change, the cancellation of the expanded form does); zeros for cosine
+  // distances do not change, the cancellation of the expanded form does).  It is used only when it
+  // matters, |mu|^2 above twice the summed variance of the centres (otherwise, and for cosine, mu
+  // is zero and the subtraction of the hot loop is skipped): cmax_bits[3] != 0 says so for L2.
   const bool centred = !cosine;
-  {
-    float* psum = reinterpret_cast<float*>(smem_raw);            // [4][64], overwritten by the pieces later
+  if (!centred) {
+    if (threadIdx.x < 16 * S) mu[threadIdx.x] = 0.f;
+    __syncthreads();
+  } else {
+    float* psum = reinterpret_cast<float*>(smem_raw);            // [4][64] sums, [4][64] sums of squares
+    float* psq = psum + 256;                                     // (overwritten by the pieces later)
     const int t = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    if (centred && cvec) {
+    if (cvec) {
       // a lane sums a float4 column of every 16th row, eight loads in flight; the four row groups of
       // a wave are added with shuffles
       const int col = t & 15, part = threadIdx.x >> 4;
-      float4 a4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      float4 a4 = make_float4(0.f, 0.f, 0.f, 0.f), q4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      auto add = [&](const float4& v) {
+        a4.x += v.x; a4.y += v.y; a4.z += v.z; a4.w += v.w;
+        q4.x = __fmaf_rn(v.x, v.x, q4.x); q4.y = __fmaf_rn(v.y, v.y, q4.y);
+        q4.z = __fmaf_rn(v.z, v.z, q4.z); q4.w = __fmaf_rn(v.w, v.w, q4.w);
+      };
       if (4 * col < k) {
         const float* base = centers + 4 * col;
         int c = part;
@@ -616,29 +627,46 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
 #pragma unroll
           for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(base + (int64_t)(c + 16 * u) * k);
 #pragma unroll
-          for (int u = 0; u < 8; ++u) { a4.x += v[u].x; a4.y += v[u].y; a4.z += v[u].z; a4.w += v[u].w; }
+          for (int u = 0; u < 8; ++u) add(v[u]);
         }
-        for (; c < n; c += 16) {
-          const float4 v = *reinterpret_cast<const float4*>(base + (int64_t)c * k);
-          a4.x += v.x; a4.y += v.y; a4.z += v.z; a4.w += v.w;
-        }
+        for (; c < n; c += 16) add(*reinterpret_cast<const float4*>(base + (int64_t)c * k));
       }
 #pragma unroll
       for (int off = 16; off <= 32; off <<= 1) {
         a4.x += __shfl_xor(a4.x, off); a4.y += __shfl_xor(a4.y, off);
         a4.z += __shfl_xor(a4.z, off); a4.w += __shfl_xor(a4.w, off);
+        q4.x += __shfl_xor(q4.x, off); q4.y += __shfl_xor(q4.y, off);
+        q4.z += __shfl_xor(q4.z, off); q4.w += __shfl_xor(q4.w, off);
       }
-      if (t < 16) *reinterpret_cast<float4*>(psum + wv * 64 + 4 * t) = a4;
+      if (t < 16) {
+        *reinterpret_cast<float4*>(psum + wv * 64 + 4 * t) = a4;
+        *reinterpret_cast<float4*>(psq + wv * 64 + 4 * t) = q4;
+      }
     } else {
-      float sum = 0.f;
-      if (centred && t < k)
-        for (int c = wv; c < n; c += 4) sum += centers[(int64_t)c * k + t];
+      float sum = 0.f, sq = 0.f;
+      if (t < k)
+        for (int c = wv; c < n; c += 4) {
+          const float v = centers[(int64_t)c * k + t];
+          sum += v;
+          sq = __fmaf_rn(v, v, sq);
+        }
       psum[wv * 64 + t] = sum;
+      psq[wv * 64 + t] = sq;
     }
     __syncthreads();
-    if (threadIdx.x < 16 * S)
-      mu[threadIdx.x] = ((psum[threadIdx.x] + psum[64 + threadIdx.x]) +
-                         (psum[128 + threadIdx.x] + psum[192 + threadIdx.x])) / (float)n;
+    if (threadIdx.x < 64) {                                      // the first wave, all of it
+      const float mt = ((psum[t] + psum[64 + t]) + (psum[128 + t] + psum[192 + t])) / (float)n;
+      const float st = ((psq[t] + psq[64 + t]) + (psq[128 + t] + psq[192 + t])) / (float)n;
+      float m2 = mt * mt, var = st - mt * mt;                    // dimensions from k on hold zeros
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) {
+        m2 += __shfl_xor(m2, off);
+        var += __shfl_xor(var, off);
+      }
+      const bool use = m2 > 2.f * (var > 0.f ? var : 0.f);
+      if (t < 16 * S) mu[t] = use ? mt : 0.f;
+      if (t == 0) cmax_bits[3] = use ? 1 : 0;
+    }
     __syncthreads();
   }
   auto load8 = [&](int c, int ch, float (&v)[8]) {
@@ -721,6 +749,7 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
   }
   __syncthreads();
   const float cmax = __int_as_float(cmax_bits[0]);
+  const bool use_mu = centred && __builtin_amdgcn_readfirstlane(cmax_bits[3]) != 0;
   const bool plain_cosine = cmax_bits[1] != 0;   // degenerate centres: no candidate filter for cosine
   const float cmin_norm = sqrtf(__int_as_float(cmax_bits[3]));   // PW, cosine: smallest |c|
 
@@ -769,8 +798,10 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
 #pragma unroll
           for (int e = 0; e < 8; ++e) q[e] = (valid && kk0 + e < k) ? x[row * k + kk0 + e] : 0.f;
         }
+        if (use_mu) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) q[e] = (valid && kk0 + e < k) ? q[e] - mu[kk0 + e] : 0.f;
+          for (int e = 0; e < 8; ++e) q[e] = (valid && kk0 + e < k) ? q[e] - mu[kk0 + e] : 0.f;
+        }
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           sum += q[e] * q[e];
