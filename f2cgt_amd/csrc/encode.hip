@@ -513,8 +513,8 @@ __device__ int exact_argmin_row_l2_pieces(const float* __restrict__ xrow, float*
 // Exact cosine assignment of one row by a whole wave.  The LDS pieces hold the centres divided by
 // their norms; with c' their leading pieces, |x . c/|c| - x . c'| <= 2^-8 |x| (1 + 2^-20), so only
 // centres whose leading-piece dot product is within 2^-6 |x| of the largest can have the smallest
-// distance; those are evaluated exactly, in fp64 from the centres in HBM, by the formula of
-// exact_argmin_row.  Needs every centre to have a direction (|c|^2 > 1e-12).
+// distance; those go through the fp32 dot product with all three pieces, and what that leaves is
+// evaluated exactly, in fp64 from the centres in HBM, by the formula of exact_argmin_row.  Needs every centre to have a direction (|c|^2 > 1e-12).
 template <int S>
 __device__ int exact_argmin_row_cosine_pieces(const float* __restrict__ xrow, float* xs, const bf16x8* ap,
                                               const float* __restrict__ centers, int n, int n_ct, int k,
@@ -542,12 +542,38 @@ __device__ int exact_argmin_row_cosine_pieces(const float* __restrict__ xrow, fl
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) smax = fmaxf(smax, __shfl_xor(smax, off));
   const float floor_s = smax - 0.015625f * sqrtf(xnorm2) - 1e-30f;
+  // second filter: the fp32 dot product with the whole normalised centre (the sum of its pieces) is
+  // within (k + 4) 2^-24 |x| of x . c / |c| (k + 2 for the sum, 2 for the rounding of c / |c|), so
+  // the nearest centre is within twice that of the largest one.  Data far from the origin passes
+  // the first filter with every centre; this one leaves the few that the fp64 stage has to read.
+  auto dot32 = [&](int c) -> float {
+    float d = 0.f;
+    const int piece_stride = n_ct * S * 64;
+#pragma nounroll
+    for (int ch = 0; ch < 2 * S; ++ch) {
+      const bf16x8* q = ap + (c >> 5) * S * 64 + (ch >> 1) * 64 + (ch & 1) * 32 + (c & 31);
+      const bf16x8 p0 = q[0], p1 = q[piece_stride], p2 = q[2 * piece_stride];
+      const float4 xa = *reinterpret_cast<const float4*>(xs + 8 * ch);
+      const float4 xb = *reinterpret_cast<const float4*>(xs + 8 * ch + 4);
+      const float xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) d = __fmaf_rn(xv[e], ((float)p0[e] + (float)p1[e]) + (float)p2[e], d);
+    }
+    return d;
+  };
+  float s32max = -INFINITY;
+  for (int c = lane; c < n; c += kWave)
+    if (dot_lead(c) >= floor_s) s32max = fmaxf(s32max, dot32(c));
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) s32max = fmaxf(s32max, __shfl_xor(s32max, off));
+  const float floor32 = s32max - 1.1920929e-7f * (float)(k + 6) * sqrtf(xnorm2) * 1.001f - 1e-30f;
   double xn = 0.0;
   for (int t = 0; t < k; ++t) xn += (double)xrow[t] * (double)xrow[t];
   double bestv = DBL_MAX;
   int besti = INT_MAX;
   for (int c = lane; c < n; c += kWave) {
     if (!(dot_lead(c) >= floor_s)) continue;
+    if (!(dot32(c) >= floor32)) continue;
     const float* cr = centers + (int64_t)c * k;
     double dot = 0.0, cn = 0.0;
     for (int t = 0; t < k; ++t) {
