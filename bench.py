@@ -32,11 +32,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # what the same counter reads for a plain copy of known size; see profiles/).  Keyed by
 # (workload name, index dtype).  Missing = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1_sq8_affine", "int64"): 18292814,
-    ("c2_sq4_affine", "int64"): 134405397,
-    ("c3_vq_16x8", "int64"): 506870699,
-    ("c4_hybrid", "int64"): 1004033132,
-    ("c5_vq_24x32", "int64"): 2170720212,
+    ("c1_sq8_affine", "int64"): 18292817,
+    ("c2_sq4_affine", "int64"): 134407238,
+    ("c3_vq_16x8", "int64"): 506966226,
+    ("c4_hybrid", "int64"): 1004036282,
+    ("c5_vq_24x32", "int64"): 2177227871,
 }
 
 
