@@ -200,6 +200,28 @@ def test_encode_random_shape(seed):
     assert np.allclose(d, ref, rtol=1e-5, atol=1e-5 * max(1.0, float(np.abs(ref).max())))
 
 
+@pytest.mark.parametrize("seed", seeds(24))
+def test_fetch_rows_random_shape(seed):
+    rng = np.random.default_rng(7000 + seed)
+    dtype = [np.uint8, np.int8, np.int16, np.float32, np.float64, np.float16][int(rng.integers(0, 6))]
+    cols = int(rng.integers(1, 200))
+    n = int(rng.integers(1, 3000))
+    m = int(rng.integers(0, 4000))
+    table = (rng.standard_normal((n, cols)) * 50).astype(dtype)
+    idx = [np.int32, np.int64][int(rng.integers(0, 2))]
+    index = rng.integers(0, n, size=m).astype(idx)
+    t_dev = dev(table)
+    assert np.array_equal(host(capi.fetch_rows(t_dev, dev(index))).view(np.uint8), table[index].view(np.uint8))
+    n_hot = int(rng.integers(0, n + 1))
+    if n_hot:
+        hot_ids = rng.permutation(n)[:n_hot]
+        hot = (rng.standard_normal((n_hot, cols)) * 50).astype(dtype)
+        slot = np.full(n, -1, dtype=np.int32)
+        slot[hot_ids] = np.arange(n_hot, dtype=np.int32)
+        got = host(capi.fetch_rows(t_dev, dev(index), dev(hot), dev(slot)))
+        assert np.array_equal(got.view(np.uint8), oc.fetch_rows(table, index, hot, slot).view(np.uint8))
+
+
 @pytest.mark.parametrize("seed", seeds(12))
 def test_module_dtype_surface_random(seed):
     """The F2CGTLib module with the reference's accepted dtypes (src/common.h:17-104): index tensors of
