@@ -636,7 +636,7 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
     float* psq = psum + 256;                                     // (overwritten by the pieces later)
     const int t = threadIdx.x & 63, wv = threadIdx.x >> 6;
     if (cvec) {
-      // a lane sums a float4 column of every 16th row, eight loads in flight; the four row groups of
+      // a lane sums a float4 column of every 16th row, sixteen loads in flight; the four row groups of
       // a wave are added with shuffles
       const int col = t & 15, part = threadIdx.x >> 4;
       float4 a4 = make_float4(0.f, 0.f, 0.f, 0.f), q4 = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -648,12 +648,12 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
       if (4 * col < k) {
         const float* base = centers + 4 * col;
         int c = part;
-        for (; c + 16 * 7 < n; c += 16 * 8) {
-          float4 v[8];
+        for (; c + 16 * 15 < n; c += 16 * 16) {
+          float4 v[16];
 #pragma unroll
-          for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(base + (int64_t)(c + 16 * u) * k);
+          for (int u = 0; u < 16; ++u) v[u] = *reinterpret_cast<const float4*>(base + (int64_t)(c + 16 * u) * k);
 #pragma unroll
-          for (int u = 0; u < 8; ++u) add(v[u]);
+          for (int u = 0; u < 16; ++u) add(v[u]);
         }
         for (; c < n; c += 16) add(*reinterpret_cast<const float4*>(base + (int64_t)c * k));
       }
