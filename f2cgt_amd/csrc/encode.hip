@@ -13,7 +13,9 @@
 // kmeans_predict never writes the matrix.  For L2 it works, like pairwise_distance, on x - mu and
 // c - mu (mu = mean of the centres): a common offset of the data then costs nothing, and the rows
 // whose best two centres are closer than the rounding of that subtraction are decided from the
-// original arrays.  A wave owns rows of x and walks the centres a tile
+// original arrays.  For cosine the normalised centres lose their mean direction m when |m| > 1/2
+// (argmin -x . c^ = argmin -x . (c^ - m)): the scores then resolve the differences between the
+// centres' directions, which is all that data far from the origin leaves.  A wave owns rows of x and walks the centres a tile
 // at a time on the matrix core: A = centre tile, B = x tile, so every lane holds 16 centre
 // scores of ONE x row per tile and the running arg-min stays in registers.  Scores use the
 // expanded form (|c|^2 - 2 x.c, the row constant |x|^2 dropped); rows whose two best scores are
@@ -510,15 +512,16 @@ __device__ int exact_argmin_row_l2_pieces(const float* __restrict__ xrow, float*
   return dhi < dlo ? hi : lo;
 }
 
-// Exact cosine assignment of one row by a whole wave.  The LDS pieces hold the centres divided by
-// their norms; with c' their leading pieces, |x . c/|c| - x . c'| <= 2^-8 |x| (1 + 2^-20), so only
-// centres whose leading-piece dot product is within 2^-6 |x| of the largest can have the smallest
+// Exact cosine assignment of one row by a whole wave.  The LDS pieces hold d = c / |c| - m (m: the
+// mean direction or zero, the same for every centre, so x . m does not matter), |d| <= cdev; with
+// d' their leading pieces, |x . d - x . d'| <= 2^-8 |x| cdev (1 + 2^-20), so only
+// centres whose leading-piece dot product is within 2^-6 |x| cdev of the largest can have the smallest
 // distance; those go through the fp32 dot product with all three pieces, and what that leaves is
 // evaluated exactly, in fp64 from the centres in HBM, by the formula of exact_argmin_row.  Needs every centre to have a direction (|c|^2 > 1e-12).
 template <int S>
 __device__ int exact_argmin_row_cosine_pieces(const float* __restrict__ xrow, float* xs, const bf16x8* ap,
                                               const float* __restrict__ centers, int n, int n_ct, int k,
-                                              int lane) {
+                                              int lane, float cdev) {
   if (lane < 16 * S) xs[lane] = lane < k ? xrow[lane] : 0.f;
   __builtin_amdgcn_wave_barrier();
   float xnorm2 = lane < 16 * S ? xs[lane] * xs[lane] : 0.f;
@@ -541,10 +544,10 @@ __device__ int exact_argmin_row_cosine_pieces(const float* __restrict__ xrow, fl
   for (int c = lane; c < n; c += kWave) smax = fmaxf(smax, dot_lead(c));
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) smax = fmaxf(smax, __shfl_xor(smax, off));
-  const float floor_s = smax - 0.015625f * sqrtf(xnorm2) - 1e-30f;
-  // second filter: the fp32 dot product with the whole normalised centre (the sum of its pieces) is
-  // within (k + 4) 2^-24 |x| of x . c / |c| (k + 2 for the sum, 2 for the rounding of c / |c|), so
-  // the nearest centre is within twice that of the largest one.  Data far from the origin passes
+  const float floor_s = smax - 0.015625f * cdev * sqrtf(xnorm2) - 1e-30f;
+  // second filter: the fp32 dot product with the whole operand (the sum of its pieces) is within
+  // ((k + 2) cdev + 3) 2^-24 |x| of x . (c / |c| - m) (the sum; the roundings of 1 / |c|, of the
+  // product and of the subtraction), so the nearest centre is within twice that of the largest one.  Data far from the origin passes
   // the first filter with every centre; this one leaves the few that the fp64 stage has to read.
   auto dot32 = [&](int c) -> float {
     float d = 0.f;
@@ -566,7 +569,7 @@ __device__ int exact_argmin_row_cosine_pieces(const float* __restrict__ xrow, fl
     if (dot_lead(c) >= floor_s) s32max = fmaxf(s32max, dot32(c));
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) s32max = fmaxf(s32max, __shfl_xor(s32max, off));
-  const float floor32 = s32max - 1.1920929e-7f * (float)(k + 6) * sqrtf(xnorm2) * 1.001f - 1e-30f;
+  const float floor32 = s32max - 1.1920929e-7f * ((float)(k + 4) * cdev + 3.f) * sqrtf(xnorm2) * 1.001f - 1e-30f;
   double xn = 0.0;
   for (int t = 0; t < k; ++t) xn += (double)xrow[t] * (double)xrow[t];
   double bestv = DBL_MAX;
@@ -707,12 +710,14 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = (in && 8 * ch + e < k) ? cr[e] : 0.f;
     }
+    if (centred) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = (in && 8 * ch + e < k) ? v[e] - mu[8 * ch + e] : 0.f;
+      for (int e = 0; e < 8; ++e) v[e] = (in && 8 * ch + e < k) ? v[e] - mu[8 * ch + e] : 0.f;
+    }
   };
   constexpr int kChunks = 2 * S;
   const int n_items = n_pad * kChunks;
-  float* partial = reinterpret_cast<float*>(smem_raw);          // [n_pad][2 S], overwritten by the pieces later
+  double* partial = reinterpret_cast<double*>(smem_raw);        // [n_pad][2 S], overwritten by the pieces later
   for (int i0 = threadIdx.x; i0 < n_items; i0 += blockDim.x * 4) {
     float v[4][8];
 #pragma unroll
@@ -723,22 +728,20 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int it = i0 + u * blockDim.x;
-      float sq = 0.f;
+      double sq = 0.0;                       // fp64: 1 / |c| must be good to a rounding or two
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sq += v[u][e] * v[u][e];
+      for (int e = 0; e < 8; ++e) sq += (double)v[u][e] * (double)v[u][e];
       if (it < n_items) partial[it] = sq;
     }
   }
   __syncthreads();
   for (int jj = threadIdx.x; jj < n_pad; jj += blockDim.x) {
-    float cn = 0.f;
+    double cn64 = 0.0;
 #pragma unroll
-    for (int ch = 0; ch < kChunks; ++ch) cn += partial[jj * kChunks + ch];
+    for (int ch = 0; ch < kChunks; ++ch) cn64 += partial[jj * kChunks + ch];
+    const float cn = (float)cn64;
     float sc = 1.f;
-    if (cosine) {
-      const float nr = sqrtf(cn);
-      sc = 1.f / (nr > 1e-30f ? nr : 1e-30f);
-    }
+    if (cosine) sc = (float)(1.0 / sqrt(cn64 > 1e-60 ? cn64 : 1e-60));
     inv[jj] = sc;
     bias[jj] = jj >= n ? INFINITY : (cosine ? 0.f : cn);
     if (jj < n && !cosine) atomicMax(cmax_bits, __float_as_int(cn));
@@ -746,6 +749,64 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
     if (PW && jj < n && cosine) atomicMin(cmax_bits + 3, __float_as_int(cn));
   }
   __syncthreads();
+  // Cosine assignment: argmin_c -x . c^ = argmin_c -x . (c^ - m) for any m, and with m the mean of
+  // the normalised centres c^ the operands of the matrix core shrink to the spread of the centres'
+  // directions: what data far from the origin leaves of the evaluation's resolution goes to the
+  // differences between centres.  Used when |m| > 1/2; mu[] then holds m (zeros otherwise).
+  if (!PW && cosine) {
+    float* psum = reinterpret_cast<float*>(smem_raw);            // [4][64]
+    const int t = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const bool degenerate = cmax_bits[1] != 0;
+    if (cvec) {
+      // as for the L2 mean: a float4 column of every 16th row per lane, sixteen loads in flight
+      const int col = t & 15, part = threadIdx.x >> 4;
+      float4 a4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (!degenerate && 4 * col < k) {
+        const float* base = centers + 4 * col;
+        int c = part;
+        for (; c + 16 * 15 < n; c += 16 * 16) {
+          float4 v[16];
+#pragma unroll
+          for (int u = 0; u < 16; ++u) v[u] = *reinterpret_cast<const float4*>(base + (int64_t)(c + 16 * u) * k);
+#pragma unroll
+          for (int u = 0; u < 16; ++u) {
+            const float sc = inv[c + 16 * u];
+            a4.x = __fmaf_rn(v[u].x, sc, a4.x); a4.y = __fmaf_rn(v[u].y, sc, a4.y);
+            a4.z = __fmaf_rn(v[u].z, sc, a4.z); a4.w = __fmaf_rn(v[u].w, sc, a4.w);
+          }
+        }
+        for (; c < n; c += 16) {
+          const float4 v = *reinterpret_cast<const float4*>(base + (int64_t)c * k);
+          const float sc = inv[c];
+          a4.x = __fmaf_rn(v.x, sc, a4.x); a4.y = __fmaf_rn(v.y, sc, a4.y);
+          a4.z = __fmaf_rn(v.z, sc, a4.z); a4.w = __fmaf_rn(v.w, sc, a4.w);
+        }
+      }
+#pragma unroll
+      for (int off = 16; off <= 32; off <<= 1) {
+        a4.x += __shfl_xor(a4.x, off); a4.y += __shfl_xor(a4.y, off);
+        a4.z += __shfl_xor(a4.z, off); a4.w += __shfl_xor(a4.w, off);
+      }
+      if (t < 16) *reinterpret_cast<float4*>(psum + wv * 64 + 4 * t) = a4;
+    } else {
+      float sum = 0.f;
+      if (!degenerate && t < k)
+        for (int c = wv; c < n; c += 4) sum = __fmaf_rn(centers[(int64_t)c * k + t], inv[c], sum);
+      psum[wv * 64 + t] = sum;
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+      const float mt = ((psum[t] + psum[64 + t]) + (psum[128 + t] + psum[192 + t])) / (float)n;
+      float m2 = mt * mt;
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) m2 += __shfl_xor(m2, off);
+      const bool use = !degenerate && m2 > 0.25f;
+      if (t < 16 * S) mu[t] = use ? mt : 0.f;
+      if (t == 0) cmax_bits[3] = use ? 1 : 0;
+    }
+    __syncthreads();
+  }
+  float dev2max = 0.f;
   for (int i0 = threadIdx.x; i0 < n_items; i0 += blockDim.x * 4) {
     float v[4][8];
 #pragma unroll
@@ -760,12 +821,17 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
       const int c = it / kChunks, ch = it % kChunks;
       const float sc = inv[c];
       bf16x8 p0, p1, p2;
+      float dev2 = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
+        float val = v[u][e] * sc;
+        if (cosine) val = (c < n && 8 * ch + e < k) ? val - mu[8 * ch + e] : 0.f;
+        dev2 = __fmaf_rn(val, val, dev2);
         __bf16 a0, a1, a2;
-        split3(v[u][e] * sc, a0, a1, a2);
+        split3(val, a0, a1, a2);
         p0[e] = a0; p1[e] = a1; p2[e] = a2;
       }
+      dev2max = fmaxf(dev2max, dev2);                            // largest 8-dimension share of |c^ - m|^2
       // chunk ch of centre c is lane (c % 32) + 32 (ch % 2) of step ch / 2 of tile c / 32
       const int at = ((c >> 5) * S + (ch >> 1)) * 64 + (ch & 1) * 32 + (c & 31);
       ap[at] = p0;
@@ -773,10 +839,22 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
       ap[2 * n_ct * S * 64 + at] = p2;
     }
   }
+  if (cosine) {                                                  // one LDS atomic per wave
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) dev2max = fmaxf(dev2max, __shfl_xor(dev2max, off));
+    if ((threadIdx.x & 63) == 0) atomicMax(cmax_bits, __float_as_int(dev2max));
+  }
   __syncthreads();
   const float cmax = __int_as_float(cmax_bits[0]);
   const bool use_mu = centred && __builtin_amdgcn_readfirstlane(cmax_bits[3]) != 0;
   const bool plain_cosine = cmax_bits[1] != 0;   // degenerate centres: no candidate filter for cosine
+  // cosine: upper bound of |c^ - m| over the centres (1 without the mean; never above 2)
+  float cdev = 1.f;
+  if (!PW && cosine && !plain_cosine && cmax_bits[3] == 1) {
+    cdev = sqrtf((float)kChunks * cmax) * 1.0001f;
+    cdev = cdev < 2.f ? cdev : 2.f;
+  }
+  cdev = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(cdev)));
   const float cmin_norm = sqrtf(__int_as_float(cmax_bits[3]));   // PW, cosine: smallest |c|
 
   const int lane = threadIdx.x & 63;
@@ -1009,7 +1087,9 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
           sd = fminf(sd, ob);
         }
       }
-      const float scale = cosine ? sqrtf(xn[b]) : xn[b] + cmax;
+      // cosine: the evaluation's share shrinks with the operands, the rounding of c / |c| (norm in
+      // fp64, one rounding for 1 / |c|, one for the product, one for - m: 3 units, doubled) does not
+      const float scale = cosine ? sqrtf(xn[b]) * (cdev + 3.5762787e-7f / unit) : xn[b] + cmax;
       besti[b] = bi;
       todo[b] = __ballot(valid && g == 0 && !((sd - bs) > unit * scale + kTinyGap));
     }
@@ -1029,7 +1109,7 @@ __global__ __launch_bounds__(256) void predict_split_kernel(const float* __restr
           if (exact < 0) exact = exact_argmin_row(x + rrow * k, centers, n, k, metric, lane);   // the original row decides
         }
         else if (plain_cosine) exact = exact_argmin_row(x + rrow * k, centers, n, k, metric, lane);
-        else exact = exact_argmin_row_cosine_pieces<S>(x + rrow * k, xs, ap, centers, n, n_ct, k, lane);
+        else exact = exact_argmin_row_cosine_pieces<S>(x + rrow * k, xs, ap, centers, n, n_ct, k, lane, cdev);
 #pragma unroll
         for (int q = 0; q < NB; ++q) besti[q] = (b == q && lane == src) ? exact : besti[q];
       }
