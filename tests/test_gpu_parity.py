@@ -721,6 +721,20 @@ def test_kmeans_predict_l2_does_not_slow_down_far_from_the_origin():
     assert np.array_equal(got[~near], want[~near])
 
 
+@pytest.mark.parametrize("offset", [3.0, 100.0])
+def test_kmeans_predict_cosine_far_from_the_origin(offset):
+    """Centres that share most of their direction: the kernel takes their mean direction out of
+    the scores; labels stay those of the fp64 cosines, duplicates go to the first copy."""
+    rng = np.random.default_rng(29)
+    x = (rng.standard_normal((20000, 32)) + offset).astype(np.float32)
+    c = (rng.standard_normal((256, 32)) + offset).astype(np.float32)
+    c[200] = c[5]
+    want, near = oc.kmeans_predict(x, c, "cosine")
+    got = host(capi.kmeans_predict(dev(x), dev(c), "cosine"))
+    assert np.array_equal(got[~near], want[~near])
+    assert not np.any(got == 200) and np.any(got == 5)
+
+
 def test_kmeans_predict_cosine_with_a_centre_without_direction():
     rng = np.random.default_rng(22)
     x = rng.standard_normal((3000, 32)).astype(np.float32)
