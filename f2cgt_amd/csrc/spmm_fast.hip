@@ -883,8 +883,8 @@ struct HybArgs {
 
 constexpr uint32_t kVqFlag = 0x80000000u;
 
-template <typename Idx, int VEC>
-__global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx* __restrict__ indptr,
+template <typename Idx, int VEC, int TB>
+__global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __restrict__ indptr,
                                                             const Idx* __restrict__ indices,
                                                             float* __restrict__ out) {
   constexpr int LIMIT = 257;
@@ -904,14 +904,14 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
   const int nrows = (int)((a.R - row0) < a.rows_per_block ? (a.R - row0) : a.rows_per_block);
   int64_t e0 = (int64_t)indptr[row0];
   e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
-  for (int i = t; i <= nrows; i += kBlock) {
+  for (int i = t; i <= nrows; i += TB) {
     int64_t v = (int64_t)indptr[row0 + i];
     v = v < e0 ? e0 : (v > a.E ? a.E : v);
     s_ptr[i] = (int)(v - e0 > 0x7fffffff ? 0x7fffffff : v - e0);
   }
-  for (int i = t; i < nrows * acc_pitch; i += kBlock) s_acc[i] = 0u;
-  for (int i = t; i < nrows; i += kBlock) s_nvq[i] = 0;
-  for (int i = t; i < a.feat_dim; i += kBlock) {
+  for (int i = t; i < nrows * acc_pitch; i += TB) s_acc[i] = 0u;
+  for (int i = t; i < nrows; i += TB) s_nvq[i] = 0;
+  for (int i = t; i < a.feat_dim; i += TB) {
     const int c4 = i >> 2, q = i & 3;
     s_par[c4 * 8 + q] = a.sq_params[i];
     s_par[c4 * 8 + 4 + q] = a.sq_params[a.param_stride + i];
@@ -925,7 +925,7 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
   for (int eb = 0; eb < ne; eb += a.edge_batch) {
     const int nb = (ne - eb) < a.edge_batch ? (ne - eb) : a.edge_batch;
     if (eb) __syncthreads();
-    for (int i = t; i < nb; i += kBlock) {
+    for (int i = t; i < nb; i += TB) {
       const int64_t id = clamp_idx(indices[e0 + eb + i], a.N);
       const int64_t m = (int64_t)a.row_map[id];
       uint32_t v;
@@ -939,7 +939,7 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
       s_erow[i] = 0;
     }
     __syncthreads();
-    for (int r = t; r < nrows; r += kBlock) {
+    for (int r = t; r < nrows; r += TB) {
       int b = s_ptr[r] - eb, e = s_ptr[r + 1] - eb;
       const bool direct = s_ptr[r + 1] - s_ptr[r] > LIMIT;
       b = b < 0 ? 0 : b;
@@ -958,7 +958,7 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
       const int lanes = a.ch2 >> 2;
       const int j = t & (lanes - 1);
       const int gslot = t / lanes;
-      const int gslots = kBlock / lanes;
+      const int gslots = TB / lanes;
       constexpr int U = 4;
       // lane j of the lanes that share an edge loads dwords 4j .. 4j+3 with one 16-byte access (the
       // lanes of an edge cover its 128-byte line once; four strided dword loads per lane kept
@@ -1002,7 +1002,7 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
     } else {
     const int j = t & (a.ch2 - 1);
     const int gslot = t / a.ch2;
-    const int gslots = kBlock / a.ch2;
+    const int gslots = TB / a.ch2;
     constexpr int U = 4;
     for (int e = gslot; e < nb; e += gslots * U) {
       uint32_t w[U], row[U], er[U];
@@ -1031,7 +1031,7 @@ __global__ __launch_bounds__(kBlock) void hybrid_acc_kernel(HybArgs a, const Idx
   // finalize: lane <-> one float4 of the block's contiguous output span
   const int items = nrows * a.chunks;
   float* ob = out + row0 * (int64_t)a.feat_dim;
-  for (int it = t; it < items; it += kBlock) {
+  for (int it = t; it < items; it += TB) {
     const int r = (int)__umulhi((uint32_t)it, a.magic);
     const int c4 = it - r * a.chunks;
     uint2 q;
@@ -1189,6 +1189,36 @@ int sq_affine_acc_run(const uint8_t* codes, const float* params, int64_t param_s
                           : launch_acc<8>(a, indptr, indices, idx_dtype, out, st, what);
 }
 
+template <int TB>
+int launch_hybrid(HybArgs a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
+                  const char* what) {
+  a.edge_batch = 4 * TB;
+  const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 1.0;
+  const int want = (int)(1.5625 * TB / (avg_deg > 0.5 ? avg_deg : 0.5));   // ~1.5 edges per thread
+  int rb = 8;
+  while (rb * 2 <= want && rb < 64) rb *= 2;
+  const size_t acc_row = (size_t)(2 * a.chunks + 8) * 4;
+  while (rb > 8 && rb * acc_row > 16 * 1024) rb /= 2;
+  a.rows_per_block = rb;
+  const size_t lds = rb * acc_row + (size_t)a.chunks * 32 + (size_t)(rb + 4) * 4 + (size_t)rb * 4 +
+                     (size_t)a.edge_batch * 6 + 16;
+  const int64_t grid = ceil_div(a.R, rb);
+  if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
+  const bool vec4 = a.feat_dim % 16 == 0 && aligned(a.sq_codes, 16) && a.ch2 >= 4;
+  const int32_t* ip32 = static_cast<const int32_t*>(indptr);
+  const int32_t* ix32 = static_cast<const int32_t*>(indices);
+  const int64_t* ip64 = static_cast<const int64_t*>(indptr);
+  const int64_t* ix64 = static_cast<const int64_t*>(indices);
+  if (idx_dtype == F2CGT_DT_I32) {
+    if (vec4) hybrid_acc_kernel<int32_t, 4, TB><<<(unsigned)grid, TB, lds, st>>>(a, ip32, ix32, out);
+    else hybrid_acc_kernel<int32_t, 1, TB><<<(unsigned)grid, TB, lds, st>>>(a, ip32, ix32, out);
+  } else {
+    if (vec4) hybrid_acc_kernel<int64_t, 4, TB><<<(unsigned)grid, TB, lds, st>>>(a, ip64, ix64, out);
+    else hybrid_acc_kernel<int64_t, 1, TB><<<(unsigned)grid, TB, lds, st>>>(a, ip64, ix64, out);
+  }
+  return launch_status(what);
+}
+
 bool hybrid_acc_eligible(const void* sq_codes, const float* vq_codebooks, const float* out, int64_t N,
                          int64_t n_sq, int64_t n_vq, int feat_dim, int w) {
   if (!aligned(sq_codes, 4) || !aligned(out, 16) || !aligned(vq_codebooks, 16)) return false;
@@ -1209,31 +1239,15 @@ int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float*
   a.chunks = feat_dim / 4;
   a.ch2 = pow2_ceil(a.chunks);
   a.magic = (uint32_t)((0x100000000ull + a.chunks - 1) / a.chunks);
-  a.edge_batch = 1024;
-  const double avg_deg = R > 0 ? (double)E / (double)R : 1.0;
-  const int want = (int)(400.0 / (avg_deg > 0.5 ? avg_deg : 0.5));
-  int rb = 8;
-  while (rb * 2 <= want && rb < 64) rb *= 2;
-  const size_t acc_row = (size_t)(2 * a.chunks + 8) * 4;
-  while (rb > 8 && rb * acc_row > 16 * 1024) rb /= 2;
-  a.rows_per_block = rb;
-  const size_t lds = rb * acc_row + (size_t)a.chunks * 32 + (size_t)(rb + 4) * 4 + (size_t)rb * 4 +
-                     (size_t)a.edge_batch * 6 + 16;
-  const int64_t grid = ceil_div(R, rb);
-  if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
-  const bool vec4 = feat_dim % 16 == 0 && aligned(sq_codes, 16) && a.ch2 >= 4;
-  const int32_t* ip32 = static_cast<const int32_t*>(indptr);
-  const int32_t* ix32 = static_cast<const int32_t*>(indices);
-  const int64_t* ip64 = static_cast<const int64_t*>(indptr);
-  const int64_t* ix64 = static_cast<const int64_t*>(indices);
-  if (idx_dtype == F2CGT_DT_I32) {
-    if (vec4) hybrid_acc_kernel<int32_t, 4><<<(unsigned)grid, kBlock, lds, st>>>(a, ip32, ix32, out);
-    else hybrid_acc_kernel<int32_t, 1><<<(unsigned)grid, kBlock, lds, st>>>(a, ip32, ix32, out);
-  } else {
-    if (vec4) hybrid_acc_kernel<int64_t, 4><<<(unsigned)grid, kBlock, lds, st>>>(a, ip64, ix64, out);
-    else hybrid_acc_kernel<int64_t, 1><<<(unsigned)grid, kBlock, lds, st>>>(a, ip64, ix64, out);
-  }
-  return launch_status(what);
+  // One wave per workgroup (8 rows at 12 edges per row) for rows of up to 128 columns and 8-32 edges:
+  // the phases of a block are dependent memory round trips, and many small blocks per CU overlap
+  // them better than few large ones, without a barrier between waves (C4: 334 -> 313 us; 128
+  // threads and 16 rows: 318; twice the rows per block at either size: 332-344).  Measured slower
+  // or equal outside that range (2, 5 or 60 edges per row, 256 columns), which keeps the 256-thread form.
+  const double avg_deg = R > 0 ? (double)E / (double)R : 0.0;
+  if (a.ch2 <= 32 && avg_deg >= 8.0 && avg_deg <= 32.0)
+    return launch_hybrid<64>(a, indptr, indices, idx_dtype, out, st, what);
+  return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what);
 }
 
 }  // namespace f2cgt
