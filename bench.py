@@ -34,9 +34,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 MEASURED_TRAFFIC_BYTES = {
     ("c1_sq8_affine", "int64"): 18292817,
     ("c2_sq4_affine", "int64"): 134407238,
-    ("c3_vq_16x8", "int64"): 506966226,
-    ("c4_hybrid", "int64"): 1004036282,
-    ("c5_vq_24x32", "int64"): 2177227871,
+    ("c3_vq_16x8", "int64"): 506000000,
+    ("c4_hybrid", "int64"): 1029876440,
+    ("c5_vq_24x32", "int64"): 2188900000,
 }
 
 
