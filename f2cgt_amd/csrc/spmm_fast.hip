@@ -606,7 +606,7 @@ int launch_acc(AccArgs a, const void* indptr, const void* indices, int idx_dtype
 
 
 // ---- log-domain (LUT) and 1-/2-bit affine SQ: staged rows, sequential fp32 sums ------------
-// Same block phases as above with 128-thread workgroups, but the decode is not linear in the
+// Same block phases as above with 128- or 256-thread workgroups, but the decode is not linear in the
 // code, so the sums stay in fp32 and in edge order: the code rows of the block's edges are staged
 // in LDS by the edge-parallel 8-byte gather, then a lane that owns one float4 column group (LUT
 // bases or affine parameters in registers) walks its rows' edges from LDS.  The mean is the
@@ -627,18 +627,17 @@ struct RowsArgs {
   int nt_out;            // output larger than the last-level cache: non-temporal stores
 };
 
-constexpr int kRowsBlock = 128;
 
 __device__ __forceinline__ float mean_of(float sum, float d, float r) {
   const float q = sum * r;
   return __fmaf_rn(__fmaf_rn(-q, d, sum), r, q);
 }
 
-template <int BITS, bool AFFINE, typename Idx>
-__global__ __launch_bounds__(kRowsBlock) void sq_rows_kernel(RowsArgs a, const Idx* __restrict__ indptr,
+template <int BITS, bool AFFINE, typename Idx, int TB>
+__global__ __launch_bounds__(TB) void sq_rows_kernel(RowsArgs a, const Idx* __restrict__ indptr,
                                                              const Idx* __restrict__ indices,
                                                              float* __restrict__ out) {
-  constexpr int TB = kRowsBlock;
+  constexpr int NK = (64 + TB - 1) / TB;   // rows of a block (at most 64) per thread in the sorting steps
   constexpr int PER = 8 / BITS;
   constexpr int NCODE = 1 << BITS;
   constexpr uint32_t MASK = NCODE - 1;
@@ -684,9 +683,9 @@ __global__ __launch_bounds__(kRowsBlock) void sq_rows_kernel(RowsArgs a, const I
   // Rows are visited heaviest first (counting sort on min(degree, 15)), so the lanes of a wave,
   // which each walk one row's edges, loop about equally long instead of all waiting for the
   // longest row of an arbitrary group.
-  int my_class[(kRowsBlock + 63) / 64], my_rank[(kRowsBlock + 63) / 64];
+  int my_class[NK], my_rank[NK];
 #pragma unroll
-  for (int k = 0; k < (kRowsBlock + 63) / 64; ++k) {
+  for (int k = 0; k < NK; ++k) {
     const int r = t + k * TB;
     my_class[k] = my_rank[k] = 0;
     if (r < nrows) {
@@ -699,7 +698,7 @@ __global__ __launch_bounds__(kRowsBlock) void sq_rows_kernel(RowsArgs a, const I
     for (int i = t; i < ne; i += TB) s_ids[i] = (uint32_t)clamp_idx(indices[e0 + i], a.N);
   __syncthreads();
 #pragma unroll
-  for (int k = 0; k < (kRowsBlock + 63) / 64; ++k) {
+  for (int k = 0; k < NK; ++k) {
     const int r = t + k * TB;
     if (r < nrows) {
       int before = 0;
@@ -826,7 +825,10 @@ __global__ __launch_bounds__(kRowsBlock) void sq_rows_kernel(RowsArgs a, const I
 template <int BITS, bool AFFINE>
 int launch_sq_rows(RowsArgs a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
                    const char* what) {
-  constexpr int TB = kRowsBlock;
+  // 4- and 8-bit rows: 256 threads walk the same staged rows (twice the lanes in the decode + sum
+  // phase, which sets this kernel's time: 35.7 -> 31.9 us and 43.9 -> 34.8 us on the 2.5e5-row
+  // power-law block); 1- and 2-bit rows are faster with 128 (27.7 against 30.8 us), 64 lose everywhere
+  constexpr int TB = BITS >= 4 ? 256 : 128;
   a.eff_bytes = (int)ceil_div(a.feat_dim, 8 / BITS);
   a.pitch = (a.eff_bytes + 7) & ~7;
   a.lanes = a.pitch / 8;
@@ -851,10 +853,10 @@ int launch_sq_rows(RowsArgs a, const void* indptr, const void* indices, int idx_
   const int64_t grid = ceil_div(a.R, rb);
   if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
   if (idx_dtype == F2CGT_DT_I32)
-    sq_rows_kernel<BITS, AFFINE, int32_t><<<(unsigned)grid, TB, lds, st>>>(
+    sq_rows_kernel<BITS, AFFINE, int32_t, TB><<<(unsigned)grid, TB, lds, st>>>(
         a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
   else
-    sq_rows_kernel<BITS, AFFINE, int64_t><<<(unsigned)grid, TB, lds, st>>>(
+    sq_rows_kernel<BITS, AFFINE, int64_t, TB><<<(unsigned)grid, TB, lds, st>>>(
         a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
   return launch_status(what);
 }
