@@ -827,7 +827,8 @@ int launch_sq_rows(RowsArgs a, const void* indptr, const void* indices, int idx_
                    const char* what) {
   // 4- and 8-bit rows: 256 threads walk the same staged rows (twice the lanes in the decode + sum
   // phase, which sets this kernel's time: 35.7 -> 31.9 us and 43.9 -> 34.8 us on the 2.5e5-row
-  // power-law block); 1- and 2-bit rows are faster with 128 (27.7 against 30.8 us), 64 lose everywhere
+  // power-law block; 512 threads: 36.6 and 41.6); 1- and 2-bit rows are faster with 128 (27.7 against
+  // 30.8 us), 64 lose everywhere
   constexpr int TB = BITS >= 4 ? 256 : 128;
   a.eff_bytes = (int)ceil_div(a.feat_dim, 8 / BITS);
   a.pitch = (a.eff_bytes + 7) & ~7;
