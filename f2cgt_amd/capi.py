@@ -21,6 +21,8 @@ SIGNATURES = {
     "f2cgt_version": ([], c_int),
     "f2cgt_last_error": ([], c_char_p),
     "f2cgt_num_cus": ([], c_int),
+    "f2cgt_set_plan_only": ([I], c_int),
+    "f2cgt_last_plan": ([P], c_int),
     "f2cgt_packbits": ([P, P, L, L, I, P], c_int),
     "f2cgt_unpackbits": ([P, P, L, L, L, I, P], c_int),
     "f2cgt_sq_compress": ([P, P, P, L, L, L, I, L, P], c_int),
@@ -39,6 +41,14 @@ SIGNATURES = {
     "f2cgt_kmeans_predict": ([P, P, P, P, L, L, L, I, P], c_int),
 }
 
+
+
+class Plan(ctypes.Structure):
+    """f2cgt_plan of include/f2cgt.h."""
+    _fields_ = [("kernel", ctypes.c_char * 48), ("grid", c_int64), ("block", ctypes.c_int32),
+                ("lds_bytes", c_int64), ("rows_per_block", ctypes.c_int32), ("aux", ctypes.c_int32 * 4)]
+
+
 _lib = None
 
 
@@ -54,6 +64,20 @@ def lib():
             fn.restype = restype
         _lib = handle
     return _lib
+
+
+def dry_run(entry, *args):
+    """Calls the fused entry point `entry` (a name in SIGNATURES) in plan-only mode: nothing is
+    launched and no pointer is read.  Returns (return code, Plan or None)."""
+    handle = lib()
+    was = handle.f2cgt_set_plan_only(1)
+    try:
+        rc = getattr(handle, entry)(*args)
+        plan = Plan()
+        got = handle.f2cgt_last_plan(ctypes.byref(plan))
+    finally:
+        handle.f2cgt_set_plan_only(was)
+    return rc, (plan if rc == 0 and got == 0 else None)
 
 
 class F2CGTError(RuntimeError):

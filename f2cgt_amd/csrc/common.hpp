@@ -38,7 +38,15 @@ inline int launch_status(const char* what) {
     if (!(cond)) return ::f2cgt::fail((code), __VA_ARGS__); \
   } while (0)
 
-int num_cus();  // compute units of the current device (cached per device)
+int num_cus();  // compute units of the current device (cached per device; 256 without a device)
+
+// ---- dry runs ------------------------------------------------------------------
+// While plan_only() is true for the calling thread, the fused aggregation launchers record the
+// kernel they chose and its launch geometry with plan_record() and return without touching the
+// device (no attribute call, no launch, no pointer dereferenced).
+bool plan_only();
+void plan_record(const char* kernel, int64_t grid, int block, int64_t lds_bytes, int rows_per_block,
+                 int a0 = 0, int a1 = 0, int a2 = 0, int a3 = 0);
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 

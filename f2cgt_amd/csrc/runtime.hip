@@ -10,7 +10,25 @@ char* error_buffer() {
   return buf;
 }
 
+namespace {
+thread_local bool t_plan_only = false;
+thread_local f2cgt_plan t_plan = {};
+}  // namespace
+
+bool plan_only() { return t_plan_only; }
+
+void plan_record(const char* kernel, int64_t grid, int block, int64_t lds_bytes, int rows_per_block, int a0,
+                 int a1, int a2, int a3) {
+  snprintf(t_plan.kernel, sizeof(t_plan.kernel), "%s", kernel);
+  t_plan.grid = grid;
+  t_plan.block = block;
+  t_plan.lds_bytes = lds_bytes;
+  t_plan.rows_per_block = rows_per_block;
+  t_plan.aux[0] = a0; t_plan.aux[1] = a1; t_plan.aux[2] = a2; t_plan.aux[3] = a3;
+}
+
 int num_cus() {
+  if (t_plan_only) return 256;   // a dry run must not depend on (or wake) a device
   static std::atomic<int> cached[64];   // 0 = not asked yet; callers may come from several threads
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
@@ -32,5 +50,18 @@ int f2cgt_version(void) { return 100; }
 const char* f2cgt_last_error(void) { return f2cgt::error_buffer(); }
 
 int f2cgt_num_cus(void) { return f2cgt::num_cus(); }
+
+int f2cgt_set_plan_only(int on) {
+  const int was = f2cgt::t_plan_only ? 1 : 0;
+  f2cgt::t_plan_only = on != 0;
+  if (on) f2cgt::t_plan = f2cgt_plan{};
+  return was;
+}
+
+int f2cgt_last_plan(f2cgt_plan* out) {
+  if (out == nullptr) return F2CGT_E_INVALID;
+  *out = f2cgt::t_plan;
+  return f2cgt::t_plan.kernel[0] ? F2CGT_OK : F2CGT_E_INVALID;
+}
 
 }  // extern "C"

@@ -451,6 +451,10 @@ template <class Dec>
 int run(Dec dec, const void* indptr, const void* indices, int idx_dtype, typename Dec::Out* out,
         int64_t R, int64_t E, int64_t N, int feat_dim, const Geometry& g, size_t lds_bytes,
         bool vec_ok, hipStream_t st, const char* what) {
+  if (plan_only()) {
+    plan_record("agg_kernel", (int64_t)g.grid.x * g.grid.y, g.block, (int64_t)lds_bytes, 0, g.block / g.G);
+    return 0;
+  }
   if (lds_bytes > 48 * 1024) {
     hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(agg_kernel<Dec, int32_t>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -684,6 +688,10 @@ extern "C" int f2cgt_sq_decompress_spmm_csr(const void* codes, int code_dtype, c
   const bool byte_codes = code_dtype == F2CGT_DT_U8 || code_dtype == F2CGT_DT_I8;
   F2CGT_REQUIRE(target_bits == 16 ? code_dtype == F2CGT_DT_I16 : byte_codes, F2CGT_E_UNSUPPORTED,
                 "%s: code dtype does not match target_bit %d", what, target_bits);
+  // 8-bit codes are signed; a uint8 tensor would mean 0..255 to the reference's dtype dispatch
+  // (src/common.h:68-82), values its encoder never produces: refused instead of guessed
+  F2CGT_REQUIRE(target_bits != 8 || code_dtype == F2CGT_DT_I8, F2CGT_E_UNSUPPORTED,
+                "%s: 8-bit codes are signed, pass them as int8 (got uint8)", what);
   if (num_rows * feat_dim == 0) return 0;
   F2CGT_REQUIRE(codebooks && (num_edges == 0 || codes), F2CGT_E_INVALID, "%s: null buffer", what);
   hipStream_t st = as_stream(stream);

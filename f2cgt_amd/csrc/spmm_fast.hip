@@ -212,6 +212,8 @@ int launch_sq_block(SqBlockArgs a, const void* indptr, const void* indices, int 
   constexpr int NOUT = LB * (8 / BITS);
   const int chunks = a.feat_dim / NOUT;
   a.cp2 = pow2_ceil(chunks);
+  // a row's chunks must fit one workgroup: with no lane group left the kernel's loops would not advance
+  if (chunks < 1 || a.cp2 > kBlock) return fail(F2CGT_E_UNSUPPORTED, "%s: %d columns exceed the row-block kernel", what, a.feat_dim);
   a.pitch = (chunks * LB + 3) & ~3;
   const int lut_bytes = AFFINE ? 0 : (((a.num_codebooks << BITS) + 3) & ~3) * 4;
   a.edge_cap = kStageBytes / (a.pitch + 4);
@@ -226,6 +228,10 @@ int launch_sq_block(SqBlockArgs a, const void* indptr, const void* indices, int 
                      (size_t)a.edge_cap * a.pitch;
   const int64_t grid = ceil_div(a.R, a.rows_per_block);
   if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
+  if (plan_only()) {
+    plan_record("sq_block_kernel", grid, kBlock, (int64_t)lds, a.rows_per_block, kBlock / a.cp2, a.edge_cap);
+    return 0;
+  }
   if (idx_dtype == F2CGT_DT_I32)
     sq_block_kernel<BITS, LB, AFFINE, int32_t><<<(unsigned)grid, kBlock, lds, st>>>(
         a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
@@ -560,6 +566,11 @@ int launch_acc_tb(AccArgs a, size_t lds, int64_t grid, const void* indptr, const
   a.fin_slots = TB / a.fin_group;
   a.fin_magic = (uint32_t)((65536 + a.fin_group - 1) / a.fin_group);
   a.nt_out = stream_output(a.R * (int64_t)a.feat_dim * 4) ? 1 : 0;
+  if (plan_only()) {
+    plan_record("sq_affine_acc_kernel", grid, TB, (int64_t)lds, a.rows_per_block, a.fin_slots, TB >> a.lane_shift,
+                a.sub_rows, a.edge_batch);
+    return 0;
+  }
   if (idx_dtype == F2CGT_DT_I32)
     sq_affine_acc_kernel<TB, BITS, int32_t><<<(unsigned)grid, TB, lds, st>>>(
         a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
@@ -853,6 +864,11 @@ int launch_sq_rows(RowsArgs a, const void* indptr, const void* indices, int idx_
                      (size_t)a.edge_cap * a.pitch + 16;
   const int64_t grid = ceil_div(a.R, rb);
   if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
+  if (plan_only()) {
+    plan_record("sq_rows_kernel", grid, TB, (int64_t)lds, a.rows_per_block, a.fin_slots, TB >> a.lane_shift,
+                a.edge_cap);
+    return 0;
+  }
   if (idx_dtype == F2CGT_DT_I32)
     sq_rows_kernel<BITS, AFFINE, int32_t, TB><<<(unsigned)grid, TB, lds, st>>>(
         a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
@@ -1097,13 +1113,19 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
 
 }  // namespace
 
+// The staged-rows kernel keeps at least eight edges of `pitch + 4` bytes in its 20 KB of staging.
+static bool sq_rows_pitch_ok(int feat_dim, int target_bits) {
+  return (((int64_t)feat_dim * target_bits + 63) / 64) * 8 + 4 <= 2048;
+}
+
 bool sq_block_eligible(const void* codes, const float* out, int64_t N, int64_t src_dim, int feat_dim,
                        int target_bits, int64_t lut_entries) {
   if ((target_bits == 1 || target_bits == 2 || target_bits == 4 || target_bits == 8) && feat_dim % 4 == 0 &&
       (int64_t)feat_dim * target_bits >= 64 &&
-      src_dim >= 8 && feat_dim <= 4096 && aligned(out, 16) && N < (1ll << 32) && src_dim < (1ll << 24) &&
-      src_dim * (8 / target_bits) >= feat_dim && lut_entries * 4 <= 16 * 1024)
-    return true;  // staged-rows kernel (any row pitch, float4 column groups)
+      src_dim >= 8 && feat_dim <= 4096 && sq_rows_pitch_ok(feat_dim, target_bits) && aligned(out, 16) &&
+      N < (1ll << 32) && src_dim < (1ll << 24) && src_dim * (8 / target_bits) >= feat_dim &&
+      lut_entries * 4 <= 16 * 1024)
+    return true;  // staged-rows kernel (any row pitch up to 2 KB, float4 column groups)
   int lb, nout;
   switch (target_bits) {
     case 8: lb = 4; nout = 4; break;
@@ -1128,7 +1150,7 @@ int sq_block_run(bool affine, const uint8_t* codes, const float* table, int64_t 
   // the 128-thread staged-rows kernel (degree-ordered rows) covers every shape with float4 column
   // groups; the 256-thread block kernel below stays for the remaining ones
   if (feat_dim % 4 == 0 && (int64_t)feat_dim * target_bits >= 64 && src_dim >= 8 && feat_dim <= 4096 &&
-      ((feat_dim * target_bits + 63) / 64) * 8 + 4 <= 2048) {
+      sq_rows_pitch_ok(feat_dim, target_bits)) {
     RowsArgs r{};
     r.codes = codes; r.table = table; r.param_stride = param_stride; r.column_slice = column_slice;
     r.num_codebooks = num_codebooks; r.R = R; r.E = E; r.N = N; r.src_dim = (int)src_dim; r.feat_dim = feat_dim;
@@ -1208,6 +1230,11 @@ int launch_hybrid(HybArgs a, const void* indptr, const void* indices, int idx_dt
   const int64_t grid = ceil_div(a.R, rb);
   if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
   const bool vec4 = a.feat_dim % 16 == 0 && aligned(a.sq_codes, 16) && a.ch2 >= 4;
+  if (plan_only()) {
+    plan_record("hybrid_acc_kernel", grid, TB, (int64_t)lds, a.rows_per_block, vec4 ? TB / (a.ch2 >> 2) : TB / a.ch2,
+                vec4 ? 4 : 1, a.edge_batch);
+    return 0;
+  }
   const int32_t* ip32 = static_cast<const int32_t*>(indptr);
   const int32_t* ix32 = static_cast<const int32_t*>(indices);
   const int64_t* ip64 = static_cast<const int64_t*>(indptr);
@@ -1225,7 +1252,8 @@ int launch_hybrid(HybArgs a, const void* indptr, const void* indices, int idx_dt
 bool hybrid_acc_eligible(const void* sq_codes, const float* vq_codebooks, const float* out, int64_t N,
                          int64_t n_sq, int64_t n_vq, int feat_dim, int w) {
   if (!aligned(sq_codes, 4) || !aligned(out, 16) || !aligned(vq_codebooks, 16)) return false;
-  if (feat_dim < 4 || feat_dim % 4 != 0 || feat_dim > 1024 || w % 4 != 0) return false;
+  // (feat_dim 4 is one chunk per row: its reciprocal 2^32 does not fit the 32-bit multiplier)
+  if (feat_dim < 8 || feat_dim % 4 != 0 || feat_dim > 1024 || w % 4 != 0) return false;
   if (N >= (1ll << 32) || n_sq >= (1ll << 30) || n_vq >= (1ll << 30)) return false;
   return true;
 }

@@ -304,7 +304,8 @@ template <int BITS, bool AFFINE>
 int decode_f4_launch(const uint8_t* codes, float* out, const float* table, int64_t param_stride,
                      int64_t column_slice, int n_cb, int64_t rows, int64_t src_dim, int64_t feat_dim,
                      hipStream_t st, const char* what) {
-  if (feat_dim % 4 != 0 || feat_dim > 8192 || !aligned(out, 16)) return -1;
+  // (one float4 per row would need the reciprocal 2^32, which does not fit the 32-bit multiplier)
+  if (feat_dim % 4 != 0 || feat_dim < 8 || feat_dim > 8192 || !aligned(out, 16)) return -1;
   const size_t lds = AFFINE ? (size_t)feat_dim * 8
                             : ((((size_t)n_cb << BITS) + 3) / 4 * 4 + (size_t)feat_dim) * 4;
   if (lds > (size_t)kMaxLutBytes) return -1;
@@ -450,7 +451,9 @@ template <int BITS, bool STORAGE>
 int encode_f4_launch(const float* src, void* dst, const float* codebooks, int64_t column_slice, int n_cb,
                      int64_t rows, int64_t feat_dim, int64_t dst_dim, hipStream_t st, const char* what) {
   constexpr int COLS = (STORAGE && BITS == 1) ? 8 : 4;
-  if (feat_dim % COLS != 0 || feat_dim > 8192 || !aligned(src, 16) || (!STORAGE && !aligned(dst, 16)) ||
+  // (one lane per row would need the reciprocal 2^32, which does not fit the 32-bit multiplier)
+  if (feat_dim % COLS != 0 || feat_dim < 2 * COLS || feat_dim > 8192 || !aligned(src, 16) ||
+      (!STORAGE && !aligned(dst, 16)) ||
       (STORAGE && BITS == 16 && !aligned(dst, 8)))
     return -1;
   F4Args a{};
@@ -598,6 +601,10 @@ extern "C" int f2cgt_sq_decompress(const void* codes, int code_dtype, float* out
     case 1: case 2: case 4: case 8:
       F2CGT_REQUIRE(byte_codes, F2CGT_E_UNSUPPORTED,
                     "sq_decompress: %d-bit codes must be uint8 or int8", target_bits);
+      // 8-bit codes are signed (sq_compress yields -128..127); the reference reads a uint8 tensor as
+      // 0..255, values its encoder never produces, so that combination is refused instead of guessed
+      F2CGT_REQUIRE(target_bits != 8 || code_dtype == F2CGT_DT_I8, F2CGT_E_UNSUPPORTED,
+                    "sq_decompress: 8-bit codes are signed, pass them as int8 (got uint8)");
       F2CGT_REQUIRE(src_dim * (8 / target_bits) >= feat_dim, F2CGT_E_INVALID,
                     "sq_decompress: %lld packed bytes per row cannot hold %lld columns",
                     (long long)src_dim, (long long)feat_dim);

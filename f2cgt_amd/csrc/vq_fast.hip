@@ -550,6 +550,10 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
 template <int BT, int H, int RPM>
 int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
                 const char* what, unsigned grid, size_t wlds) {
+  if (plan_only()) {
+    plan_record("vq_wave_kernel", grid, kThreads, (int64_t)wlds, 0, H, RPM, a.dense_store);
+    return 0;
+  }
   const void* kern = idx_dtype == F2CGT_DT_I32 ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t>)
                                                : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t>);
   const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
@@ -597,6 +601,10 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     if (avg_deg <= 60.0) return launch_wave<BT, 2, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
   } else if (avg_deg <= 15.0) {
     return launch_wave<BT, 1, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+  }
+  if (plan_only()) {
+    plan_record("vq_pipe_kernel", grid, kThreads, (int64_t)lds, kRows);
+    return 0;
   }
   const void* kern = idx_dtype == F2CGT_DT_I32 ? reinterpret_cast<const void*>(vq_pipe_kernel<BT, int32_t>)
                                                : reinterpret_cast<const void*>(vq_pipe_kernel<BT, int64_t>);

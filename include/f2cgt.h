@@ -56,6 +56,26 @@ const char* f2cgt_last_error(void);
 /* Number of compute units of the current device (the kernels size their grids by it). */
 int f2cgt_num_cus(void);
 
+/* Dry runs of the fused aggregation entry points (no counterpart in the reference; for tests and
+ * tools that want to know what a shape dispatches to, with or without a GPU).  While switched on
+ * for the calling thread, f2cgt_spmm_csr and the f2cgt_*_spmm_csr operators validate their
+ * arguments and choose kernel and launch geometry exactly as usual, then return 0 without touching
+ * the device or dereferencing any pointer (pointers only need the alignment of the real buffers;
+ * the device is taken to have 256 compute units).  f2cgt_last_plan copies the last choice:
+ * grid / block / lds_bytes of the launch, destination rows per workgroup (0 = not row-blocked),
+ * and kernel-specific lane-group counts in aux[] (every one of them must be >= 1 for the kernel's
+ * loops to advance).  f2cgt_set_plan_only returns the previous setting. */
+typedef struct {
+  char kernel[48];
+  int64_t grid;
+  int32_t block;
+  int64_t lds_bytes;
+  int32_t rows_per_block;
+  int32_t aux[4];
+} f2cgt_plan;
+int f2cgt_set_plan_only(int on);
+int f2cgt_last_plan(f2cgt_plan* out);
+
 /* ---- bit packing ------------------------------------------------------------- */
 
 /* Replaces packbits(), src/packbits.cu:44-64 (kernel :6-42).
@@ -89,8 +109,10 @@ int f2cgt_sq_encode(const float* src, void* dst, const float* codebooks, int64_t
                     void* stream);
 
 /* Replaces sq_decompress(), src/sq_quantization.cu:158-182 (kernel :85-156).
- * codes [rows, src_dim] of code_dtype (U8/I8 packed bytes for bits < 8, I8/U8 for 8,
- * I16 for 16) -> out fp32 [rows, feat_dim].  Codebook per OUTPUT column. */
+ * codes [rows, src_dim] of code_dtype (U8/I8 packed bytes for bits < 8, I8 for 8, I16 for 16)
+ * -> out fp32 [rows, feat_dim].  Codebook per OUTPUT column.  8-bit codes are signed; U8 with
+ * target_bits 8 is refused (F2CGT_E_UNSUPPORTED): the reference's dtype dispatch
+ * (src/common.h:68-82) would read such a tensor as 0..255, which its encoder never writes. */
 int f2cgt_sq_decompress(const void* codes, int code_dtype, float* out, const float* codebooks,
                         int64_t rows, int64_t src_dim, int64_t feat_dim,
                         int64_t num_codebooks, int target_bits, int64_t column_slice,
@@ -133,7 +155,8 @@ int f2cgt_vq_decompress_spmm_csr(const void* codes, int code_dtype, const float*
 
 /* Replaces SqDecompressSpMMFusionCsr(), src/fusion_spmm.cu:240-272 (kernel :143-238).
  * Codebook per PACKED BYTE (:180): byte j uses codebook j*(8/bits) / column_slice, which
- * equals the per-column choice of f2cgt_sq_decompress iff column_slice % (8/bits) == 0. */
+ * equals the per-column choice of f2cgt_sq_decompress iff column_slice % (8/bits) == 0.
+ * Code dtypes as for f2cgt_sq_decompress (8-bit codes must be I8). */
 int f2cgt_sq_decompress_spmm_csr(const void* codes, int code_dtype, const float* codebooks,
                                  const void* indptr, const void* indices, int idx_dtype,
                                  float* out, int64_t num_rows, int64_t num_edges,
