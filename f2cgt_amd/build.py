@@ -42,7 +42,10 @@ def _run(cmd):
     return proc.stdout
 
 
-def build_capi(verbose=True):
+def build_capi(verbose=True, experiments=False):
+    """experiments=True also compiles the kernels that were measured and not adopted (they are
+    selected at run time by the environment variables their sources name); the shipped library
+    is built without them."""
     os.makedirs(LIB, exist_ok=True)
     os.makedirs(OBJ, exist_ok=True)
     hipcc = shutil.which("hipcc") or os.path.join(ROCM, "bin", "hipcc")
@@ -50,7 +53,8 @@ def build_capi(verbose=True):
 
     def compile_one(src):
         obj = os.path.join(OBJ, src.replace(".hip", ".o"))
-        out = _run([hipcc, *HIP_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
+        extra = ["-DF2CGT_EXPERIMENTS=1"] if experiments else []
+        out = _run([hipcc, *HIP_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj])
         if verbose and out.strip():
             print(out)
         return obj
@@ -90,11 +94,11 @@ def build_extension(verbose=True):
     return EXT_LIB
 
 
-def build_all(verbose=True):
-    build_capi(verbose)
+def build_all(verbose=True, experiments=False):
+    build_capi(verbose, experiments)
     build_extension(verbose)
 
 
 if __name__ == "__main__":
-    build_all()
+    build_all(experiments="--experiments" in sys.argv[1:])
     sys.exit(0)

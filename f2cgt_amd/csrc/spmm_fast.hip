@@ -16,6 +16,8 @@
 // per-row loop inside the same kernel.
 #include "spmm_fast.hpp"
 
+#include <cstdlib>
+
 namespace f2cgt {
 namespace {
 
@@ -559,6 +561,157 @@ __global__ __launch_bounds__(TB) void sq_affine_acc_kernel(AccArgs a, const Idx*
     acc_block<TB, BITS, 2, Idx>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
 }
 
+#ifdef F2CGT_EXPERIMENTS
+// ---- persistent form (measured, not adopted) ---------------------------------------------------
+// A block's life is a chain of dependent memory round trips (indptr -> indices -> code rows) before
+// its first store, and with 2-10 edges per row the launch is over after two or three such chains per
+// workgroup slot.  Here a workgroup walks the blocks blk, blk + grid, ... and fetches the row
+// offsets and the source ids of its next block into registers while the current one gathers and
+// stores, so only the code-row fetch of every block after the first stays on the critical path.
+// The barriers order LDS traffic only (a workgroup-scope fence on the whole address space would
+// drain the loads in flight at every barrier).  On the 2.5e5-row power-law block it ran at 24.4 us
+// against 23.1 us for one workgroup per block: the hardware already starts a new workgroup the
+// moment a slot frees, and 13-14 of them per CU overlap their chains as well as the prefetch does.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+template <int TB, int BITS, typename Idx>
+__global__ __launch_bounds__(TB) void sq_affine_acc_pkernel(AccArgs a, const Idx* __restrict__ indptr,
+                                                            const Idx* __restrict__ indices,
+                                                            float* __restrict__ out) {
+  constexpr int CAP_N = BITS == 4 ? 17 : 257;
+  constexpr int CAP_W = BITS == 4 ? 4369 : 257;
+  constexpr int NID = 2;   // prefetched source ids per thread: edge_batch = NID * TB
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint32_t* s_acc = reinterpret_cast<uint32_t*>(smem);                         // [sub_rows][pitch_n]
+  int* s_ptr = reinterpret_cast<int*>(s_acc + (size_t)a.sub_rows * a.pitch_n);  // [RB + 1]
+  float* s_rdeg = reinterpret_cast<float*>(s_ptr + a.rows_per_block + 4);      // [RB]
+  uint32_t* s_wflag = reinterpret_cast<uint32_t*>(s_rdeg + a.rows_per_block);  // [waves]
+  uint2* s_edge = reinterpret_cast<uint2*>(s_wflag + 4);                       // [edge_batch]
+
+  const int t = threadIdx.x;
+  const int rb = a.rows_per_block;       // rb + 1 <= TB: one row offset per thread
+  const int64_t nblocks = (a.R + rb - 1) / rb;
+  const FinParams first = acc_fin_params(a);
+  const int64_t e_last = a.E > 0 ? a.E - 1 : 0;
+
+  // row offsets of a block, one per thread, plus its first and last offset for everybody
+  Idx p_lo = 0, p_hi = 0, p_e0 = 0, p_end = 0;
+  auto fetch_ptr = [&](int64_t blk) {
+    const int64_t row0 = blk * rb;
+    const int nr = (int)((a.R - row0) < rb ? (a.R - row0) : rb);
+    const int i = t <= nr ? t : nr;
+    p_lo = indptr[row0 + i];
+    p_hi = indptr[row0 + (i < nr ? i + 1 : nr)];
+    p_e0 = indptr[row0];
+    p_end = indptr[row0 + nr];
+  };
+  Idx ids[NID];
+#pragma unroll
+  for (int j = 0; j < NID; ++j) ids[j] = 0;
+  bool ids_ready = false;   // ids[] hold the first edges of the block about to start
+
+  int64_t blk = blockIdx.x;
+  if (blk < nblocks) fetch_ptr(blk);
+  for (; blk < nblocks; blk += gridDim.x) {
+    const int64_t row0 = blk * rb;
+    const int nrows = (int)((a.R - row0) < rb ? (a.R - row0) : rb);
+    int64_t e0 = (int64_t)p_e0;
+    e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
+    uint32_t level = 0;
+    if (t <= nrows) {
+      int64_t v = (int64_t)p_lo;
+      v = v < e0 ? e0 : (v > a.E ? a.E : v);
+      const int p = (int)(v - e0 > 0x7fffffff ? 0x7fffffff : v - e0);
+      s_ptr[t] = p;
+      if (t < nrows) {
+        int64_t v2 = (int64_t)p_hi;
+        v2 = v2 < e0 ? e0 : (v2 > a.E ? a.E : v2);
+        const int deg = (int)(v2 - e0 > 0x7fffffff ? 0x7fffffff : v2 - e0) - p;
+        s_rdeg[t] = deg > 0 ? __builtin_amdgcn_rcpf((float)deg) : 0.f;
+        level = (deg > CAP_N ? 1u : 0u) | (deg > CAP_W ? 2u : 0u);
+      }
+    }
+    {
+      const uint32_t wl = (__ballot(level & 1u) ? 1u : 0u) | (__ballot(level & 2u) ? 2u : 0u);
+      if ((t & (kWave - 1)) == 0) s_wflag[t / kWave] = wl;
+    }
+    // the row offsets of the next block start their trip now
+    const int64_t next = blk + gridDim.x;
+    const bool has_next = next < nblocks;
+    if (has_next) fetch_ptr(next);
+    lds_barrier();
+    uint32_t block_level = 0;
+#pragma unroll
+    for (int w = 0; w < TB / kWave; ++w) block_level |= s_wflag[w];
+    const int ne = s_ptr[nrows];
+    const bool simple = block_level == 0 && ne <= a.edge_batch && nrows <= a.sub_rows;
+    if (simple) {
+      // every edge of the block is tagged once; the ids come from the registers when they were prefetched
+      uint32_t* flat = reinterpret_cast<uint32_t*>(s_edge);
+#pragma unroll
+      for (int j = 0; j < NID; ++j) {
+        const int i = t + j * TB;
+        if (i < ne) {
+          const Idx raw = ids_ready ? ids[j] : indices[e0 + i];
+          flat[2 * i] = (uint32_t)clamp_idx(raw, a.N);
+        }
+      }
+      if (t < nrows) {
+        const int b = s_ptr[t], e = s_ptr[t + 1];
+        for (int k = b; k < e; ++k) flat[2 * k + 1] = (uint32_t)t;
+      }
+      acc_zero<TB>(s_acc, nrows * a.pitch_n);
+      lds_barrier();
+      acc_gather<TB, BITS, 2>(a, s_acc, s_edge, 0, ne, 0, a.pitch_n);
+    } else {
+      lds_barrier();   // (keeps the barrier count of the two branches equal)
+    }
+    // the source ids of the next block: its offsets have had the gather to arrive
+    ids_ready = false;
+    if (has_next) {
+      int64_t e0n = (int64_t)p_e0, e1n = (int64_t)p_end;
+      e0n = e0n < 0 ? 0 : (e0n > a.E ? a.E : e0n);
+      e1n = e1n < e0n ? e0n : (e1n > a.E ? a.E : e1n);
+      if (e1n - e0n <= a.edge_batch) {
+        ids_ready = true;
+#pragma unroll
+        for (int j = 0; j < NID; ++j) {
+          int64_t at = e0n + t + j * TB;
+          at = at > e_last ? e_last : at;
+          ids[j] = indices[at];
+        }
+      }
+    }
+    if (simple) {
+      lds_barrier();
+      acc_finalize<TB, BITS, 2>(a, first, s_acc, s_rdeg, row0, 0, nrows, a.pitch_n, out);
+    } else if (block_level & 2u) {
+      const bool is64 = sizeof(Idx) == 8;
+      acc_direct_block<TB, BITS>(a, s_ptr, e0, row0, nrows,
+                                 is64 ? reinterpret_cast<const int64_t*>(indices) : nullptr,
+                                 is64 ? nullptr : reinterpret_cast<const int32_t*>(indices), out);
+    } else if (BITS == 4 && (block_level & 1u)) {
+      acc_block<TB, BITS, 4, Idx>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
+    } else {
+      acc_block<TB, BITS, 2, Idx>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
+    }
+    lds_barrier();   // the block's LDS is reused by the next one
+  }
+}
+
+#endif  // F2CGT_EXPERIMENTS
+
+#ifdef F2CGT_EXPERIMENTS
+static bool acc_persistent_enabled() {   // F2CGT_ACC_PERSIST=1 selects the persistent form
+  const char* v = getenv("F2CGT_ACC_PERSIST");
+  return v != nullptr && v[0] == '1';
+}
+#endif
+
 template <int TB, int BITS>
 int launch_acc_tb(AccArgs a, size_t lds, int64_t grid, const void* indptr, const void* indices, int idx_dtype,
                   float* out, hipStream_t st, const char* what) {
@@ -571,6 +724,22 @@ int launch_acc_tb(AccArgs a, size_t lds, int64_t grid, const void* indptr, const
                 a.sub_rows, a.edge_batch);
     return 0;
   }
+#ifdef F2CGT_EXPERIMENTS
+  if (a.rows_per_block + 1 <= TB && a.edge_batch == 2 * TB && acc_persistent_enabled()) {
+    // as many workgroups as the device holds at once (LDS bound), each walking blocks grid apart
+    int64_t per_cu = lds > 0 ? (int64_t)(160 * 1024) / (int64_t)lds : 16;
+    per_cu = per_cu > 2048 / TB ? 2048 / TB : (per_cu < 1 ? 1 : per_cu);
+    int64_t pgrid = per_cu * num_cus();
+    pgrid = pgrid > grid ? grid : pgrid;
+    if (idx_dtype == F2CGT_DT_I32)
+      sq_affine_acc_pkernel<TB, BITS, int32_t><<<(unsigned)pgrid, TB, lds, st>>>(
+          a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
+    else
+      sq_affine_acc_pkernel<TB, BITS, int64_t><<<(unsigned)pgrid, TB, lds, st>>>(
+          a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
+    return launch_status(what);
+  }
+#endif
   if (idx_dtype == F2CGT_DT_I32)
     sq_affine_acc_kernel<TB, BITS, int32_t><<<(unsigned)grid, TB, lds, st>>>(
         a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
@@ -607,6 +776,12 @@ int launch_acc(AccArgs a, const void* indptr, const void* indices, int idx_dtype
   while (sub > 8 && sub * acc_row > 24 * 1024) sub -= 8;
   int rb = sub * (int)(0.6 * a.edge_batch / (dg * sub));
   rb = rb < sub ? sub : (rb > 256 ? 256 / sub * sub : rb);
+#ifdef F2CGT_EXPERIMENTS
+  if (const char* v = getenv("F2CGT_ACC_RB")) {   // rows per block, a multiple of 8
+    const int want = atoi(v);
+    if (want >= 8) { sub = want / 8 * 8; rb = sub; }
+  }
+#endif
   a.rows_per_block = rb;
   a.sub_rows = sub;
   const size_t lds = sub * acc_row + (size_t)(rb + 4) * 4 + (size_t)rb * 4 + 16 + (size_t)a.edge_batch * 8 + 16;

@@ -18,6 +18,9 @@
 // Workgroups are bound to a (column tile, row stripe); wide features (D = 768) use six tiles.
 #include "spmm_fast.hpp"
 
+#include <cstdlib>
+#include <type_traits>
+
 namespace f2cgt {
 namespace {
 
@@ -536,6 +539,9 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
             if (sub != 0) continue;
           }
           mean(n, acc);
+#ifdef F2CGT_EXPERIMENTS
+          if (a.dense_store == 2 && acc[0][0] != 12345.678f) continue;   // no stores: what the rest of the kernel costs
+#endif
 #pragma unroll
           for (int h = 0; h < H; ++h)
             store_nt4(orow + (int64_t)row * a.feat_dim + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
@@ -546,6 +552,352 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     eb1 = eb2; ne1 = ne2;
   }
 }
+
+#ifdef F2CGT_EXPERIMENTS
+// ---- strip variant: a lane owns 32 columns of a row --------------------------------------------
+// The vector ALUs bound this operator before HBM or LDS do: the 128 adds of an edge and column tile
+// are two wave instructions, and everything else a wave executes per edge comes on top of them.
+// Here a quad of lanes owns a destination row of the 128-column tile and a wave works on 16 rows at
+// a time: a lane reads its own code bytes straight from HBM (one load per edge; nothing is staged
+// in LDS), turns them into LDS addresses once per code, and issues eight 16-byte reads per edge.
+// The LDS serves 16 consecutive lanes together from 64 four-byte banks, so those lanes (four rows)
+// must hit 16 different 16-byte groups of a 256-byte window whatever their codes are: lane l reads
+// chunk j ^ x(l) of its 128 bytes in step j (x = 2 * (row & 3) + (quarter >> 1); the quarter's low
+// bit picks the half of the window), i.e. the address of step 0 xor (j << 4).  The accumulators are
+// therefore held in step order.  For the stores they go, four rows at a time, through 2 KB of
+// wave-private staging laid out like the output tile and come back one float4 per lane in address
+// order: every store instruction writes two whole 512-byte row pieces.
+// Per wave the stages of consecutive 16-row groups are software pipelined through registers:
+//     P  indptr[row], indptr[row + 1]                    issued three groups ahead
+//     I  the row's first KE source ids, four per lane     two groups ahead
+//     C  the lane's code bytes of those KE edges          one group ahead (ids handed round the quad)
+//     X  codebook reads + adds in edge order, mean
+//     S  staging round trips + stores of the group before, spread over the first eight edges of X
+//        (two waves per SIMD cannot hide an LDS round trip that nothing else is issued behind)
+// Rows with more than KE edges finish their tail straight from HBM (same order, unpipelined).
+constexpr int kSRows = 16;     // rows per group (64 lanes / 4)
+
+template <int W> struct strip_code;
+template <> struct strip_code<8> { using type = uint32_t; };
+template <> struct strip_code<16> { using type = uint16_t; };
+template <> struct strip_code<32> { using type = uint8_t; };
+
+template <int S>
+__device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, S * 0x55, 0xf, 0xf, true);
+}
+
+template <int W, int KE, bool IL, int kSThreads, int kStgRows, typename Idx>
+__global__ __launch_bounds__(kSThreads) void vq_strip_kernel(VqArgs a, const Idx* __restrict__ indptr,
+                                                             const Idx* __restrict__ indices,
+                                                             float* __restrict__ out) {
+  // IL (32-wide codes only): the lanes of a quad interleave instead of owning a quarter each: lane t
+  // holds the chunks 4 i + t of the row's 32, so a quad's store i is 64 contiguous bytes and nothing
+  // has to be turned round; a lane then needs all four codes of the tile (one dword), and the rows
+  // of a 16-lane group stay conflict free by walking i in the order i ^ (row & 3).
+  static_assert(!IL || W == 32, "interleaved quads need one code per 32 columns");
+  using CT = typename strip_code<IL ? 8 : W>::type;
+  typedef float f4v __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) f4v lds_float4;
+  constexpr int kWaves = kSThreads / 64;
+  constexpr int BT = 128 / W;           // code bytes per row and tile
+  constexpr int NCODE = IL ? 4 : BT / 4;   // codes a lane reads per edge
+  constexpr int CPC = 8 / NCODE;        // 16-byte chunks per code
+  constexpr int XSH = IL ? 6 : 4;       // the steps of one code differ in this address bit (and up)
+  static_assert(KE % 4 == 0 && KE >= 8 && KE <= 16, "edges per row held in registers");
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* s_cb = reinterpret_cast<float*>(smem);
+  const int wave = uni((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+
+  int tile, stripe;
+  if (a.stripes_per_xcd > 0) {
+    const int xcd = blockIdx.x % kXcds, k = blockIdx.x / kXcds;
+    if (k >= a.stripes_per_xcd * a.n_tiles) return;
+    tile = k % a.n_tiles;
+    stripe = xcd * a.stripes_per_xcd + k / a.n_tiles;
+  } else {
+    tile = blockIdx.x % a.n_tiles;
+    stripe = blockIdx.x / a.n_tiles;
+  }
+  const int tile_cols = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
+  stage_codebook_tile<kSThreads, false>(s_cb, a.codebooks, a.K, a.w, tile, tile_cols);
+  __syncthreads();
+
+  const int64_t total_waves = (int64_t)a.n_stripes * kWaves;
+  const int64_t rows_per_wave = ((a.R + total_waves - 1) / total_waves + kSRows - 1) / kSRows * kSRows;
+  const int64_t row_begin = ((int64_t)stripe * kWaves + wave) * rows_per_wave;
+  if (row_begin >= a.R) return;
+  const int64_t row_end = row_begin + rows_per_wave < a.R ? row_begin + rows_per_wave : a.R;
+  const int64_t n_groups = (row_end - row_begin + kSRows - 1) / kSRows;
+
+  const int q = lane & 3, rr = lane >> 2, x = IL ? (rr & 3) : (((rr & 3) << 1) | (q >> 1));
+  // LDS addresses (the tile starts the workgroup's LDS; staging follows it)
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+  // step 0 inside a code's 512 bytes: chunk x of the lane's quarter, or chunk 4 x + q of the row
+  const uint32_t lane_base = lds0 + (IL ? (uint32_t)(x * 64 + q * 16) : (uint32_t)(q * 128 + x * 16));
+  uint32_t lane_base_s[NCODE];   // ... of the first step of code s: steps j = s * CPC + r read at (this ^ (r << XSH))
+#pragma unroll
+  for (int s = 0; s < NCODE; ++s) lane_base_s[s] = lane_base ^ (uint32_t)((s * CPC) << XSH);
+  const uint32_t stg0 = lds0 + (uint32_t)a.K * 512u + (uint32_t)(wave * kStgRows * 512);
+  const uint32_t stg_wr = stg0 + (uint32_t)((rr & (kStgRows - 1)) * 512 + q * 128 + x * 16);  // chunk of step 0
+  const uint32_t stg_rd = stg0 + (uint32_t)(lane * 16);
+  // byte i of the permuted code word = code of the chunks (i * CPC ..) ^ x
+  const uint32_t slot_x = (uint32_t)(x / CPC);   // (interleaved: steps 2 m, 2 m + 1 belong to quarter m ^ (x >> 1))
+  const uint32_t sel = (0u ^ slot_x) | ((1u ^ slot_x) << 8) | ((2u ^ slot_x) << 16) | ((3u ^ slot_x) << 24);
+  const uint8_t* code_base = a.codes + tile * BT + (IL ? 0 : q * NCODE);
+  const uint32_t n_last = (uint32_t)(a.N - 1);
+  const int64_t e_last = a.E - 1;
+  // a lane's float4 of the staged rows: column (lane & 31) * 4 of staged row 2 i + (lane >> 5)
+  const uint32_t out_lane = (uint32_t)((lane & 31) * 4) + (uint32_t)(lane >> 5) * (uint32_t)a.feat_dim;
+  const bool col_ok = (lane & 31) * 4 < tile_cols;
+  const bool nt = a.dense_store == 1 || a.dense_store == 3;
+
+  // pipeline registers: two generations of everything that is in flight for two steps
+  Idx praw0[2] = {0, 0}, praw1[2] = {0, 0};          // P -> I
+  Idx iraw[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};     // I -> C
+  int degq[5] = {0, 0, 0, 0, 0};                     // degq[d]: degree of this lane's row in group g + d
+  CT cbuf[2][KE];                                     // C -> X (copied out at the top of the step that uses them)
+#pragma unroll
+  for (int k = 0; k < KE; ++k) cbuf[0][k] = cbuf[1][k] = 0;
+
+  auto group_row = [&](int64_t g) {            // row of this lane in group g (groups past the end repeat the last)
+    const int64_t gg = g < n_groups ? g : n_groups - 1;
+    return row_begin + gg * kSRows + rr;
+  };
+  auto edge_reads = [&](uint32_t cw, f4v (&v)[8]) {
+    uint32_t pw = cw;
+    if (NCODE > 1) pw = __builtin_amdgcn_perm(cw, cw, sel);
+    uint32_t addr[NCODE];
+#pragma unroll
+    for (int s = 0; s < NCODE; ++s) addr[s] = (((pw >> (8 * s)) & 0xffu) << 9) + lane_base_s[s];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      v[j] = *(const lds_float4*)(uintptr_t)(addr[j / CPC] ^ (uint32_t)((j % CPC) << XSH));
+  };
+  auto add_edge = [&](uint32_t cw, float (&acc)[8][4]) {
+    f4v v[8];
+    edge_reads(cw, v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      acc[j][0] += v[j][0]; acc[j][1] += v[j][1]; acc[j][2] += v[j][2]; acc[j][3] += v[j][3];
+    }
+  };
+  // The stores of group g in eight steps: ops 0, 2, 4, 6 put the rows [4 p, 4 p + 4) of the group
+  // into the staging area (chunk j ^ x of a lane at its place in the row); ops 1, 3, 5, 7 fetch them
+  // back in address order (stage_fetch) and, once the edge work issued behind that has covered the
+  // round trip, store them (stage_store).
+  auto stage_put = [&](int p, const float (&acc)[8][4]) {
+    __builtin_amdgcn_wave_barrier();
+    if ((rr / kStgRows) == p) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        *(lds_float4*)(uintptr_t)(stg_wr ^ (uint32_t)(j << 4)) = f4v{acc[j][0], acc[j][1], acc[j][2], acc[j][3]};
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  auto stage_fetch = [&](f4v (&sv)[kStgRows / 2]) {
+#pragma unroll
+    for (int i = 0; i < kStgRows / 2; ++i) sv[i] = *(const lds_float4*)(uintptr_t)(stg_rd + (uint32_t)(i * 1024));
+    __builtin_amdgcn_wave_barrier();
+  };
+  auto stage_store = [&](int p, const f4v (&sv)[kStgRows / 2], int64_t g) {
+    const int64_t grow0 = row_begin + g * kSRows + p * kStgRows;    // uniform
+    float* obase = out + grow0 * (int64_t)a.feat_dim + tile * 128;  // uniform
+#pragma unroll
+    for (int i = 0; i < kStgRows / 2; ++i) {
+      const int64_t lrow = grow0 + 2 * i + (lane >> 5);
+      if (lrow < row_end && col_ok) {
+        float* o = obase + (int64_t)(2 * i) * a.feat_dim + out_lane;
+        if (nt) store_nt4(o, sv[i][0], sv[i][1], sv[i][2], sv[i][3]);
+        else *reinterpret_cast<float4*>(o) = make_float4(sv[i][0], sv[i][1], sv[i][2], sv[i][3]);
+      }
+    }
+  };
+  // interleaved quads: store i of a lane is the chunk 4 (i ^ x) + q of its row, straight from the registers
+  auto direct_store = [&](int i, const float (&acc)[8][4], int64_t g) {
+    const int64_t row = row_begin + g * kSRows + rr;
+    const int col = ((i ^ x) << 4) + q * 4;
+    if (row < row_end && col < tile_cols) {
+      float* o = out + row * (int64_t)a.feat_dim + tile * 128 + col;
+      if (nt) store_nt4(o, acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
+      else *reinterpret_cast<float4*>(o) = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
+    }
+  };
+  auto store_op = [&](int op, const float (&acc)[8][4], int64_t g) {   // unpipelined form
+    if (IL) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (i == op) direct_store(i, acc, g);
+      return;
+    }
+    if ((op & 1) == 0) {
+      stage_put(op >> 1, acc);
+    } else {
+      f4v sv[kStgRows / 2];
+      stage_fetch(sv);
+      stage_store(op >> 1, sv, g);
+    }
+  };
+
+  // One step = one 16-row group.  Loads are consumed two steps after they were issued and the
+  // results are stored at the end of the step: the memory counter retires loads and stores in
+  // issue order, so a wait for a load also waits for every older store, and a store takes several
+  // microseconds to be acknowledged while the write path is busy.  With this order the youngest
+  // store a wait can depend on is two steps old.
+  auto step = [&](auto par, int64_t g) {
+    constexpr int PAR = decltype(par)::value;
+    // ---- codes of group g (issued two steps ago) leave their landing registers ----
+    CT ccur[KE];
+#pragma unroll
+    for (int k = 0; k < KE; ++k) ccur[k] = cbuf[PAR][k];
+    // ---- C(g + 2): code bytes of the edges whose ids were issued two steps ago ----
+    {
+      uint32_t nid[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint64_t raw = (uint64_t)(int64_t)iraw[PAR][i];
+        uint32_t id = (raw >> 32) ? ((int64_t)raw < 0 ? 0u : n_last) : ((uint32_t)raw < n_last ? (uint32_t)raw : n_last);
+        nid[i] = (q * 4 + i) < degq[2] ? id : 0u;     // edges past the row's end read row 0 (a cached line)
+      }
+#pragma unroll
+      for (int k = 0; k < KE; ++k) {
+        uint32_t id;
+        switch (k >> 2) {
+          case 0: id = quad_bcast<0>(nid[k & 3]); break;
+          case 1: id = quad_bcast<1>(nid[k & 3]); break;
+          case 2: id = quad_bcast<2>(nid[k & 3]); break;
+          default: id = quad_bcast<3>(nid[k & 3]); break;
+        }
+        cbuf[PAR][k] = *reinterpret_cast<const CT*>(code_base + (uint64_t)id * (uint32_t)a.n_cb);
+      }
+    }
+    // ---- I(g + 4): the row's first KE source ids, four per lane ----
+    {
+      const int64_t row = group_row(g + 4);
+      int64_t b = (int64_t)praw0[PAR], e = (int64_t)praw1[PAR];
+      b = b < 0 ? 0 : (b > a.E ? a.E : b);
+      e = e < b ? b : (e > a.E ? a.E : e);
+      const int64_t d = e - b;
+      degq[4] = (g + 4 >= 0 && g + 4 < n_groups && row < row_end) ? (int)(d > 0x3fffffff ? 0x3fffffff : d) : 0;
+      if (q * 4 < KE) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          int64_t at = b + q * 4 + i;
+          at = at > e_last ? e_last : at;
+          iraw[PAR][i] = indices[at];
+        }
+      }
+    }
+    // ---- P(g + 6) ----
+    {
+      int64_t row = group_row(g + 6);
+      row = row < a.R ? row : a.R - 1;
+      praw0[PAR] = indptr[row];
+      praw1[PAR] = indptr[row + 1];
+    }
+    // ---- X(g) ----
+    if (g >= 0) {
+      float acc[8][4];
+      const int64_t row = row_begin + g * kSRows + rr;
+      const int deg = degq[0];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j][0] = acc[j][1] = acc[j][2] = acc[j][3] = 0.f;
+#pragma unroll
+      for (int k = 0; k < KE; ++k) {
+        if (__ballot(k < deg) == 0) break;
+        if (a.dense_store == 3 && k >= 1) break;   // experiment: stores only
+        if (k == 0) {
+          if (0 < deg) {   // the first edge lands in the accumulators as it is
+            f4v v[8];
+            edge_reads((uint32_t)ccur[0], v);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { acc[j][0] = v[j][0]; acc[j][1] = v[j][1]; acc[j][2] = v[j][2]; acc[j][3] = v[j][3]; }
+          }
+        } else if (k < deg) {
+          add_edge((uint32_t)ccur[k], acc);
+        }
+      }
+      if (__ballot(deg > KE) != 0) {
+        // the tail of long rows, in edge order, straight from HBM
+        int64_t b = 0;
+        if (deg > KE) {
+          b = (int64_t)indptr[row];
+          b = b < 0 ? 0 : (b > a.E ? a.E : b);
+        }
+        for (int k = KE; __ballot(k < deg) != 0; ++k) {
+          if (k < deg) {
+            const int64_t id = clamp_idx(indices[b + k], a.N);
+            const CT cw = *reinterpret_cast<const CT*>(code_base + (uint64_t)id * (uint32_t)a.n_cb);
+            add_edge((uint32_t)cw, acc);
+          }
+        }
+      }
+      if (deg > 1) {
+        const float d = (float)deg;
+        float r = __builtin_amdgcn_rcpf(d);
+        r = __fmaf_rn(__fmaf_rn(-d, r, 1.f), r, r);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int t = 0; t < 4; ++t) acc[j][t] = div_by(acc[j][t], d, r);
+      }
+      if (a.dense_store != 2) {
+        if (IL) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) direct_store(i, acc, g);
+        } else {
+#pragma unroll
+          for (int op = 0; op < 2 * (kSRows / kStgRows); ++op) store_op(op, acc, g);
+        }
+      }
+    }
+#pragma unroll
+    for (int d = 0; d < 4; ++d) degq[d] = degq[d + 1];
+  };
+
+  for (int64_t g = -6; g < n_groups; g += 2) {
+    step(std::integral_constant<int, 0>{}, g);
+    if (g + 1 < n_groups) step(std::integral_constant<int, 1>{}, g + 1);
+  }
+}
+
+template <int W, int KE, bool IL, int kSThreads, int kStgRows>
+int launch_strip(const VqArgs& a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
+                 const char* what, unsigned grid) {
+  const size_t lds = (size_t)a.K * 128 * 4 + (IL ? 0 : (size_t)(kSThreads / 64) * kStgRows * 512);
+  if (plan_only()) {
+    plan_record("vq_strip_kernel", grid, kSThreads, (int64_t)lds, kSRows, W, KE, IL ? 1 : 0, kStgRows);
+    return 0;
+  }
+  const void* kern = idx_dtype == F2CGT_DT_I32 ? reinterpret_cast<const void*>(vq_strip_kernel<W, KE, IL, kSThreads, kStgRows, int32_t>)
+                                               : reinterpret_cast<const void*>(vq_strip_kernel<W, KE, IL, kSThreads, kStgRows, int64_t>);
+  const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return fail((int)e, "%s: cannot reserve %zu B of LDS", what, lds);
+  if (idx_dtype == F2CGT_DT_I32)
+    vq_strip_kernel<W, KE, IL, kSThreads, kStgRows, int32_t><<<grid, kSThreads, lds, st>>>(a, static_cast<const int32_t*>(indptr),
+                                                                static_cast<const int32_t*>(indices), out);
+  else
+    vq_strip_kernel<W, KE, IL, kSThreads, kStgRows, int64_t><<<grid, kSThreads, lds, st>>>(a, static_cast<const int64_t*>(indptr),
+                                                                static_cast<const int64_t*>(indices), out);
+  return launch_status(what);
+}
+
+template <int W>
+int launch_strip_w(const VqArgs& a, int ke, const void* indptr, const void* indices, int idx_dtype, float* out,
+                   hipStream_t st, const char* what, unsigned grid) {
+  constexpr bool IL = W == 32;
+  const char* v = getenv("F2CGT_VQ_VAR");
+  const int var = v ? atoi(v) : 0;
+  if (IL) {
+    if (ke <= 12 && var == 1) return launch_strip<W, 12, IL, 768, 4>(a, indptr, indices, idx_dtype, out, st, what, grid);
+    if (ke <= 12) return launch_strip<W, 12, IL, 512, 4>(a, indptr, indices, idx_dtype, out, st, what, grid);
+    return launch_strip<W, 16, IL, 512, 4>(a, indptr, indices, idx_dtype, out, st, what, grid);
+  }
+  if (var == 1) return launch_strip<W, 16, IL, 512, 8>(a, indptr, indices, idx_dtype, out, st, what, grid);
+  return launch_strip<W, 16, IL, 512, 4>(a, indptr, indices, idx_dtype, out, st, what, grid);
+}
+
+#endif  // F2CGT_EXPERIMENTS
 
 template <int BT, int H, int RPM>
 int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
@@ -595,6 +947,24 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
   // with few edges per row the output dominates and its store pattern decides (fanout 2 at the C3
   // shape: 845 -> 405 us); from about 8 edges per row the detour through LDS costs more than it saves
   a.dense_store = avg_deg <= 8.0;
+#ifdef F2CGT_EXPERIMENTS
+  {
+    const char* v = getenv("F2CGT_VQ_STRIP");
+    const int mode = v ? atoi(v) : 0;     // 0 off; tens: 0 plain, 1 non-temporal, 2 no stores; units: 2 = KE by degree, 6 = KE 16
+    if (mode == 20) a.dense_store = 2;
+    if (mode % 10 > 0 && avg_deg <= 24.0) {
+      VqArgs b = a;
+      b.dense_store = (mode / 10) % 10;
+      if (mode >= 100) b.N = 1;   // experiment: every source id reads row 0
+      const int ke = (mode % 10) == 6 ? 16 : (avg_deg <= 6.0 ? 8 : (avg_deg <= 10.0 ? 12 : 16));
+      switch (a.w) {
+        case 8: return launch_strip_w<8>(b, ke, indptr, indices, idx_dtype, out, st, what, grid);
+        case 16: return launch_strip_w<16>(b, ke, indptr, indices, idx_dtype, out, st, what, grid);
+        default: return launch_strip_w<32>(b, ke, indptr, indices, idx_dtype, out, st, what, grid);
+      }
+    }
+  }
+#endif
   if (a.feat_dim % 8 == 0) {
     if (avg_deg <= 15.0) return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
     if (avg_deg <= 30.0) return launch_wave<BT, 2, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
