@@ -28,16 +28,24 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F32_PEAK_TFLOPS = 157.3
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE, each scaled by
-# what the same counter reads for a plain copy of known size; see profiles/).  Keyed by
-# (workload name, index dtype).  Missing = not measured.
-MEASURED_TRAFFIC_BYTES = {
-    ("c1_sq8_affine", "int64"): 18292817,
-    ("c2_sq4_affine", "int64"): 134407238,
-    ("c3_vq_16x8", "int64"): 506000000,
-    ("c4_hybrid", "int64"): 1029876440,
-    ("c5_vq_24x32", "int64"): 2188900000,
-}
+
+
+def _measured_traffic(workload, idx):
+    """HBM bytes per launch from profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each
+    scaled by what the same counter reads for a plain copy of known size; written by
+    `python3 -m f2cgt_amd.profile_summary`).  A figure only counts for the kernel sources it was
+    measured on: None when the record is missing or the sources have changed since."""
+    try:
+        from f2cgt_amd import profile_summary
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as fh:
+            rec = json.load(fh)
+        sha = profile_summary.csrc_sha16()
+        for e in rec.get("entries", []):
+            if e.get("workload") == workload and e.get("idx") == idx and e.get("csrc_sha16") == sha:
+                return int(e["bytes"])
+    except (OSError, ValueError, KeyError):
+        pass
+    return None
 
 
 def _launcher(capi, wl, out):
@@ -115,6 +123,28 @@ def _others(idx):
         gbs = wl["algo_bytes"] / (ms_launch * 1e-3) / 1e9
         res[wl["name"]] = {"launch_us": ms_launch * 1e3, "edges_per_s": wl["E"] / (ms_step * 1e-3),
                            "algorithmic_GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS}
+        del wl
+        torch.cuda.empty_cache()
+    # the operator at the size of a sampled minibatch block: the first R destination rows of the same
+    # graphs (the reference's own test block is batch 1024 with fanout 15,
+    # tests/test_fusion_decompress_spmm.py:36-90; the first layer of a three-layer sampler sees ~5e4 rows)
+    for name in ("c2", "c3"):
+        wl = synth.WORKLOADS[name](device="cuda", idx_dtype=torch.int64)
+        row_bytes = wl["codes"].shape[1]
+        fixed = wl["codebooks"].numel() * 4 if "codebooks" in wl else 2 * wl["feat_dim"] * 4
+        for rows in (1024, 4096, 16384, 65536):
+            small = dict(wl)
+            small["indptr"] = wl["indptr"][:rows + 1].contiguous()
+            small["E"] = int(small["indptr"][-1])
+            small["indices"] = wl["indices"][:small["E"]].contiguous()
+            small["R"] = rows
+            nbytes = small["E"] * (row_bytes + 8) + (rows + 1) * 8 + rows * wl["feat_dim"] * 4 + fixed
+            out = torch.empty((rows, wl["feat_dim"]), dtype=torch.float32, device="cuda")
+            _, ms_launch = _time_steps(_launcher(capi, small, out), 1000, 200)
+            res["%s_first_%d_rows" % (wl["name"], rows)] = {
+                "launch_us": ms_launch * 1e3, "edges": small["E"], "algorithmic_GBps": nbytes / (ms_launch * 1e-3) / 1e9,
+                "frac_hbm_peak": nbytes / (ms_launch * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            del small, out
         del wl
         torch.cuda.empty_cache()
     # source ids passed through a fixed bijection (hot rows no longer contiguous), and int32 indices
@@ -286,7 +316,7 @@ def main():
 
     wl, ms_per_step, launch_ms = _run_workload(args.workload, args.idx, args.steps, args.warmup)
     achieved = wl["algo_bytes"] / (launch_ms * 1e-3) / 1e9
-    traffic = MEASURED_TRAFFIC_BYTES.get((wl["name"], args.idx))
+    traffic = _measured_traffic(wl["name"], args.idx)
     result = {
         "metric": "edges aggregated/sec, fused decompress-SpMM",
         "value": wl["E"] / (ms_per_step * 1e-3),

@@ -160,6 +160,41 @@ __device__ __forceinline__ void stage_codebook_tile(float* __restrict__ s_cb, co
   }
 }
 
+// The same staging in two halves for a kernel that has other loads to issue while the tile is on
+// its way: stage_codebook_load fills v[8] (K <= 256: one pass of eight float4 per thread of a
+// 1024-thread workgroup), stage_codebook_store writes them to LDS.  Needs the float4 conditions of
+// stage_codebook_tile (stage_codebook_vec_ok).
+__device__ __forceinline__ bool stage_codebook_vec_ok(const float* codebooks, int w, int tile_cols) {
+  return (reinterpret_cast<uintptr_t>(codebooks) & 15) == 0 && (tile_cols & 3) == 0 && (w & 3) == 0;
+}
+template <int THREADS>
+__device__ __forceinline__ void stage_codebook_load(float4 (&v)[8], const float* __restrict__ codebooks, int K, int w,
+                                                    int tile, int tile_cols) {
+  const int n4 = K * 32;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int i = threadIdx.x + u * THREADS;
+    const int code = i >> 5, c = (i & 31) * 4;
+    const bool on = i < n4 && c < tile_cols;
+    const int col = tile * 128 + c;
+    const int sub = col / w;
+    const int64_t at = on ? ((int64_t)sub * K + code) * w + (col - sub * w) : 0;
+    v[u] = *reinterpret_cast<const float4*>(codebooks + at);
+    if (!on) v[u] = float4{0.f, 0.f, 0.f, 0.f};
+  }
+}
+template <int THREADS, bool PAIR>
+__device__ __forceinline__ void stage_codebook_store(float* __restrict__ s_cb, const float4 (&v)[8], int K) {
+  const int n4 = K * 32;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int i = threadIdx.x + u * THREADS;
+    const int code = i >> 5, c = (i & 31) * 4;
+    const int pos = PAIR ? ((c >> 2) & 1) * 64 + (c >> 3) * 4 : c;
+    if (i < n4) *reinterpret_cast<float4*>(s_cb + (code << 7) + pos) = v[u];
+  }
+}
+
 // Correctly rounded fp32 exp2 / log2: the fp64 library result rounded once.
 __device__ __forceinline__ float exp2_cr(float x) { return (float)exp2((double)x); }
 __device__ __forceinline__ float log2_cr(float x) { return (float)log2((double)x); }

@@ -14,6 +14,8 @@
 #include "common.hpp"
 #include "spmm_fast.hpp"
 
+#include <cstdlib>
+
 #include <type_traits>
 
 namespace f2cgt {
@@ -649,7 +651,11 @@ extern "C" int f2cgt_vq_decompress_spmm_csr(const void* codes, int code_dtype, c
   F2CGT_REQUIRE(codebooks && (num_edges == 0 || codes), F2CGT_E_INVALID, "%s: null buffer", what);
   hipStream_t st = as_stream(stream);
   const int D = (int)feat_dim, n_cb = (int)num_codebooks, k = (int)K, w = (int)width;
-  if (code_dtype == F2CGT_DT_U8 &&
+  bool fast_ok = code_dtype == F2CGT_DT_U8;
+#ifdef F2CGT_EXPERIMENTS
+  if (const char* v = getenv("F2CGT_VQ_GENERIC")) fast_ok = fast_ok && v[0] != '1';   // per-row skeleton for every shape
+#endif
+  if (fast_ok &&
       vq_pipe_eligible(codes, codebooks, out, num_rows, num_edges, num_src_rows, D, n_cb, k, w))
     return vq_pipe_run(static_cast<const uint8_t*>(codes), codebooks, indptr, indices, idx_dtype, out, num_rows,
                        num_edges, num_src_rows, D, n_cb, k, w, st, what);

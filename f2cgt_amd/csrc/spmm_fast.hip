@@ -25,6 +25,20 @@ constexpr int kBlock = 256;
 constexpr int kStageBytes = 18 * 1024;  // LDS staging per workgroup -> 7-8 workgroups per CU
 constexpr int kGatherUnroll = 8;
 
+// Rows per block for small launches.  A block is a chain of dependent round trips, so the launch
+// time is set by how many of them a CU overlaps: below `target` workgroups the blocks are shrunk to
+// (at least) `floor` rows so that the grid does not fall short of a few workgroups per CU.
+// Integer-accumulating kernel (128 threads, target 2048), power-law block, 400-byte output rows:
+// 16384 rows 7.3 us with 56 rows per block, 5.5 us with 8; 65536 rows 10.4 / 9.5 us with 56 / 32;
+// from 2.5e5 rows on the degree-based size is best.  Staged-rows kernel (256 threads, target
+// 1024, at least 16 rows): 16384 rows 10.7 / 7.8 / 9.7 us with 8 / 16 / 64 rows per block.
+inline int shrink_rows_per_block(int rb, int64_t R, int floor, int step, int target) {
+  const int64_t want = R / target;
+  int cap = (int)(want > rb ? rb : want) / step * step;
+  cap = cap < floor ? floor : cap;
+  return rb < cap ? rb : cap;
+}
+
 template <int LB> struct word_of;
 template <> struct word_of<1> { using type = uint8_t; };
 template <> struct word_of<2> { using type = uint16_t; };
@@ -776,6 +790,14 @@ int launch_acc(AccArgs a, const void* indptr, const void* indices, int idx_dtype
   while (sub > 8 && sub * acc_row > 24 * 1024) sub -= 8;
   int rb = sub * (int)(0.6 * a.edge_batch / (dg * sub));
   rb = rb < sub ? sub : (rb > 256 ? 256 / sub * sub : rb);
+  {
+    const int small = shrink_rows_per_block(rb, a.R, 8, 8, 2048);
+    if (small < rb) {
+      rb = small;
+      sub = sub > rb ? rb : sub;
+      rb = rb / sub * sub;
+    }
+  }
 #ifdef F2CGT_EXPERIMENTS
   if (const char* v = getenv("F2CGT_ACC_RB")) {   // rows per block, a multiple of 8
     const int want = atoi(v);
@@ -1034,6 +1056,13 @@ int launch_sq_rows(RowsArgs a, const void* indptr, const void* indices, int idx_
   const double dg = avg_deg > 0.5 ? avg_deg : 0.5;
   int rb = ((int)(0.6 * a.edge_cap / dg) + 4) / 8 * 8;
   rb = rb < 8 ? 8 : (rb > 64 ? 64 : rb);
+  rb = shrink_rows_per_block(rb, a.R, 16, 8, 1024);
+#ifdef F2CGT_EXPERIMENTS
+  if (const char* v = getenv("F2CGT_ROWS_RB")) {
+    const int want = atoi(v);
+    if (want >= 8 && want <= 64) rb = want / 8 * 8;
+  }
+#endif
   a.rows_per_block = rb;
   const size_t lds = lut_bytes + (size_t)(rb + 4) * 4 + 64 + (size_t)rb * 4 + (size_t)a.edge_cap * 4 +
                      (size_t)a.edge_cap * a.pitch + 16;
@@ -1399,6 +1428,12 @@ int launch_hybrid(HybArgs a, const void* indptr, const void* indices, int idx_dt
   while (rb * 2 <= want && rb < 64) rb *= 2;
   const size_t acc_row = (size_t)(2 * a.chunks + 8) * 4;
   while (rb > 8 && rb * acc_row > 16 * 1024) rb /= 2;
+#ifdef F2CGT_EXPERIMENTS
+  if (const char* v = getenv("F2CGT_HYB_RB")) {
+    const int want = atoi(v);
+    if (want == 8 || want == 16 || want == 32 || want == 64) rb = want;
+  }
+#endif
   a.rows_per_block = rb;
   const size_t lds = rb * acc_row + (size_t)a.chunks * 32 + (size_t)(rb + 4) * 4 + (size_t)rb * 4 +
                      (size_t)a.edge_batch * 6 + 16;

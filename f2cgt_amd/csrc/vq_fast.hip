@@ -294,6 +294,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   using CW = typename code_word<BT>::type;
   constexpr int kWaves = kThreads / 64;
   constexpr int kMini = kWChunk / RPM;          // mini-blocks (RPM rows each) per chunk
+  const bool K_FITS_ONE_PASS = a.K * 32 <= 8 * kThreads;
   extern __shared__ __align__(16) unsigned char smem[];
   float* s_cb = reinterpret_cast<float*>(smem);
   const int wave = uni((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
@@ -312,8 +313,6 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     stripe = blockIdx.x / a.n_tiles;
   }
   const int tile_cols = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
-  stage_codebook_tile<kThreads, H == 2>(s_cb, a.codebooks, a.K, a.w, tile, tile_cols);
-  __syncthreads();
 
   // A wave owns one contiguous range of rows (a multiple of 4, the same for every wave, so the
   // work is balanced to one mini-block); chunk c of the wave covers rows [chunk_row0 + 48 c, +48).
@@ -321,7 +320,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   const int64_t rows_per_wave = ((a.R + total_waves - 1) / total_waves + kWRows - 1) / kWRows * kWRows;
   const int64_t chunk_stride = kWChunk;
   const int64_t chunk_row0 = ((int64_t)stripe * kWaves + wave) * rows_per_wave;
-  if (chunk_row0 >= a.R) return;
+  const bool has_rows = chunk_row0 < a.R;
   const int64_t row_end = chunk_row0 + rows_per_wave < a.R ? chunk_row0 + rows_per_wave : a.R;
   const int64_t n_chunks = (row_end - chunk_row0 + kWChunk - 1) / kWChunk;
   const int64_t n_mini = (row_end - chunk_row0 + RPM - 1) / RPM;
@@ -373,13 +372,40 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     return (int64_t)(((uint64_t)hi << 32) | lo);
   };
 
-  issue_P(0);
-  park_P(0);
+  // The codebook tile and the wave's first row offsets travel together, and the source ids of the
+  // first mini-block are on their way while the tile is written to LDS: a launch over few rows is
+  // mostly this start-up (128 KB per CU, then three dependent round trips before the first sum).
   int eb0 = 0, ne0 = 0;      // mini-block g
   int eb1 = 0, ne1 = 0;      // g + 1
   int64_t Ireg = 0;
+  int64_t g_first = -2;
+  if (K_FITS_ONE_PASS && stage_codebook_vec_ok(a.codebooks, a.w, tile_cols)) {
+    float4 cbv[8];
+    stage_codebook_load<kThreads>(cbv, a.codebooks, a.K, a.w, tile, tile_cols);
+    if (has_rows) {
+      issue_P(0);
+      park_P(0);
+      if (n_mini > 0) {
+        bounds(0, eb1, ne1);
+        const int64_t e0 = chunk_e0(0);
+        const bool on = ne1 <= kWEdges && lane < ne1;
+        const Idx* src = on ? indices + e0 + eb1 + lane : indptr;
+        Ireg = (int64_t)*src;
+        g_first = -1;
+      }
+    }
+    stage_codebook_store<kThreads, H == 2>(s_cb, cbv, a.K);
+    __syncthreads();
+    if (!has_rows) return;
+  } else {
+    stage_codebook_tile<kThreads, H == 2>(s_cb, a.codebooks, a.K, a.w, tile, tile_cols);
+    __syncthreads();
+    if (!has_rows) return;
+    issue_P(0);
+    park_P(0);
+  }
   CW Creg = {};
-  for (int64_t g = -2; g < n_mini; ++g) {
+  for (int64_t g = g_first; g < n_mini; ++g) {
     // chunk-level P stage, driven by the position of g inside its chunk
     if (g >= 0) {
       const int64_t c = g / kMini;

@@ -110,3 +110,23 @@ def test_unsigned_eight_bit_log_codes_are_refused():
     rc, plan = capi.dry_run("f2cgt_sq_decompress_spmm_csr", A16, capi.DT_I8, A16, A16, A16, capi.DT_I64, A16, 4, 8,
                             10, 16, 16, 1, 8, 16, None)
     assert rc == 0 and plan is not None
+
+
+def test_rows_per_block_follow_the_launch_size():
+    # integer-accumulating kernel: the degree decides from 2.5e5 rows on, smaller launches get smaller
+    # blocks (at least 8 rows) so that a CU still overlaps several of them
+    want = {(250_000, 2): 64, (65_536, 2): 32, (16_384, 2): 8, (1024, 2): 8, (10_000, 10): 8}
+    for (rows, fanout), rb in want.items():
+        bits, d = (8, 128) if fanout == 10 else (4, 100)
+        rc, plan = plan_affine(bits, d, rows=rows, fanout=fanout)
+        assert rc == 0 and plan.kernel.decode() == "sq_affine_acc_kernel"
+        assert plan.rows_per_block == rb, (rows, fanout, plan.rows_per_block)
+        assert plan.rows_per_block % plan.aux[2] == 0 and plan.grid == -(-rows // rb)
+    # staged-rows kernel: at least 16 rows, about a thousand workgroups
+    for rows, rb in ((250_000, 64), (65_536, 64), (16_384, 16), (4096, 16), (20_000, 16)):
+        rc, plan = plan_log_sq(4, 100, rows=rows, fanout=2)
+        assert rc == 0 and plan.kernel.decode() == "sq_rows_kernel"
+        assert plan.rows_per_block == rb, (rows, plan.rows_per_block)
+    # long rows keep their small degree-based blocks
+    rc, plan = plan_log_sq(4, 100, rows=4096, fanout=60)
+    assert rc == 0 and plan.rows_per_block == 8

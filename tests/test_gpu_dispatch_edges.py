@@ -69,3 +69,35 @@ def test_fused_log_sq_with_either_workgroup_size(bits, feat_dim):
         got = capi.sq_decompress_spmm_csr(dev(stored), dev(cb), dev(indptr), dev(indices), bits, column_slice, feat_dim)
         torch.cuda.synchronize()
         assert np.allclose(got.cpu().numpy(), want, rtol=RTOL, atol=RTOL * 3.0)
+
+
+@pytest.mark.parametrize("rows", [16383, 16384, 32767, 32768, 65535, 65536, 114687, 114688])
+def test_fused_sq_on_both_sides_of_the_rows_per_block_steps(rows):
+    # launches below ~2000 workgroups shrink their row blocks in steps of 8 rows: the integer-accumulating
+    # kernel (affine, 128 threads) and the staged-rows kernel (log domain, 256 threads) at every step
+    print("case rows-per-block steps rows=%d" % rows, flush=True)
+    rng = np.random.default_rng(rows)
+    n, d = 3000, 100
+    deg = rng.integers(0, 5, size=rows)
+    indptr = np.zeros(rows + 1, dtype=np.int64)
+    indptr[1:] = np.cumsum(deg)
+    indices = rng.integers(0, n, size=int(indptr[-1]))
+    raw = rng.integers(0, 16, size=(n, d), dtype=np.uint8)
+    packed = oc.packbits(raw, 4)
+    params = np.stack([rng.standard_normal(d), 0.01 + rng.random(d)]).astype(np.float32)
+    got = capi.sq_affine_decompress_spmm_csr(dev(packed), dev(params), dev(indptr), dev(indices), 4, d)
+    torch.cuda.synchronize()
+    # the decode is affine in the code: the mean of the codes, then one scale and shift per output
+    dec = oc.sq_affine_decompress(packed, params, 4, d)
+    sums = np.zeros((rows, d), dtype=np.float64)
+    np.add.at(sums, np.repeat(np.arange(rows), deg), dec[indices].astype(np.float64))
+    want = (sums / np.maximum(deg, 1)[:, None]).astype(np.float32)
+    assert np.allclose(got.cpu().numpy(), want, rtol=RTOL, atol=RTOL * np.abs(dec).max())
+    cb = np.array([[0.01, 3.0, -6.643856, 1.5849625, 0.4]], dtype=np.float32)
+    got = capi.sq_decompress_spmm_csr(dev(packed), dev(cb), dev(indptr), dev(indices), 4, d, d)
+    torch.cuda.synchronize()
+    dec = oc.sq_decompress(packed, cb, 4, d, d)
+    sums[:] = 0
+    np.add.at(sums, np.repeat(np.arange(rows), deg), dec[indices].astype(np.float64))
+    want = (sums / np.maximum(deg, 1)[:, None]).astype(np.float32)
+    assert np.allclose(got.cpu().numpy(), want, rtol=RTOL, atol=RTOL * np.abs(dec).max())

@@ -72,8 +72,6 @@ def _oracle_rows(wl, rows):
 @pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
 @pytest.mark.parametrize("idx", [torch.int64, torch.int32])
 def test_full_size_workload(name, idx):
-    if name in ("c4", "c5") and idx == torch.int32:
-        pytest.skip("int32 indices are exercised at full size on c1-c3")
     wl = synth.WORKLOADS[name](device="cuda", idx_dtype=idx)
     R, D = wl["R"], wl["feat_dim"]
     out = _fused(wl)
