@@ -21,7 +21,7 @@ OBJ = os.path.join(PKG, "build")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 HIP_SOURCES = ["runtime.hip", "packbits.hip", "sq.hip", "vq.hip", "spmm.hip", "spmm_fast.hip",
-               "vq_fast.hip", "encode.hip", "fetch.hip"]
+               "vq_fast.hip", "encode.hip", "fetch.hip", "kmeans.hip"]
 HIP_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -39,6 +39,8 @@ SIGNATURES = {
     "f2cgt_fetch_rows": ([P, P, P, P, I, P, L, L, L, L, P], c_int),
     "f2cgt_pairwise_distance": ([P, P, P, L, L, L, I, P], c_int),
     "f2cgt_kmeans_predict": ([P, P, P, P, L, L, L, I, P], c_int),
+    "f2cgt_kmeans_update_workspace_bytes": ([L, L], c_int64),
+    "f2cgt_kmeans_update": ([P, P, P, P, P, P, I, ctypes.c_float, P, L, L, L, L, P], c_int),
 }
 
 
@@ -263,3 +265,19 @@ def kmeans_predict(x, centers, metric, u8=False, out=None):
                                       METRIC_COSINE if metric == "cosine" else METRIC_L2, _stream()),
            "kmeans_predict")
     return out
+
+
+def kmeans_update(x, labels, centers, stop=None, rule=0, tol=0.0, workspace=None, shift=None):
+    """One centre update in place (f2cgt_kmeans_update); -> shift tensor [2] = (sum |dc|, sum |dc|^2)."""
+    import torch
+    n, k = centers.shape
+    need = lib().f2cgt_kmeans_update_workspace_bytes(n, k)
+    if workspace is None:
+        workspace = torch.empty((need,), dtype=torch.uint8, device=x.device)
+    if shift is None:
+        shift = torch.empty((2,), dtype=torch.float32, device=x.device)
+    u8 = labels.dtype == torch.uint8
+    _check(lib().f2cgt_kmeans_update(_ptr(x), None if u8 else _ptr(labels), _ptr(labels) if u8 else None,
+                                     _ptr(centers), _ptr(shift), _ptr(stop), rule, tol, _ptr(workspace),
+                                     workspace.numel(), x.shape[0], n, k, _stream()), "kmeans_update")
+    return shift

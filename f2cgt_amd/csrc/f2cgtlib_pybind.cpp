@@ -283,16 +283,55 @@ torch::Tensor pairwise_distance(torch::Tensor x, torch::Tensor y, std::string me
   return dist;
 }
 
+// Extension: one Lloyd centre update in place (the update half of examples/my_kmeans.py:87-113).
+// -> shift fp32 [2] on the device = (sum_c |dc|, sum_c |dc|^2).  `stop` (int32 [1] on the device, optional)
+// freezes the centres once `rule` is met (1: sum |dc|^2 < tol; 2: (sum |dc|)^2 < tol), see include/f2cgt.h.
+torch::Tensor kmeans_update(torch::Tensor x, torch::Tensor labels, torch::Tensor centers,
+                            c10::optional<torch::Tensor> stop, int64_t rule, double tol) {
+  x = dev_contig(x, "data");
+  labels = dev_contig(labels, "labels");
+  TORCH_CHECK(centers.is_cuda() && centers.is_contiguous() && centers.scalar_type() == torch::kFloat32 &&
+                  centers.dim() == 2,
+              "centers must be a contiguous float32 GPU tensor [n, k] (it is updated in place)");
+  TORCH_CHECK(x.dim() == 2 && x.scalar_type() == torch::kFloat32 && x.size(1) == centers.size(1),
+              "data must be float32 [m, k]");
+  TORCH_CHECK(labels.dim() == 1 && labels.size(0) == x.size(0) &&
+                  (labels.scalar_type() == torch::kInt64 || labels.scalar_type() == torch::kUInt8),
+              "labels must be int64 or uint8 [m]");
+  int32_t* stop_ptr = nullptr;
+  if (stop.has_value()) {
+    TORCH_CHECK(stop->is_cuda() && stop->scalar_type() == torch::kInt32 && stop->numel() == 1,
+                "stop must be an int32 GPU tensor with one element");
+    stop_ptr = stop->data_ptr<int32_t>();
+  }
+  c10::DeviceGuard guard(x.device());
+  const int64_t n = centers.size(0), k = centers.size(1);
+  auto ws = torch::empty({f2cgt_kmeans_update_workspace_bytes(n, k)},
+                         torch::TensorOptions().dtype(torch::kUInt8).device(x.device()));
+  auto shift = empty_f32({2}, x);
+  const bool u8 = labels.scalar_type() == torch::kUInt8;
+  check_rc(f2cgt_kmeans_update(x.data_ptr<float>(), u8 ? nullptr : labels.data_ptr<int64_t>(),
+                               u8 ? static_cast<const uint8_t*>(labels.data_ptr()) : nullptr,
+                               centers.data_ptr<float>(), shift.data_ptr<float>(), stop_ptr, (int)rule, (float)tol,
+                               ws.data_ptr(), ws.numel(), x.size(0), n, k, current_stream()),
+           "kmeans_update");
+  return shift;
+}
+
 // Counterpart of the reference's raft-backed KMeans (src/kmeans.h:13-31, src/kmeans.cu).
-// predict() is the fused MFMA distance + arg-min kernel.  fit() is Lloyd's algorithm on
-// top of it with centres initialised from randomly chosen rows (raft's k-means++ and its
-// RNG stream are not reproduced; fit() is not a bit-parity target).
+// predict() is the fused MFMA distance + arg-min kernel.  fit() is Lloyd's algorithm on the device:
+// assignment (f2cgt_kmeans_predict) and centre update (f2cgt_kmeans_update) per iteration, stopped by
+// raft's rule (sum of squared centre shifts below tol) which the update kernel evaluates itself; the
+// host looks at the flag every eighth iteration only.  The centres start from distinct random rows
+// (raft: random rows for cosine, k-means++ for L2; its RNG stream is not reproduced, so fit() is not a
+// bit-parity target).  raft's batching and restart parameters have no counterpart here: a value other
+// than the default draws a warning instead of being dropped silently.
 class KMeans {
  public:
   KMeans(int64_t n_cluster, int64_t feat_dim, std::string metric, int max_iter, double tol, int n_init,
          double oversampling_factor, int batch_samples, int batch_centroids, bool inertia_check)
       : metric_(std::move(metric)), max_iter_(max_iter), tol_(tol), n_clusters_(n_cluster) {
-    (void)n_init; (void)oversampling_factor; (void)batch_samples; (void)batch_centroids; (void)inertia_check;
+    warn_ignored(n_init, oversampling_factor, batch_samples, batch_centroids, inertia_check);
     TORCH_CHECK(n_cluster > 0 && feat_dim > 0, "KMeans: n_cluster and feat_dim must be positive");
     centers_ = torch::zeros({n_cluster, feat_dim},
                             torch::TensorOptions().dtype(torch::kFloat32).device(torch::kCUDA));
@@ -300,12 +339,22 @@ class KMeans {
   KMeans(torch::Tensor centers, std::string metric, int max_iter, double tol, int n_init,
          double oversampling_factor, int batch_samples, int batch_centroids, bool inertia_check)
       : metric_(std::move(metric)), max_iter_(max_iter), tol_(tol) {
-    (void)n_init; (void)oversampling_factor; (void)batch_samples; (void)batch_centroids; (void)inertia_check;
+    warn_ignored(n_init, oversampling_factor, batch_samples, batch_centroids, inertia_check);
     TORCH_CHECK(centers.device().is_cuda(), "centers must be a CUDA tensor");
     TORCH_CHECK(centers.dim() == 2 && centers.scalar_type() == torch::kFloat32,
                 "centers must be float32 [n_cluster, feat_dim]");
     centers_ = centers.contiguous();
     n_clusters_ = centers.size(0);
+  }
+
+  static void warn_ignored(int n_init, double oversampling_factor, int batch_samples, int batch_centroids,
+                           bool inertia_check) {
+    auto warn = [](const char* text) { py::module_::import("warnings").attr("warn")(std::string(text)); };
+    if (n_init != 1) warn("KMeans: n_init is ignored (one run from one random start)");
+    if (oversampling_factor != 2.0) warn("KMeans: oversampling_factor is ignored (no k-means|| seeding)");
+    if (batch_samples != (1 << 15)) warn("KMeans: batch_samples is ignored (the kernels stream all rows)");
+    if (batch_centroids != 0) warn("KMeans: batch_centroids is ignored (all centres are scored together)");
+    if (inertia_check) warn("KMeans: inertia_check is ignored (the centre shift alone stops the fit)");
   }
 
   void fit(torch::Tensor x) {
@@ -317,18 +366,18 @@ class KMeans {
     auto pick = torch::randperm(x.size(0), torch::TensorOptions().dtype(torch::kInt64).device(x.device()))
                     .slice(0, 0, n_clusters_);
     centers_.copy_(x.index_select(0, pick));
-    auto ones = torch::ones({x.size(0)}, x.options());
+    auto stop = torch::zeros({1}, torch::TensorOptions().dtype(torch::kInt32).device(x.device()));
+    const bool small = n_clusters_ <= 256;
+    n_iter_ = 0;
     for (int it = 0; it < max_iter_; ++it) {
-      auto labels = kmeans_predict_impl(x, centers_, metric_, false);
-      auto sums = torch::zeros_like(centers_).index_add_(0, labels, x);
-      auto cnt = torch::zeros({n_clusters_}, x.options()).index_add_(0, labels, ones);
-      auto fresh = sums / cnt.clamp_min(1.0).unsqueeze(1);
-      auto next = torch::where(cnt.unsqueeze(1) > 0, fresh, centers_);
-      const double shift = (next - centers_).pow(2).sum().item<double>();
-      centers_.copy_(next);
-      if (shift < tol_) break;
+      auto labels = kmeans_predict_impl(x, centers_, metric_, small);
+      kmeans_update(x, labels, centers_, stop, /*rule=*/1, tol_);
+      ++n_iter_;
+      if ((it & 7) == 7 && stop.item<int>() != 0) break;   // later steps are no-ops once the flag is up
     }
   }
+
+  int64_t n_iter() const { return n_iter_; }
 
   torch::Tensor predict(torch::Tensor x, bool normalize_weights) {
     (void)normalize_weights;  // sample weights only scale raft's inertia, never the labels
@@ -343,6 +392,7 @@ class KMeans {
   int max_iter_;
   double tol_;
   int64_t n_clusters_;
+  int64_t n_iter_ = 0;
   torch::Tensor centers_;
 };
 
@@ -500,7 +550,9 @@ PYBIND11_MODULE(F2CGTLib, m) {
       .def("kmeans_predict", &kmeans_predict, py::arg("x"), py::arg("centers"), py::arg("metric"))
       .def("vq_encode", &vq_encode, py::arg("x"), py::arg("centers"), py::arg("metric"))
       .def("fetch_rows", &fetch_rows, py::arg("table"), py::arg("index"), py::arg("hot") = py::none(),
-           py::arg("slot_map") = py::none());
+           py::arg("slot_map") = py::none())
+      .def("kmeans_update", &kmeans_update, py::arg("data"), py::arg("labels"), py::arg("centers"),
+           py::arg("stop") = py::none(), py::arg("rule") = 0, py::arg("tol") = 0.0);
   py::class_<KMeans>(m, "KMeans")
       .def(py::init<int64_t, int64_t, std::string, int, double, int, double, int, int, bool>(),
            py::arg("n_cluster"), py::arg("feat_dim"), py::arg("metric"), py::arg("max_iter") = 300,
@@ -514,5 +566,6 @@ PYBIND11_MODULE(F2CGTLib, m) {
            py::arg("inertia_check") = false)
       .def("fit", &KMeans::fit, py::arg("data"))
       .def("predict", &KMeans::predict, py::arg("data"), py::arg("normalize_weights") = true)
-      .def("get_centers", &KMeans::get_centers);
+      .def("get_centers", &KMeans::get_centers)
+      .def_property_readonly("n_iter", &KMeans::n_iter);   // extension: update steps issued by the last fit()
 }

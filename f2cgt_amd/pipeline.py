@@ -30,9 +30,10 @@ def _capi():
 
 # ---- encode pipeline -----------------------------------------------------------------------------
 def normalize(data):
-    """examples/process_compress.py:16-18."""
-    data_norm = data.norm(dim=1, p=2)
-    return data / data_norm.reshape(-1, 1) * data_norm.mean()
+    """Every row rescaled to the mean row norm: directions kept, lengths equalised
+    (examples/process_compress.py:16-18; same operation order, divide then multiply)."""
+    lengths = torch.linalg.vector_norm(data, ord=2, dim=1, keepdim=True)
+    return (data / lengths) * lengths.mean()
 
 
 def sampling(sample_size, num_items, hotness=None, generator=None):
@@ -50,18 +51,16 @@ def sq_metadata(sample):
     """(fmin, fmax, emin, emax, mean) of one column slice from a sample of its rows:
     float64 percentiles of |x| floored at 1e-5 / 2e-5, log2 in float64, mean lifted by 0.1 when
     below 0.1 (examples/process_compress.py:45-68)."""
-    epsilon = 1e-5
-    sample = sample.float().abs().cpu()
-    fmin = max(np.percentile(sample.numpy(), 0.5), epsilon)
-    fmax = max(np.percentile(sample.numpy(), 99.5), 2 * epsilon)
-    fmin = torch.tensor(fmin)
-    fmax = torch.tensor(fmax)
-    emin = torch.log2(fmin)
-    emax = torch.log2(fmax).add(epsilon)
-    mean = sample.mean()
-    if mean < 0.1:
-        mean += 0.1
-    return fmin, fmax, emin, emax, mean
+    floor = 1e-5
+    magnitude = sample.float().abs().cpu()
+    # one percentile and one log2 at a time, as the reference does: numpy returns the sample's own
+    # precision for a scalar quantile (float64 for a list of them), and torch's scalar and vector
+    # log2 do not agree to the last bit
+    lo, hi = np.percentile(magnitude.numpy(), 0.5), np.percentile(magnitude.numpy(), 99.5)
+    fmin, fmax = torch.tensor(max(lo, floor)), torch.tensor(max(hi, 2 * floor))
+    level = magnitude.mean()
+    level = level + 0.1 if level < 0.1 else level
+    return fmin, fmax, torch.log2(fmin), torch.log2(fmax) + floor, level
 
 
 def sq_compress(features, target_bits, column_slice, hotness=None, sample_index=None, batch_rows=1_000_000):
@@ -95,7 +94,72 @@ def sq_compress(features, target_bits, column_slice, hotness=None, sample_index=
     return out, codebooks
 
 
-def vq_metadata(features, n_clusters, column_slice, hotness=None, sample_index=None, max_iter=30):
+class KMeansTrainer:
+    """Codebook trainer of the offline compressor (examples/my_kmeans.py:73-113, 150-184), on the
+    device from start to finish: assignment by `kmeans_predict`, centre update and stopping rule by
+    `kmeans_update`.
+
+    As in the reference: `cosine` starts from random unit-circle pairs (cos / sin of uniform angles,
+    :9-24), `euclidean` from distinct random non-zero rows (:27-31); a centre is the plain mean of its
+    members whatever the metric and keeps its value when it has none (:128-147); the fit ends when
+    (sum_c |centre shift|)^2 < tol, with tol growing by a factor 1.2 per iteration (:100-111).
+    The rule is evaluated by the update kernel, which freezes the centres when it holds; the host
+    reads the flag every `check_every` iterations, so the loop runs without a read-back per step.
+    """
+
+    def __init__(self, num_clusters, metric="cosine", tol=1e-4, mode="fast", max_iter=1000, check_every=8,
+                 generator=None):
+        if metric not in ("cosine", "euclidean"):
+            raise ValueError("metric must be 'cosine' or 'euclidean'")
+        if mode not in ("fast", "normal"):
+            raise ValueError("mode must be 'fast' or 'normal'")
+        self.num_clusters, self.metric, self.tol, self.mode = num_clusters, metric, tol, mode
+        self.max_iter, self.check_every, self.generator = max_iter, check_every, generator
+        self.centers, self.n_iter = None, 0
+
+    def _initial_centers(self, data):
+        n, width = self.num_clusters, data.shape[1]
+        if self.metric == "cosine":
+            half = width // 2
+            if width % 2 == 0:
+                angles = torch.rand((n, half), generator=self.generator) * (2 * math.pi)
+                start = torch.cat([torch.cos(angles), torch.sin(angles)], dim=1)
+            else:
+                radii = torch.rand((n, 1), generator=self.generator)
+                angles = torch.rand((n, half + 1), generator=self.generator) * (2 * math.pi)
+                start = radii * torch.cat([torch.cos(angles[:, :half]), torch.sin(angles)], dim=1)
+            return start.float().cuda()
+        alive = torch.nonzero(torch.count_nonzero(data, dim=1)).flatten()
+        if alive.numel() < n:
+            raise ValueError("fewer non-zero rows than clusters")
+        pick = torch.randperm(alive.numel(), generator=self.generator)[:n].to(alive.device)
+        return data[alive[pick]].float().cuda()
+
+    def fit(self, data):
+        capi = _capi()
+        data = data.float().cuda().contiguous()
+        centers = self._initial_centers(data).contiguous()
+        metric = "cosine" if self.metric == "cosine" else "l2"
+        stop = torch.zeros((1,), dtype=torch.int32, device="cuda")
+        tol, self.n_iter = float(self.tol), 0
+        for it in range(self.max_iter):
+            labels = capi.kmeans_predict(data, centers, metric)
+            capi.kmeans_update(data, labels, centers, stop, 2, tol)
+            tol *= 1.2
+            self.n_iter += 1
+            if it % self.check_every == self.check_every - 1 and int(stop.item()):
+                break
+        self.centers = centers
+
+    def get_centers(self):
+        return self.centers
+
+    def predict(self, data, normalize_weights=False):
+        metric = "cosine" if self.metric == "cosine" else "l2"
+        return _capi().kmeans_predict(data.float().cuda().contiguous(), self.centers, metric)
+
+
+def vq_metadata(features, n_clusters, column_slice, hotness=None, sample_index=None, max_iter=1000):
     """Codebooks fp32 [ceil(D / column_slice), n_clusters, column_slice]: per slice, rows of a
     sample inside the rim quantile are dropped, k-means (cosine, tol 5e-2) runs on the rest and the
     centres are rescaled to their mean norm (examples/process_compress.py:147-182)."""
@@ -111,7 +175,7 @@ def vq_metadata(features, n_clusters, column_slice, hotness=None, sample_index=N
         distance = data.norm(dim=1, p=2)
         rim = torch.quantile(distance, min(1.0, 0.00625 * (data.shape[1] / 8)))
         data = data[torch.ge(distance, rim)].contiguous()
-        km = capi.KMeans(n_clusters, hi - lo, "cosine", max_iter=max_iter, tol=5e-2)
+        km = KMeansTrainer(n_clusters, metric="cosine", tol=5e-2, max_iter=max_iter)
         km.fit(data)
         centers = normalize(km.get_centers())
         codebooks[i, :, :hi - lo] = centers
@@ -272,9 +336,12 @@ class TensorCache:
         self.slot_map = None
 
     def compute_weight_size(self, hotness):
-        full_size = self.data.numel() * self.data.element_size()
-        item_size = self.data.element_size() * self.data.shape[1] * torch.mean(hotness[hotness > 0]).item()
-        return full_size, item_size
+        """(bytes of the whole table, bytes of a row weighted by the mean hotness of the rows that are
+        ever touched): the two inputs of the reference's cache-split cost model
+        (examples/tensor_cache.py:102-106)."""
+        row_bytes = self.data.shape[1] * self.data.element_size()
+        touched = hotness[hotness > 0]
+        return self.data.shape[0] * row_bytes, row_bytes * float(touched.float().mean())
 
 
 class CompressionManager:
@@ -304,6 +371,11 @@ class CompressionManager:
         self.seeds_data = None
         self.is_two_level = len(self.methods) >= 2
         self.is_fusion = fusion
+        # the seed rows are fetched and decoded on a stream of their own while the caller goes on to
+        # sample and gather the block (examples/compress.py:36-53); default priority
+        self.seeds_task_stream = torch.cuda.Stream()
+        self.seeds_task_event = torch.cuda.Event()
+        self.check_seed_keys = True   # a host round trip per call; the reference's hash map query has no such check
         if self.is_two_level:
             self.seeds_data = TensorCache(place(compress_data["seeds_compression_data"]))
             keys = compress_data["seeds"].long().cuda()
@@ -319,12 +391,19 @@ class CompressionManager:
                                   self.feat_dim)
 
     def get_seeds_data(self, seeds_key):
+        """Decoded first-level rows of `seeds_key`, produced on `seeds_task_stream`; the result may be
+        used on another stream only after `seeds_task_event` (reorganize_seeds_data waits for it)."""
         if not self.is_two_level:
             return None
-        slots = self.seed_slot[seeds_key.long()].long()
-        if bool((slots < 0).any()):
-            raise KeyError("a requested id is not a seed row")
-        return self._decompress(0, self.seeds_data[slots])
+        side = self.seeds_task_stream
+        side.wait_stream(torch.cuda.current_stream())      # seeds_key may still be in the making
+        with torch.cuda.stream(side):
+            slots = self.seed_slot[seeds_key.long()].long()
+            if self.check_seed_keys and bool((slots < 0).any()):
+                raise KeyError("a requested id is not a seed row")
+            seeds_feature = self._decompress(0, self.seeds_data[slots])
+            self.seeds_task_event.record(side)
+        return seeds_feature
 
     def get_all_data(self, keys):
         data = self.data[keys]
@@ -350,6 +429,11 @@ class CompressionManager:
                                            self.configs[level][1], self.configs[level][0], self.feat_dim)
 
     def reorganize_seeds_data(self, seeds_feature, all_feature, num_dst):
+        if seeds_feature is not None:
+            # the consumer joins the seed stream here (examples/compress.py:74-75)
+            current = torch.cuda.current_stream()
+            current.wait_event(self.seeds_task_event)
+            seeds_feature.record_stream(current)
         if not self.is_fusion:
             if seeds_feature is None:
                 return None
@@ -375,20 +459,19 @@ class MySAGEConv(nn.Module):
                  activation=None):
         super().__init__()
         if aggregator_type != "mean":
-            raise ValueError("For fusion SAGEConv, aggregator_type must be'mean'.")
-        self._in_src_feats, self._in_dst_feats = (in_feats, in_feats) if isinstance(in_feats, int) else in_feats
-        self._out_feats = out_feats
-        self.norm = norm
-        self.activation = activation
-        self.fc_neigh = nn.Linear(self._in_src_feats, out_feats, bias=False)
-        self.fc_self = nn.Linear(self._in_dst_feats, out_feats, bias=bias)
-        self.reset_parameters()
+            raise ValueError("the fused layer aggregates by mean only (got %r)" % (aggregator_type,))
+        src_width, dst_width = (in_feats, in_feats) if isinstance(in_feats, int) else tuple(in_feats)
         self.sm = compression_manager
+        self.activation, self.norm = activation, norm
+        # the reference's attribute names (examples/conv.py:29-31): checkpoints of either load into the other
+        self.fc_neigh = nn.Linear(src_width, out_feats, bias=False)
+        self.fc_self = nn.Linear(dst_width, out_feats, bias=bias)
+        self.reset_parameters()
 
     def reset_parameters(self):
-        gain = nn.init.calculate_gain("relu")
-        nn.init.xavier_uniform_(self.fc_self.weight, gain=gain)
-        nn.init.xavier_uniform_(self.fc_neigh.weight, gain=gain)
+        """Glorot-uniform weights scaled for a ReLU that follows (examples/conv.py:38-42)."""
+        for layer in (self.fc_self, self.fc_neigh):
+            nn.init.xavier_uniform_(layer.weight, gain=nn.init.calculate_gain("relu"))
 
     def forward(self, csc, feat):
         capi = _capi()

@@ -221,6 +221,23 @@ int f2cgt_kmeans_predict(const float* x, const float* centers, int64_t* labels_i
                          uint8_t* labels_u8, int64_t m, int64_t n, int64_t k, int metric,
                          void* stream);
 
+/* One Lloyd iteration's centre update, after f2cgt_kmeans_predict has produced the labels.
+ * Replaces the update half of the reference's two training loops: compute_new_centers and the
+ * centre-shift test of examples/my_kmeans.py:87-113,128-147 (plain mean whatever the metric, a centre
+ * without members keeps its value) and the loop inside raft::cluster::kmeans::fit, src/kmeans.cu:61-75.
+ * x fp32 [m,k]; labels int64 [m] or uint8 [m] (exactly one non-NULL; values clamped to [0,n));
+ * centers fp32 [n,k], updated in place; shift fp32 [2] (device) receives sum_c |dc| and sum_c |dc|^2.
+ * stop (device int32, may be NULL): when it is nonzero on entry the call does nothing, and the call
+ * sets it when stop_rule says the centres are final (1: sum_c |dc|^2 < tol, raft's rule; 2:
+ * (sum_c |dc|)^2 < tol, the rule of examples/my_kmeans.py:105; 0: never) -- a training loop can then
+ * run without reading anything back per iteration.  workspace: device scratch for the partial sums,
+ * at least f2cgt_kmeans_update_workspace_bytes(n, k) bytes, 16-byte aligned, contents irrelevant.
+ * The sums are fp32 atomic adds: their last bits depend on the order the hardware takes them in. */
+int64_t f2cgt_kmeans_update_workspace_bytes(int64_t n, int64_t k);
+int f2cgt_kmeans_update(const float* x, const int64_t* labels_i64, const uint8_t* labels_u8, float* centers,
+                        float* shift, int32_t* stop, int stop_rule, float tol, void* workspace,
+                        int64_t workspace_bytes, int64_t m, int64_t n, int64_t k, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

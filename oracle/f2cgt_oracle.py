@@ -27,6 +27,11 @@ What pins each function (tests/test_oracle_*.py):
   fetch_rows            torch.index_select on the full table; a cache of any subset of
                         rows must not change the result.
   sq_affine_*, hybrid   closed forms stated by the benchmark configuration.
+  kmeans_update         per-cluster means by boolean masks in fp64, a hand-computed case, and the
+                        invariants of a Lloyd step (inertia never rises, a fixed point stays put).
+  sq_lut(fma=True)      the same table with the product and sum of the exponent fused into one
+                        rounding (what a contracting compiler makes of the kernel text); the test
+                        counts the entries on which the two readings differ.
 
 PARITY UNPINNED (nothing in the reference or in this container fixes them):
   * last-ulp behaviour of CUDA `exp2f`/`log2f` inside the reference kernels.  This
@@ -35,7 +40,12 @@ PARITY UNPINNED (nothing in the reference or in this container fixes them):
   * raft 23.10's internal rounding and tie rule in `kmeans_predict` /
     `pairwise_distance` (third-party, not vendored).  This oracle follows the torch
     statement in examples/my_kmeans.py:43-55,116-125 (first minimum wins).
-  * `KMeans.fit` (raft k-means++/random initialisation and RNG stream).
+  * `KMeans.fit` (raft k-means++/random initialisation and RNG stream): only the update step and
+    the stopping rules are restated here.
+  * whether the reference's CUDA build contracts `fabs(value) * k + emin`
+    (src/sq_quantization.cu:146-151, src/fusion_spmm.cu:203-207) into one fused multiply-add:
+    nvcc does so by default, the torch statement of the same formula (tests/test_sq.py:96-106)
+    cannot.  `sq_lut` follows the torch statement; `sq_lut(..., fma=True)` gives the other reading.
 """
 from __future__ import annotations
 
@@ -154,8 +164,13 @@ def sq_codes_to_storage(codes_f32: np.ndarray, target_bits: int) -> np.ndarray:
     return codes_f32.astype(np.int16)
 
 
-def sq_lut(codebooks: np.ndarray, target_bits: int) -> np.ndarray:
+def sq_lut(codebooks: np.ndarray, target_bits: int, fma: bool = False) -> np.ndarray:
     """Decoded value of every raw code, per codebook: fp32 [n_cb, 2**bits].
+
+    fma=True: the exponent |v| * k + emin rounded once (the product of two fp32 values is exact in
+    fp64, the sum is formed there and rounded to fp32), which is what a compiler that contracts
+    the kernel's `fabs(value) * k + emin` (src/sq_quantization.cu:146-151) into a fused multiply-add
+    evaluates.  Not used by any parity check: it measures how far the two readings are apart.
 
     The index is the raw bit pattern as stored (unsigned for bits < 8, the
     two's-complement pattern of the signed code for 8/16 bits).  Formula:
@@ -178,7 +193,10 @@ def sq_lut(codebooks: np.ndarray, target_bits: int) -> np.ndarray:
     sign = np.where(v >= 0, F32(1), F32(-1))
     emin, emax = codebooks[:, 2:3], codebooks[:, 3:4]
     k = ((emax - emin) / drange).astype(F32)
-    t = (np.abs(v)[None, :] * k).astype(F32) + emin
+    if fma:
+        t = (np.abs(v)[None, :].astype(np.float64) * k.astype(np.float64) + emin.astype(np.float64)).astype(F32)
+    else:
+        t = (np.abs(v)[None, :] * k).astype(F32) + emin
     return (exp2_f32(t.astype(F32)) * sign[None, :]).astype(F32)
 
 
@@ -386,3 +404,33 @@ def kmeans_predict(x: np.ndarray, centers: np.ndarray, metric: str):
     gap = part[:, 1] - part[:, 0]
     scale = np.maximum(np.abs(part[:, 1]), 1e-30)
     return labels.astype(np.int64), (gap / scale) < 1e-6
+
+
+def kmeans_update(x: np.ndarray, labels: np.ndarray, centers: np.ndarray):
+    """One Lloyd centre update (examples/my_kmeans.py:128-147, compute_new_centers): a centre becomes
+    the plain mean of the rows assigned to it, whatever the metric; a centre without members keeps
+    its value.  -> (new centres fp32, sum_c |dc|, sum_c |dc|^2): the centre shift of :100-103 and its
+    squared form (the quantity raft's fit tests, src/kmeans.cu:61-75).  The sums run in fp64: the
+    GPU adds in fp32 in an order of its own, so the comparison carries a tolerance."""
+    x64 = x.astype(np.float64)
+    n, k = centers.shape
+    sums = np.zeros((n, k), dtype=np.float64)
+    np.add.at(sums, labels.astype(np.int64), x64)
+    counts = np.bincount(labels.astype(np.int64), minlength=n).astype(np.float64)
+    new = centers.astype(np.float64).copy()
+    has = counts > 0
+    new[has] = sums[has] / counts[has, None]
+    new = new.astype(F32)
+    d2 = ((new.astype(np.float64) - centers.astype(np.float64)) ** 2).sum(axis=1)
+    return new, float(np.sqrt(d2).sum()), float(d2.sum())
+
+
+def kmeans_stop(shift_abs: float, shift_sq: float, tol: float, rule: int) -> bool:
+    """Stopping rules: 1 = raft (sum of squared centre shifts below tol, src/kmeans.cu:61-75 via
+    KMeansParams.tol), 2 = the reference's own trainer ((sum of centre shifts)^2 < tol,
+    examples/my_kmeans.py:105), with its tol growing by 1.2 per iteration (:111) left to the caller."""
+    if rule == 1:
+        return shift_sq < tol
+    if rule == 2:
+        return shift_abs * shift_abs < tol
+    return False
