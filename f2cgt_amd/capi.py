@@ -41,6 +41,7 @@ SIGNATURES = {
     "f2cgt_kmeans_predict": ([P, P, P, P, L, L, L, I, P], c_int),
     "f2cgt_kmeans_update_workspace_bytes": ([L, L], c_int64),
     "f2cgt_kmeans_update": ([P, P, P, P, P, P, I, ctypes.c_float, P, L, L, L, L, P], c_int),
+    "f2cgt_kmeans_update_static": ([P, P, P, P, P, P, I, ctypes.c_float, L, L, L, P], c_int),
 }
 
 

@@ -8,7 +8,8 @@
 // raft's kmeans::fit (src/kmeans.cu:61-75) stops on the squared form of the same shift.
 //
 // The partial sums are scratch memory beyond inputs and outputs (n * k floats and n counters):
-// they live in a workspace the caller passes.
+// f2cgt_kmeans_update takes them from a workspace the caller passes, f2cgt_kmeans_update_static
+// from a device array of this file (for callers that cannot allocate).
 #include "common.hpp"
 
 namespace f2cgt {
@@ -16,6 +17,13 @@ namespace {
 
 constexpr int kKmThreads = 256;
 constexpr int kKmLdsFloats = 12 * 1024;   // per-workgroup partial sums kept in LDS up to this many entries
+
+// Scratch of the allocation-free entry point: 65536 sums and 4096 counters, 272 KB that every device
+// the library runs on holds until the process ends.  The name is a host-side stand-in, not a device
+// address: host code only ever uses the pointer hipGetSymbolAddress returns for the current device.
+constexpr int64_t kStaticSums = 65536;
+constexpr int64_t kStaticCenters = 4096;
+static __device__ __align__(256) unsigned char scratch[(kStaticSums + kStaticCenters) * 4];
 
 struct KmArgs {
   const float* x;
@@ -192,3 +200,32 @@ extern "C" int f2cgt_kmeans_update(const float* x, const int64_t* labels_i64, co
   return km_run(what, a, as_stream(stream));
 }
 
+extern "C" int f2cgt_kmeans_update_static(const float* x, const int64_t* labels_i64, const uint8_t* labels_u8,
+                                          float* centers, float* shift, int32_t* stop, int stop_rule, float tol,
+                                          int64_t m, int64_t n, int64_t k, void* stream) {
+  const char* what = "kmeans_update_static";
+  if (int rc = km_check(what, x, labels_i64, labels_u8, centers, shift, m, n, k, stop_rule)) return rc;
+  F2CGT_REQUIRE(n * k <= kStaticSums && n <= kStaticCenters, F2CGT_E_UNSUPPORTED,
+                "%s: at most %lld sums (n * k) and %lld centres fit the built-in scratch (got %lld and %lld); "
+                "use f2cgt_kmeans_update with a workspace",
+                what, (long long)kStaticSums, (long long)kStaticCenters, (long long)(n * k), (long long)n);
+  // the device address of the scratch array, looked up once per device (every device has its own copy)
+  static void* scratch_of[64] = {nullptr};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= 64) return fail(F2CGT_E_DEVICE, "%s: no current device", what);
+  void* base = __atomic_load_n(&scratch_of[dev], __ATOMIC_ACQUIRE);
+  if (base == nullptr) {
+    e = hipGetSymbolAddress(&base, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || base == nullptr)
+      return fail((int)(e != hipSuccess ? e : hipErrorInvalidSymbol), "%s: cannot resolve the scratch array: %s", what,
+                  hipGetErrorString(e));
+    __atomic_store_n(&scratch_of[dev], base, __ATOMIC_RELEASE);
+  }
+  KmArgs a{};
+  a.x = x; a.labels_i64 = labels_i64; a.labels_u8 = labels_u8; a.centers = centers; a.shift = shift; a.stop = stop;
+  a.sums = static_cast<float*>(base);
+  a.counts = reinterpret_cast<uint32_t*>(a.sums + n * k);
+  a.m = m; a.n = (int)n; a.k = (int)k; a.rule = stop_rule; a.tol = tol;
+  return km_run(what, a, as_stream(stream));
+}

@@ -238,6 +238,17 @@ int f2cgt_kmeans_update(const float* x, const int64_t* labels_i64, const uint8_t
                         float* shift, int32_t* stop, int stop_rule, float tol, void* workspace,
                         int64_t workspace_bytes, int64_t m, int64_t n, int64_t k, void* stream);
 
+/* f2cgt_kmeans_update without a workspace and without any allocation (no counterpart in the
+ * reference: it is for callers that cannot allocate device memory -- code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  The partial sums live in a device array
+ * inside the library (272 KB per device, kept until the process ends), so the problem is limited to
+ * n * k <= 65536 sums and n <= 4096 centres; larger ones return F2CGT_E_UNSUPPORTED.  Same arguments,
+ * results and stop-flag behaviour as f2cgt_kmeans_update.  Every call on a device uses that device's
+ * one array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not. */
+int f2cgt_kmeans_update_static(const float* x, const int64_t* labels_i64, const uint8_t* labels_u8,
+                               float* centers, float* shift, int32_t* stop, int stop_rule, float tol,
+                               int64_t m, int64_t n, int64_t k, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
