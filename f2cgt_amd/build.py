@@ -25,11 +25,13 @@ HIP_SOURCES = ["runtime.hip", "packbits.hip", "sq.hip", "vq.hip", "spmm.hip", "s
 HIP_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    # MFMA results go to ordinary VGPRs: the arg-min update of the encode kernel then reads the
-    # scores directly instead of copying every accumulator out of the AGPR file first
-    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-pragmas",
 ]
+# MFMA results go to ordinary VGPRs: the arg-min update of the encode kernel then reads the scores
+# directly instead of copying every accumulator out of the AGPR file first.  An internal LLVM switch:
+# a compiler that no longer knows it must not break the build (the kernels are correct either way,
+# the encode step is slower without it), so it is probed before use.
+OPTIONAL_LLVM_FLAGS = ["-amdgpu-mfma-vgpr-form"]
 
 CAPI_LIB = os.path.join(LIB, "libf2cgt_hip.so")
 EXT_LIB = os.path.join(LIB, "F2CGTLib" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
@@ -42,6 +44,25 @@ def _run(cmd):
     return proc.stdout
 
 
+def _optional_flags(hipcc, verbose=True):
+    """The OPTIONAL_LLVM_FLAGS this compiler accepts, as `-mllvm <flag>` pairs."""
+    import tempfile
+
+    accepted = []
+    with tempfile.TemporaryDirectory() as tmp:
+        src = os.path.join(tmp, "probe.hip")
+        with open(src, "w") as fh:
+            fh.write("#include <hip/hip_runtime.h>\n__global__ void probe(float* p) { p[0] = 1.f; }\n")
+        for flag in OPTIONAL_LLVM_FLAGS:
+            proc = subprocess.run([hipcc, "--offload-arch=gfx950", "-c", src, "-o", os.path.join(tmp, "probe.o"),
+                                   "-mllvm", flag], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+            if proc.returncode == 0:
+                accepted += ["-mllvm", flag]
+            elif verbose:
+                print("build: this hipcc does not accept -mllvm %s; building without it" % flag)
+    return accepted
+
+
 def build_capi(verbose=True, experiments=False):
     """experiments=True also compiles the kernels that were measured and not adopted (they are
     selected at run time by the environment variables their sources name); the shipped library
@@ -50,10 +71,11 @@ def build_capi(verbose=True, experiments=False):
     os.makedirs(OBJ, exist_ok=True)
     hipcc = shutil.which("hipcc") or os.path.join(ROCM, "bin", "hipcc")
     sources = [s for s in HIP_SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    optional = _optional_flags(hipcc, verbose)
 
     def compile_one(src):
         obj = os.path.join(OBJ, src.replace(".hip", ".o"))
-        extra = ["-DF2CGT_EXPERIMENTS=1"] if experiments else []
+        extra = optional + (["-DF2CGT_EXPERIMENTS=1"] if experiments else [])
         out = _run([hipcc, *HIP_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj])
         if verbose and out.strip():
             print(out)

@@ -132,8 +132,15 @@ struct PlainDec {
     return r;
   }
   __device__ void accum(const Ctx&, const Raw& r, Acc (&acc)[NOUT_]) const {
+    if constexpr (std::is_same<T, __half>::value) {
+      // the reference sums in the feature type (src/fusion_spmm.cu:30-34): a half-precision sum is
+      // rounded to half after every edge, which the fp32 accumulator reproduces by rounding here
 #pragma unroll
-    for (int i = 0; i < NOUT_; ++i) acc[i] += (Acc)r.v[i];
+      for (int i = 0; i < NOUT_; ++i) acc[i] = __half2float(__float2half_rn(acc[i] + __half2float(r.v[i])));
+    } else {
+#pragma unroll
+      for (int i = 0; i < NOUT_; ++i) acc[i] += (Acc)r.v[i];
+    }
   }
 };
 

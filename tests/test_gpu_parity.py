@@ -303,9 +303,9 @@ def test_spmm_csr_f16_f64_and_empty():
     got = host(capi.spmm_csr(dev(f64), dev(indptr), dev(indices)))
     assert np.array_equal(got, oc.spmm_csr(f64, indptr, indices))
     f16 = rng.standard_normal((500, 33)).astype(np.float16)
-    got16 = host(capi.spmm_csr(dev(f16), dev(indptr), dev(indices))).astype(np.float32)
-    want16 = oc.spmm_csr(f16.astype(np.float32), indptr, indices)
-    assert np.allclose(got16, want16, rtol=2e-3, atol=2e-3)
+    # half features: the sum is rounded to half after every edge, as the reference's DType accumulator is
+    got16 = host(capi.spmm_csr(dev(f16), dev(indptr), dev(indices)))
+    assert got16.dtype == np.float16 and np.array_equal(got16, oc.spmm_csr(f16, indptr, indices))
     # no rows, no edges
     e = capi.spmm_csr(dev(f64.astype(np.float32)), dev(np.zeros(1, np.int64)), dev(np.zeros(0, np.int64)))
     assert e.shape == (0, 33)
