@@ -209,6 +209,37 @@ def _others(idx):
                                      "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
     del wl, out, feat
     torch.cuda.empty_cache()
+    # the aggregation together with the dense layer that consumes it, at the widest shape (768
+    # features -> 256 hidden units, fp32 like the reference's model): the aggregation alone, the GEMM
+    # alone, the module's *_linear op (one aggregation, one GEMM), its row-blocked form (bounded
+    # staging memory) and the blocked form with the next block's aggregation on a second stream
+    import f2cgt_amd
+    shim = f2cgt_amd.load()
+    wl = synth.WORKLOADS["c5"](device="cuda", idx_dtype=torch.int64)
+    hidden = 256
+    weight = torch.randn((hidden, wl["feat_dim"]), device="cuda") * 0.03
+    bias = torch.randn((hidden,), device="cuda")
+    agg = torch.empty((wl["R"], wl["feat_dim"]), dtype=torch.float32, device="cuda")
+    hid = torch.empty((wl["R"], hidden), dtype=torch.float32, device="cuda")
+    agg_only = _launcher(capi, wl, agg)
+    _, t_agg = _time_steps(agg_only, 30, 5)
+    _, t_gemm = _time_steps(lambda: torch.addmm(bias, agg, weight.t(), out=hid), 30, 5)
+
+    def two_pass():
+        agg_only()
+        torch.addmm(bias, agg, weight.t(), out=hid)
+
+    _, t_two = _time_steps(two_pass, 30, 5)
+    layer = {"aggregation_us": t_agg * 1e3, "gemm_fp32_us": t_gemm * 1e3, "aggregate_then_gemm_us": t_two * 1e3,
+             "gemm_TFLOPps": 2 * wl["R"] * wl["feat_dim"] * hidden / (t_gemm * 1e-3) / 1e12}
+    for block_rows, overlap in ((0, False), (65536, False), (131072, False), (65536, True), (131072, True)):
+        _, t = _time_steps(lambda: shim.vq_decompress_spmm_csr_linear(
+            wl["codes"], wl["codebooks"], wl["indptr"], wl["indices"], wl["feat_dim"], weight, bias, block_rows,
+            overlap), 30, 5)
+        layer["linear_op_block_%d%s_us" % (block_rows, "_overlap" if overlap else "")] = t * 1e3
+    res["c5_first_layer_768_to_256"] = layer
+    del wl, agg, hid, weight
+    torch.cuda.empty_cache()
     enc = synth.c5_encode(device="cuda")
     labels = torch.empty((enc["m"],), dtype=torch.uint8, device="cuda")
     _, ms = _time_steps(lambda: capi.kmeans_predict(enc["x"], enc["centers"], "l2", u8=True, out=labels), 50, 5)

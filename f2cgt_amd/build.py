@@ -105,7 +105,7 @@ def build_extension(verbose=True):
            "-Wno-deprecated-declarations"]
     cmd += ["-I" + p for p in includes]
     cmd += [os.path.join(CSRC, "f2cgtlib_pybind.cpp"), "-o", EXT_LIB,
-            "-L" + LIB, "-lf2cgt_hip", "-L" + torch_lib,
+            "-L" + LIB, "-lf2cgt_hip", "-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-L" + torch_lib,
             "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python",
             "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib]
     out = _run(cmd)

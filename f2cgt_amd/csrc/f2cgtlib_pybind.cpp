@@ -11,6 +11,11 @@
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <map>
+#include <mutex>
 #include <string>
 
 #include "../../include/f2cgt.h"
@@ -473,6 +478,181 @@ torch::Tensor hybrid_decompress_spmm_csr(torch::Tensor row_map, torch::Tensor sq
   return out;
 }
 
+void check_hip(hipError_t err, const char* what) {
+  TORCH_CHECK(err == hipSuccess, what, ": ", hipGetErrorString(err));
+}
+
+// One extra stream (default priority) and its events per device, made on first use and kept for
+// the life of the process.  Calls that overlap on one device from several host threads would share
+// the events; the module is used from one thread per device like the reference's.
+struct SideStream {
+  hipStream_t stream = nullptr;
+  hipEvent_t inputs_ready = nullptr, agg_done[2] = {nullptr, nullptr}, gemm_done[2] = {nullptr, nullptr};
+};
+
+SideStream* side_stream_of(int device) {
+  static std::mutex lock;
+  static std::map<int, SideStream> made;
+  std::lock_guard<std::mutex> hold(lock);
+  auto it = made.find(device);
+  if (it != made.end()) return &it->second;
+  SideStream s;
+  check_hip(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+  for (hipEvent_t* ev : {&s.inputs_ready, &s.agg_done[0], &s.agg_done[1], &s.gemm_done[0], &s.gemm_done[1]})
+    check_hip(hipEventCreateWithFlags(ev, hipEventDisableTiming), "hipEventCreateWithFlags");
+  return &made.emplace(device, s).first->second;
+}
+
+// Aggregation followed by the dense layer that consumes it (the first layer of the GraphSAGE model,
+// examples/models/sage.py:62-70 with the mean aggregator: h = fc_neigh(mean over the neighbours)).
+// At the reference's widest shape (768 features -> 256 units, 341k destination rows) the fp32 GEMM
+// takes 1.75 ms at 86 % of the matrix cores' fp32 peak and the aggregation 0.5 ms, so the multiply
+// is not moved into the aggregation kernel: it would slow the part that already dominates.
+//   block_rows == 0   one aggregation into a full-size buffer, one GEMM (the fastest form measured)
+//   block_rows  > 0   destination rows in blocks of that many: the aggregate exists one block at a
+//                     time, which bounds the extra memory to block_rows*feat_dim*4 bytes (1 GB at
+//                     the shape above otherwise); ~6 % slower with 65536-row blocks
+//   overlap           with blocks: the aggregation of block b+1 runs on a second stream beside the
+//                     GEMM of block b, with two staging buffers.  Measured slower than running them
+//                     one after the other (the two kernels contend for the same compute units), so
+//                     it is off by default and kept for measurement.
+// `agg(indptr_ptr, indices_ptr, rows, edges, dst, stream)` enqueues one block on `stream`.  With
+// blocks the call reads the edge offsets of the block boundaries on the host, so it cannot be
+// captured into a graph.
+template <class Agg>
+torch::Tensor aggregate_then_linear(const Graph& g, int64_t feat_dim, const torch::Tensor& like,
+                                    torch::Tensor weight, const c10::optional<torch::Tensor>& bias,
+                                    int64_t block_rows, bool overlap, Agg agg) {
+  weight = dev_contig(weight, "weight");
+  TORCH_CHECK(weight.dim() == 2 && weight.scalar_type() == torch::kFloat32 && weight.size(1) == feat_dim,
+              "weight must be float32 [out_features, feat_dim]");
+  torch::Tensor b;
+  if (bias.has_value()) {
+    b = dev_contig(*bias, "bias");
+    TORCH_CHECK(b.dim() == 1 && b.scalar_type() == torch::kFloat32 && b.size(0) == weight.size(0),
+                "bias must be float32 [out_features]");
+  }
+  TORCH_CHECK(block_rows >= 0, "block_rows must be >= 0 (0 = all rows at once)");
+  auto out = empty_f32({g.rows, weight.size(0)}, like);
+  if (g.rows == 0) return out;
+  if (block_rows == 0) block_rows = g.rows;
+  block_rows = std::min(block_rows, g.rows);
+  const int64_t n_blocks = (g.rows + block_rows - 1) / block_rows;
+  auto wt = weight.t();
+  auto gemm = [&](torch::Tensor dst, const torch::Tensor& a) {
+    if (b.defined())
+      at::addmm_out(dst, b, a, wt);
+    else
+      at::mm_out(dst, a, wt);
+  };
+  if (n_blocks == 1) {
+    auto whole = empty_f32({g.rows, feat_dim}, like);
+    agg(g.indptr.data_ptr(), g.indices.data_ptr(), g.rows, g.edges, whole.data_ptr<float>(), current_stream());
+    gemm(out, whole);
+    return out;
+  }
+  // edge offsets at the block boundaries: the one host read of the call
+  auto at_rows = torch::arange(0, n_blocks + 1, torch::TensorOptions().dtype(torch::kInt64).device(like.device()))
+                     .mul_(block_rows).clamp_max_(g.rows);
+  auto bounds = g.indptr.index_select(0, at_rows).to(torch::kInt64).cpu();
+  const int64_t* e = bounds.data_ptr<int64_t>();
+  TORCH_CHECK(e[0] >= 0 && e[n_blocks] <= g.edges, "indptr does not fit indices");
+  for (int64_t blk = 0; blk < n_blocks; ++blk)
+    TORCH_CHECK(e[blk] <= e[blk + 1], "indptr must be non-decreasing");
+
+  // indptr of every block relative to the block's first edge (so that the kernel choice sees the
+  // block's own degree), all blocks in one [n_blocks, block_rows + 1] tensor
+  auto opts64 = torch::TensorOptions().dtype(torch::kInt64).device(like.device());
+  auto pos = torch::arange(0, n_blocks, opts64).mul_(block_rows).unsqueeze(1) +
+             torch::arange(0, block_rows + 1, opts64).unsqueeze(0);
+  auto rebased = (g.indptr.index_select(0, pos.clamp_max_(g.rows).reshape({-1})).reshape({n_blocks, block_rows + 1}) -
+                  bounds.slice(0, 0, n_blocks).to(like.device()).to(g.indptr.scalar_type()).unsqueeze(1))
+                     .contiguous();
+
+  const bool piped = overlap && n_blocks > 1;
+  hipStream_t main_stream = static_cast<hipStream_t>(current_stream());
+  SideStream* side = piped ? side_stream_of(like.device().index()) : nullptr;
+  hipStream_t agg_stream = piped ? side->stream : main_stream;
+  torch::Tensor stage[2];
+  for (int i = 0; i < (piped ? 2 : 1); ++i) stage[i] = empty_f32({block_rows, feat_dim}, like);
+  if (piped) {
+    check_hip(hipEventRecord(side->inputs_ready, main_stream), "hipEventRecord");
+    check_hip(hipStreamWaitEvent(agg_stream, side->inputs_ready, 0), "hipStreamWaitEvent");
+  }
+  const int64_t isz = g.indices.element_size(), psz = g.indptr.element_size();
+  try {
+  for (int64_t blk = 0; blk < n_blocks; ++blk) {
+    const int64_t r0 = blk * block_rows, n = std::min(block_rows, g.rows - r0);
+    const int slot = piped ? (int)(blk & 1) : 0;
+    // the GEMM that last read this staging buffer must be over
+    if (piped && blk >= 2) check_hip(hipStreamWaitEvent(agg_stream, side->gemm_done[slot], 0), "hipStreamWaitEvent");
+    agg(static_cast<const char*>(rebased.data_ptr()) + blk * (block_rows + 1) * psz,
+        static_cast<const char*>(g.indices.data_ptr()) + e[blk] * isz, n, e[blk + 1] - e[blk],
+        stage[slot].data_ptr<float>(), static_cast<void*>(agg_stream));
+    if (piped) {
+      check_hip(hipEventRecord(side->agg_done[slot], agg_stream), "hipEventRecord");
+      check_hip(hipStreamWaitEvent(main_stream, side->agg_done[slot], 0), "hipStreamWaitEvent");
+    }
+    gemm(out.narrow(0, r0, n), stage[slot].narrow(0, 0, n));
+    if (piped) check_hip(hipEventRecord(side->gemm_done[slot], main_stream), "hipEventRecord");
+  }
+  } catch (...) {
+    // a refused launch: nothing on the second stream may still use the staging buffers when they
+    // are released
+    if (piped) (void)hipStreamSynchronize(agg_stream);
+    throw;
+  }
+  // every launch on the second stream is followed by a wait on the caller's stream, so the staging
+  // buffers go back to the allocator under the caller's stream as usual
+  return out;
+}
+
+torch::Tensor vq_decompress_spmm_csr_linear(torch::Tensor compress_feat, torch::Tensor codebooks,
+                                            torch::Tensor indptr, torch::Tensor indices, int64_t feat_dim,
+                                            torch::Tensor weight, c10::optional<torch::Tensor> bias,
+                                            int64_t block_rows, bool overlap) {
+  compress_feat = dev_contig(compress_feat, "compress_feat");
+  codebooks = dev_contig(codebooks, "codebooks");
+  TORCH_CHECK(compress_feat.dim() == 2, "compress_feat must be [rows, n_codebooks]");
+  TORCH_CHECK(codebooks.dim() == 3 && codebooks.scalar_type() == torch::kFloat32,
+              "VQ codebooks must be float32 [n_codebooks, K, width]");
+  TORCH_CHECK(compress_feat.size(1) == codebooks.size(0), "compress_feat has ", compress_feat.size(1),
+              " columns but there are ", codebooks.size(0), " codebooks");
+  Graph g = graph_of(indptr, indices);
+  c10::DeviceGuard guard(compress_feat.device());
+  const int tag = dtype_tag(compress_feat, "compress_feat");
+  return aggregate_then_linear(
+      g, feat_dim, compress_feat, weight, bias, block_rows, overlap,
+      [&](const void* ip, const void* ix, int64_t rows, int64_t edges, float* dst, void* stream) {
+        check_rc(f2cgt_vq_decompress_spmm_csr(compress_feat.data_ptr(), tag, codebooks.data_ptr<float>(), ip, ix,
+                                              g.tag, dst, rows, edges, compress_feat.size(0), feat_dim,
+                                              codebooks.size(0), codebooks.size(1), codebooks.size(2),
+                                              stream),
+                 "vq_decompress_spmm_csr_linear");
+      });
+}
+
+torch::Tensor sq_decompress_spmm_csr_linear(torch::Tensor compress_feat, torch::Tensor codebooks,
+                                            torch::Tensor indptr, torch::Tensor indices, int64_t target_bit,
+                                            int64_t column_slice, int64_t feat_dim, torch::Tensor weight,
+                                            c10::optional<torch::Tensor> bias, int64_t block_rows, bool overlap) {
+  compress_feat = dev_contig(compress_feat, "compress_feat");
+  TORCH_CHECK(compress_feat.dim() == 2, "compress_feat must be 2-D");
+  codebooks = sq_codebooks_checked(codebooks);
+  Graph g = graph_of(indptr, indices);
+  c10::DeviceGuard guard(compress_feat.device());
+  const int tag = dtype_tag(compress_feat, "compress_feat");
+  return aggregate_then_linear(
+      g, feat_dim, compress_feat, weight, bias, block_rows, overlap,
+      [&](const void* ip, const void* ix, int64_t rows, int64_t edges, float* dst, void* stream) {
+        check_rc(f2cgt_sq_decompress_spmm_csr(compress_feat.data_ptr(), tag, codebooks.data_ptr<float>(), ip, ix,
+                                              g.tag, dst, rows, edges, compress_feat.size(0),
+                                              compress_feat.size(1), feat_dim, codebooks.size(0), (int)target_bit,
+                                              column_slice, stream),
+                 "sq_decompress_spmm_csr_linear");
+      });
+}
+
 torch::Tensor kmeans_predict(torch::Tensor x, torch::Tensor centers, std::string metric) {
   return kmeans_predict_impl(x, centers, metric, false);
 }
@@ -545,6 +725,13 @@ PYBIND11_MODULE(F2CGTLib, m) {
       .def("hybrid_decompress_spmm_csr", &hybrid_decompress_spmm_csr, py::arg("row_map"),
            py::arg("sq_codes"), py::arg("sq_params"), py::arg("vq_codes"), py::arg("vq_codebooks"),
            py::arg("indptr"), py::arg("indices"), py::arg("feat_dim"))
+      .def("vq_decompress_spmm_csr_linear", &vq_decompress_spmm_csr_linear, py::arg("compress_feat"),
+           py::arg("codebooks"), py::arg("indptr"), py::arg("indices"), py::arg("feat_dim"),
+           py::arg("weight"), py::arg("bias") = py::none(), py::arg("block_rows") = 0, py::arg("overlap") = false)
+      .def("sq_decompress_spmm_csr_linear", &sq_decompress_spmm_csr_linear, py::arg("compress_feat"),
+           py::arg("codebooks"), py::arg("indptr"), py::arg("indices"), py::arg("target_bit"),
+           py::arg("column_slice"), py::arg("feat_dim"), py::arg("weight"), py::arg("bias") = py::none(),
+           py::arg("block_rows") = 0, py::arg("overlap") = false)
       .def("sq_encode", &sq_encode, py::arg("src"), py::arg("codebooks"), py::arg("target_bits"),
            py::arg("column_slice"))
       .def("kmeans_predict", &kmeans_predict, py::arg("x"), py::arg("centers"), py::arg("metric"))

@@ -763,27 +763,10 @@ int launch_acc_tb(AccArgs a, size_t lds, int64_t grid, const void* indptr, const
   return launch_status(what);
 }
 
-template <int BITS>
-int launch_acc(AccArgs a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
-               const char* what) {
-  a.eff_bytes = (int)ceil_div(a.feat_dim, 8 / BITS);
-  a.lanes = (int)ceil_div(a.eff_bytes, 8);
-  const int lanes2 = pow2_ceil(a.lanes);
-  a.lane_shift = 0;
-  while ((1 << a.lane_shift) < lanes2) ++a.lane_shift;
-  // rows of the accumulator array start lanes2 banks apart so that the lane groups of a wave,
-  // which mostly work on neighbouring rows, spread over all 32 banks
-  const int skew = lanes2 % 32;
-  a.pitch_n = ((4 * a.lanes + 31) / 32 * 32 + skew + 3) & ~3;
-  a.pitch_w = ((8 * a.lanes + 31) / 32 * 32 + skew + 3) & ~3;
-  a.f4_per_row = a.feat_dim / 4;
-  const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 1.0;
-  const double dg = avg_deg > 0.5 ? avg_deg : 0.5;
-  // the wide layout runs on half the rows at a time, so it must fit twice into the narrow one
-  const size_t acc_row = (size_t)(a.pitch_n * 2 > a.pitch_w ? a.pitch_n : (a.pitch_w + 1) / 2) * 4;
-  // 128-thread workgroups: more, smaller blocks in flight per CU overlap the dependent
-  // indptr -> indices -> code-row loads of one block with the output stores of others
-  constexpr int TB = 128;
+// Block geometry for TB-thread workgroups, then the launch.
+template <int TB, int BITS>
+int launch_acc_sized(AccArgs a, double dg, size_t acc_row, const void* indptr, const void* indices, int idx_dtype,
+                     float* out, hipStream_t st, const char* what) {
   a.edge_batch = 2 * TB;
   int sub = ((int)(TB / dg) + 4) / 8 * 8;  // ~one edge per thread and sub-block, multiple of 8 rows
   sub = sub < 8 ? 8 : (sub > 64 ? 64 : sub);
@@ -810,6 +793,35 @@ int launch_acc(AccArgs a, const void* indptr, const void* indices, int idx_dtype
   const int64_t grid = ceil_div(a.R, rb);
   if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
   return launch_acc_tb<TB, BITS>(a, lds, grid, indptr, indices, idx_dtype, out, st, what);
+}
+
+template <int BITS>
+int launch_acc(AccArgs a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
+               const char* what) {
+  a.eff_bytes = (int)ceil_div(a.feat_dim, 8 / BITS);
+  a.lanes = (int)ceil_div(a.eff_bytes, 8);
+  const int lanes2 = pow2_ceil(a.lanes);
+  a.lane_shift = 0;
+  while ((1 << a.lane_shift) < lanes2) ++a.lane_shift;
+  // rows of the accumulator array start lanes2 banks apart so that the lane groups of a wave,
+  // which mostly work on neighbouring rows, spread over all 32 banks
+  const int skew = lanes2 % 32;
+  a.pitch_n = ((4 * a.lanes + 31) / 32 * 32 + skew + 3) & ~3;
+  a.pitch_w = ((8 * a.lanes + 31) / 32 * 32 + skew + 3) & ~3;
+  a.f4_per_row = a.feat_dim / 4;
+  const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 1.0;
+  const double dg = avg_deg > 0.5 ? avg_deg : 0.5;
+  // the wide layout runs on half the rows at a time, so it must fit twice into the narrow one
+  const size_t acc_row = (size_t)(a.pitch_n * 2 > a.pitch_w ? a.pitch_n : (a.pitch_w + 1) / 2) * 4;
+  // 128-thread workgroups: more, smaller blocks in flight per CU overlap the dependent
+  // indptr -> indices -> code-row loads of one block with the output stores of others
+#ifdef F2CGT_EXPERIMENTS
+  if (const char* v = getenv("F2CGT_ACC_TB")) {   // workgroup size for an A/B: 64 or 256
+    if (atoi(v) == 64) return launch_acc_sized<64, BITS>(a, dg, acc_row, indptr, indices, idx_dtype, out, st, what);
+    if (atoi(v) == 256) return launch_acc_sized<256, BITS>(a, dg, acc_row, indptr, indices, idx_dtype, out, st, what);
+  }
+#endif
+  return launch_acc_sized<128, BITS>(a, dg, acc_row, indptr, indices, idx_dtype, out, st, what);
 }
 
 
@@ -1486,6 +1498,13 @@ int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float*
   // threads and 16 rows: 318; twice the rows per block at either size: 332-344).  Measured slower
   // or equal outside that range (2, 5 or 60 edges per row, 256 columns), which keeps the 256-thread form.
   const double avg_deg = R > 0 ? (double)E / (double)R : 0.0;
+#ifdef F2CGT_EXPERIMENTS
+  if (const char* v = getenv("F2CGT_HYB_TB")) {   // workgroup size for an A/B: 64, 128 or 256
+    if (atoi(v) == 64) return launch_hybrid<64>(a, indptr, indices, idx_dtype, out, st, what);
+    if (atoi(v) == 128) return launch_hybrid<128>(a, indptr, indices, idx_dtype, out, st, what);
+    if (atoi(v) == 256) return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what);
+  }
+#endif
   if (a.ch2 <= 32 && avg_deg >= 8.0 && avg_deg <= 32.0)
     return launch_hybrid<64>(a, indptr, indices, idx_dtype, out, st, what);
   return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what);

@@ -39,6 +39,7 @@ struct VqArgs {
   int n_tiles, n_stripes;
   int stripes_per_xcd;  // > 0: the column tiles of a stripe share one XCD (see the kernel)
   int dense_store;      // sparse rows: results go through LDS so that every store instruction is dense
+  int store_late;       // experiments build only: selects the LATE form of the wave kernel (1..3)
 };
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -287,7 +288,7 @@ constexpr int kWPtr = 56;                     // ints per offset buffer: [0..48]
 
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
-template <int BT, int H, int RPM, typename Idx>
+template <int BT, int H, int RPM, typename Idx, int LATE = 0>
 __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* __restrict__ indptr,
                                                            const Idx* __restrict__ indices,
                                                            float* __restrict__ out) {
@@ -405,6 +406,25 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     park_P(0);
   }
   CW Creg = {};
+  // The two 16-byte stores of a lane and step are issued where the results are ready, at the end of
+  // the step.  A wave's memory operations retire in order and the compiler's wait in front of the
+  // first use of a load also covers every store issued before that load, so the wave then sleeps
+  // on its stores at the top of the next step while the other waves of the CU work.  LATE (built
+  // with the experiments only, chosen by F2CGT_VQ_DEFER) holds the results in registers instead
+  // and stores them in the next step: 1 = at its end, 2 = behind its loads, so that the stores have
+  // that step's sums to complete, 3 = as 2 with a wait for them in front of the sums.  All three
+  // were measured much slower than the direct form (24 x 32 codebooks: 493 us direct, 860-910 / 960
+  // / 580-680 us), although the instructions of a step are the same: not adopted.
+  float4 pend_v[2] = {make_float4(0.f, 0.f, 0.f, 0.f), make_float4(0.f, 0.f, 0.f, 0.f)};
+  float* pend_p[2] = {out, out};
+  bool pend_on[2] = {false, false};
+  auto flush_stores = [&]() {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if (pend_on[j]) store_nt4(pend_p[j], pend_v[j].x, pend_v[j].y, pend_v[j].z, pend_v[j].w);
+      pend_on[j] = false;
+    }
+  };
   for (int64_t g = g_first; g < n_mini; ++g) {
     // chunk-level P stage, driven by the position of g inside its chunk
     if (g >= 0) {
@@ -435,6 +455,10 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       const Idx* src = on ? indices + e0 + eb2 + lane : indptr;
       Ireg = (int64_t)*src;
     }
+    if constexpr (LATE >= 2) {
+      flush_stores();   // results of mini-block g - 1
+      if (LATE == 3) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
     // compute mini-block g
     if (g >= 0) {
       const int64_t c = g / kMini;
@@ -448,6 +472,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       // them takes the row's edges s, s + SPR, ... and the partial sums are added across the slots
       constexpr int SPR = kRowsPerPass / (RPM < kRowsPerPass ? RPM : kRowsPerPass);
       constexpr int kPasses = RPM * SPR / kRowsPerPass;
+      static_assert(LATE == 0 || H * kPasses == 2, "two pending stores per lane");
       // sum of the codebook entries of this slot's share of row `row` (all of it when SPR == 1),
       // in edge order; returns the row's edge count
       auto row_sum = [&](int row, int sub, float (&acc)[H][4]) -> int {
@@ -514,7 +539,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
             for (int t = 0; t < 4; ++t) acc[h][t] = div_by(acc[h][t], d, r);
         }
       };
-      if (H == 2 && SPR == 1 && kPasses == 1 && a.dense_store) {
+      if (H == 2 && SPR == 1 && kPasses == 1 && a.dense_store == 1) {
         // Four rows, sixteen lanes each.  A lane's result is 32 consecutive bytes, which as two
         // stores would be 16 of every 32 bytes per instruction (half-written sectors on the way to
         // memory).  The wave's 1 KB staging area, free once the edge loops are done, turns them
@@ -543,7 +568,13 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
           __builtin_amdgcn_wave_barrier();
           const float4 v = stg[row * 16 + c4];
           const int col = 64 * p + 4 * c4;
-          if (row < nr && col < tile_cols) store_nt4(obase + col, v.x, v.y, v.z, v.w);
+          if constexpr (LATE) {
+            pend_v[p] = v;
+            pend_p[p] = obase + col;
+            pend_on[p] = row < nr && col < tile_cols;
+          } else {
+            if (row < nr && col < tile_cols) store_nt4(obase + col, v.x, v.y, v.z, v.w);
+          }
         }
       } else if (col_on) {
         float* orow = out + row0 * (int64_t)a.feat_dim + tile * 128 + col0;
@@ -569,14 +600,23 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
           if (a.dense_store == 2 && acc[0][0] != 12345.678f) continue;   // no stores: what the rest of the kernel costs
 #endif
 #pragma unroll
-          for (int h = 0; h < H; ++h)
-            store_nt4(orow + (int64_t)row * a.feat_dim + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+          for (int h = 0; h < H; ++h) {
+            if constexpr (LATE) {
+              pend_v[pass * H + h] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+              pend_p[pass * H + h] = orow + (int64_t)row * a.feat_dim + 4 * h;
+              pend_on[pass * H + h] = true;
+            } else {
+              store_nt4(orow + (int64_t)row * a.feat_dim + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+            }
+          }
         }
       }
     }
+    if constexpr (LATE == 1) flush_stores();
     eb0 = eb1; ne0 = ne1;
     eb1 = eb2; ne1 = ne2;
   }
+  if constexpr (LATE) flush_stores();
 }
 
 #ifdef F2CGT_EXPERIMENTS
@@ -925,6 +965,20 @@ int launch_strip_w(const VqArgs& a, int ke, const void* indptr, const void* indi
 
 #endif  // F2CGT_EXPERIMENTS
 
+#ifdef F2CGT_EXPERIMENTS
+// the 4-row, int64 form of the wave kernel with its stores held back (see LATE in the kernel)
+template <int BT, int LATE>
+int launch_wave_late(const VqArgs& a, const void* indptr, const void* indices, float* out, hipStream_t st,
+                     const char* what, unsigned grid, size_t wlds) {
+  const void* kern = reinterpret_cast<const void*>(vq_wave_kernel<BT, 2, 4, int64_t, LATE>);
+  const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
+  if (e != hipSuccess) return fail((int)e, "%s: cannot reserve %zu B of LDS", what, wlds);
+  vq_wave_kernel<BT, 2, 4, int64_t, LATE><<<grid, kThreads, wlds, st>>>(a, static_cast<const int64_t*>(indptr),
+                                                                         static_cast<const int64_t*>(indices), out);
+  return launch_status(what);
+}
+#endif
+
 template <int BT, int H, int RPM>
 int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
                 const char* what, unsigned grid, size_t wlds) {
@@ -932,6 +986,13 @@ int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int id
     plan_record("vq_wave_kernel", grid, kThreads, (int64_t)wlds, 0, H, RPM, a.dense_store);
     return 0;
   }
+#ifdef F2CGT_EXPERIMENTS
+  if (H == 2 && RPM == 4 && idx_dtype == F2CGT_DT_I64) {
+    if (a.store_late == 1) return launch_wave_late<BT, 1>(a, indptr, indices, out, st, what, grid, wlds);
+    if (a.store_late == 2) return launch_wave_late<BT, 2>(a, indptr, indices, out, st, what, grid, wlds);
+    if (a.store_late == 3) return launch_wave_late<BT, 3>(a, indptr, indices, out, st, what, grid, wlds);
+  }
+#endif
   const void* kern = idx_dtype == F2CGT_DT_I32 ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t>)
                                                : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t>);
   const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
@@ -975,6 +1036,7 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
   a.dense_store = avg_deg <= 8.0;
 #ifdef F2CGT_EXPERIMENTS
   {
+    if (const char* d = getenv("F2CGT_VQ_DEFER")) a.store_late = atoi(d);
     const char* v = getenv("F2CGT_VQ_STRIP");
     const int mode = v ? atoi(v) : 0;     // 0 off; tens: 0 plain, 1 non-temporal, 2 no stores; units: 2 = KE by degree, 6 = KE 16
     if (mode == 20) a.dense_store = 2;

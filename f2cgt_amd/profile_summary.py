@@ -51,10 +51,11 @@ N_SIMD, N_XCD, N_CU = 1024, 8, 256
 
 
 def csrc_sha16():
-    """Content hash of the kernel sources: a traffic figure belongs to the kernels it was measured on."""
+    """Content hash of the kernel sources (*.hip, *.hpp): a traffic figure belongs to the kernels it was
+    measured on."""
     h = hashlib.sha256()
     for path in sorted(glob.glob(os.path.join(PKG, "csrc", "*"))):
-        if os.path.isfile(path):
+        if os.path.isfile(path) and path.endswith((".hip", ".hpp")):
             h.update(os.path.basename(path).encode())
             h.update(open(path, "rb").read())
     return h.hexdigest()[:16]
