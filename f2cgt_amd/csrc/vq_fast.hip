@@ -407,14 +407,17 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   }
   CW Creg = {};
   // The two 16-byte stores of a lane and step are issued where the results are ready, at the end of
-  // the step.  A wave's memory operations retire in order and the compiler's wait in front of the
-  // first use of a load also covers every store issued before that load, so the wave then sleeps
-  // on its stores at the top of the next step while the other waves of the CU work.  LATE (built
-  // with the experiments only, chosen by F2CGT_VQ_DEFER) holds the results in registers instead
-  // and stores them in the next step: 1 = at its end, 2 = behind its loads, so that the stores have
-  // that step's sums to complete, 3 = as 2 with a wait for them in front of the sums.  All three
-  // were measured much slower than the direct form (24 x 32 codebooks: 493 us direct, 860-910 / 960
-  // / 580-680 us), although the instructions of a step are the same: not adopted.
+  // the step, back to back from one base register.  In the direct (not LDS-staged) form they are
+  // the two halves of the lane's 32 bytes, and they have to reach the L1 together: issued a few
+  // instructions apart (separate predicated blocks) the halves are written to memory separately
+  // and the kernel falls into a regime twice as slow (24 x 32 codebooks: 497 -> 870-960 us, L2 ->
+  // memory write-credit stalls up from 2e4 to 3.7e7 cycles per launch).  LATE (built with the
+  // experiments only, chosen by F2CGT_VQ_DEFER) holds the results in registers and stores them later:
+  // 1 = at the end of the step, 2 = behind the loads of the next step, so that the stores have that
+  // step's sums to complete, 3 = as 2 with a wait for them in front of the sums.  With whole-line
+  // stores (the LDS-staged form, F2CGT_VQ_DENSE=1) all placements run at the same speed (520 us),
+  // i.e. a wave does not lose time waiting for its own stores and there is nothing to gain by
+  // moving them; with the half-line pair every LATE form is in the slow regime.  Not adopted.
   float4 pend_v[2] = {make_float4(0.f, 0.f, 0.f, 0.f), make_float4(0.f, 0.f, 0.f, 0.f)};
   float* pend_p[2] = {out, out};
   bool pend_on[2] = {false, false};
@@ -1037,6 +1040,7 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
 #ifdef F2CGT_EXPERIMENTS
   {
     if (const char* d = getenv("F2CGT_VQ_DEFER")) a.store_late = atoi(d);
+    if (const char* d = getenv("F2CGT_VQ_DENSE")) a.dense_store = atoi(d) != 0;   // results through LDS at any degree
     const char* v = getenv("F2CGT_VQ_STRIP");
     const int mode = v ? atoi(v) : 0;     // 0 off; tens: 0 plain, 1 non-temporal, 2 no stores; units: 2 = KE by degree, 6 = KE 16
     if (mode == 20) a.dense_store = 2;

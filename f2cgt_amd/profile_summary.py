@@ -6,7 +6,7 @@ HBM-traffic record profiles/traffic.json that bench.py reads.
 Nothing is run here.  <rocprof_out_dir> is expected to hold, per workload w in c1..c5, the output
 directories of these runs (`cd /tmp && export TMPDIR=/tmp` first, every run on its own, from the
 repository root; B = `python3 bench.py --workload <w> --steps 2000 --warmup 200 --cpu-seconds 0`,
-with 300 / 60 steps for c4 / c5; T = B except for c2, where T = `python3 bench.py --workload c2
+with 300 steps for c4 and c5 (30 and 100 warm-up launches); T = B except for c2, where T = `python3 bench.py --workload c2
 --cpu-seconds 0` and T20 = `python3 bench.py --workload c2 --steps 20 --warmup 5 --cpu-seconds 0`):
 
     trace_<w>   rocprofv3 --kernel-trace --stats --output-format csv -d <dir>/trace_<w> -o t -- T
@@ -46,7 +46,7 @@ WORKLOADS = {
     "c4": ("hybrid_acc_kernel", "c4_hybrid"),
     "c5": ("vq_wave_kernel", "c5_vq_24x32"),
 }
-STEPS = {"c1": (2000, 200), "c2": (2000, 200), "c3": (2000, 200), "c4": (300, 30), "c5": (60, 10)}
+STEPS = {"c1": (2000, 200), "c2": (2000, 200), "c3": (2000, 200), "c4": (300, 30), "c5": (300, 100)}
 N_SIMD, N_XCD, N_CU = 1024, 8, 256
 
 
