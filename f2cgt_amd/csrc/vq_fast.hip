@@ -39,7 +39,8 @@ struct VqArgs {
   int n_tiles, n_stripes;
   int stripes_per_xcd;  // > 0: the column tiles of a stripe share one XCD (see the kernel)
   int dense_store;      // sparse rows: results go through LDS so that every store instruction is dense
-  int store_late;       // experiments build only: selects the LATE form of the wave kernel (1..3)
+  int store_late;       // experiments build only: selects the LATE form of the wave kernel (1..3; 9 = time stamps)
+  unsigned long long* trace;   // experiments build only: per wave {start, first step, end} in 100 MHz ticks
 };
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -269,11 +270,12 @@ __global__ __launch_bounds__(kThreads) void vq_pipe_kernel(VqArgs a, const Idx* 
 // pipeline, with wave-private staging in LDS.  After the codebook is staged no workgroup barrier
 // is left: a wave that waits for its loads does not hold the other fifteen, and the LDS
 // operations of one wave execute in order, so its own stage hand-overs need no synchronisation.
-// A wave owns chunks of 48 consecutive destination rows and walks them as mini-blocks of RPM rows
-// (<= 64 edges: one edge per lane in the I and C stages; larger ones are summed straight from
-// HBM).  RPM follows the average degree: 4 up to 15 edges per row, and 2 or 1 above, where the
-// lane groups left over in a pass share a row's edges and add their partial sums:
-//     P  the 49 row offsets of a chunk     one load per chunk, issued while the previous chunk
+// A wave takes chunks of 16 consecutive destination rows from its workgroup's range (dealt through
+// a counter in LDS) and walks them as mini-blocks of RPM rows (<= 64 edges: one edge per lane in the
+// I and C stages; larger ones are summed straight from HBM).  RPM follows the average degree: 4 up
+// to 15 edges per row, and 2 or 1 above, where the lane groups left over in a pass share a row's
+// edges and add their partial sums:
+//     P  the 17 row offsets of a chunk     one load per chunk, issued while the previous chunk
 //                                          starts, parked half a chunk later (two LDS buffers)
 //     I  source id of edge `lane`          issued two mini-blocks ahead, stays in the register
 //     C  code bytes of edge `lane`         issued one mini-block ahead, parked in LDS when due
@@ -282,9 +284,9 @@ __global__ __launch_bounds__(kThreads) void vq_pipe_kernel(VqArgs a, const Idx* 
 // block-synchronous version of this kernel.
 constexpr int kWRows = 4;
 constexpr int kWEdges = 64;
-constexpr int kWMini = 12;                    // mini-blocks per chunk
+constexpr int kWMini = 4;                     // 4-row mini-blocks per chunk
 constexpr int kWChunk = kWRows * kWMini;      // rows per chunk
-constexpr int kWPtr = 56;                     // ints per offset buffer: [0..48] offsets, [52..53] first edge
+constexpr int kWPtr = 56;                     // ints per offset buffer: [0..16] offsets, [52..53] first edge, [55] of the first buffer: next chunk
 
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
@@ -295,6 +297,10 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   using CW = typename code_word<BT>::type;
   constexpr int kWaves = kThreads / 64;
   constexpr int kMini = kWChunk / RPM;          // mini-blocks (RPM rows each) per chunk
+  constexpr bool HELD = LATE >= 1 && LATE <= 3; // results held in registers, stored later
+  constexpr bool TRACE = LATE == 9;             // time stamps per wave
+  unsigned long long t_start = 0;
+  if constexpr (TRACE) t_start = wall_clock64();
   const bool K_FITS_ONE_PASS = a.K * 32 <= 8 * kThreads;
   extern __shared__ __align__(16) unsigned char smem[];
   float* s_cb = reinterpret_cast<float*>(smem);
@@ -315,16 +321,28 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   }
   const int tile_cols = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
 
-  // A wave owns one contiguous range of rows (a multiple of 4, the same for every wave, so the
-  // work is balanced to one mini-block); chunk c of the wave covers rows [chunk_row0 + 48 c, +48).
-  const int64_t total_waves = (int64_t)a.n_stripes * kWaves;
-  const int64_t rows_per_wave = ((a.R + total_waves - 1) / total_waves + kWRows - 1) / kWRows * kWRows;
-  const int64_t chunk_stride = kWChunk;
-  const int64_t chunk_row0 = ((int64_t)stripe * kWaves + wave) * rows_per_wave;
-  const bool has_rows = chunk_row0 < a.R;
-  const int64_t row_end = chunk_row0 + rows_per_wave < a.R ? chunk_row0 + rows_per_wave : a.R;
-  const int64_t n_chunks = (row_end - chunk_row0 + kWChunk - 1) / kWChunk;
-  const int64_t n_mini = (row_end - chunk_row0 + RPM - 1) / RPM;
+  // A workgroup owns one contiguous range of rows, cut into chunks of 16 rows.  The waves deal the
+  // chunks among themselves through a counter in LDS: wave w starts with chunk w and takes the next
+  // free one whenever it starts a chunk (the one after the chunk it is working on, so that its row
+  // offsets and source ids are loaded a chunk ahead).  With equal fixed shares the oldest wave of
+  // each SIMD, which the hardware serves first, finished 25 % earlier than the youngest and the CU
+  // ran its last quarter with ever fewer waves (16 x 8 codebooks: waves 0-3 done at 69 us, 12-15 at
+  // 92 us); uneven degrees add to that.
+  const int64_t rows_per_wg = ((a.R + a.n_stripes - 1) / a.n_stripes + kWChunk - 1) / kWChunk * kWChunk;
+  const int64_t wg_row0 = (int64_t)stripe * rows_per_wg;
+  const int64_t row_end = wg_row0 + rows_per_wg < a.R ? wg_row0 + rows_per_wg : a.R;   // of the workgroup
+  const int64_t wg_chunks = row_end > wg_row0 ? (row_end - wg_row0 + kWChunk - 1) / kWChunk : 0;
+  const bool has_rows = wave < wg_chunks;
+  int* s_next = reinterpret_cast<int*>(smem + (size_t)a.K * 128 * 4 + (size_t)kWaves * kStage) + 55;
+  auto minis_of = [&](int64_t base) {   // mini-blocks of the chunk that starts at row `base`
+    const int64_t left = row_end - base;
+    return (int64_t)(((left < kWChunk ? left : (int64_t)kWChunk) + RPM - 1) / RPM);
+  };
+  int64_t base_cur = wg_row0 + (int64_t)wave * kWChunk;   // first row of the chunk being worked on
+  int64_t base_next = 0;
+  bool have_next = false;
+  int par = 0;                                             // offset buffer of the current chunk
+  int64_t n_mini = has_rows ? minis_of(base_cur) : 0;      // mini-blocks of the chunks taken so far
 
   // lanes per row: 32 lanes with one float4 each (H == 1) or 16 lanes with a whole 8-column code
   // each (H == 2); the wave then works on 2 or 4 rows at a time
@@ -337,16 +355,15 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   const uint8_t* code_base = a.codes + tile * BT;
   const uint32_t n_last = (uint32_t)(a.N - 1);
 
-  // loads and parks the offsets of chunk c into buffer (c & 1); returns nothing, the data is in LDS
+  // loads the row offsets of the chunk that starts at row0, and parks them in offset buffer `which`
   int64_t Preg = 0;
-  auto issue_P = [&](int64_t c) {
-    const int64_t row0 = chunk_row0 + c * chunk_stride;
+  auto issue_P = [&](int64_t row0) {
     const int64_t left = row_end - row0;
     const int nr = (int)(left < kWChunk ? left : kWChunk);
     Preg = (int64_t)indptr[row0 + (lane < nr ? lane : nr)];
   };
-  auto park_P = [&](int64_t c) {
-    int* buf = s_ptr + (int)(c & 1) * kWPtr;
+  auto park_P = [&](int which) {
+    int* buf = s_ptr + which * kWPtr;
     const uint32_t lo = (uint32_t)uni((int)(uint32_t)Preg);
     const uint32_t hi = (uint32_t)uni((int)(uint32_t)((uint64_t)Preg >> 32));
     int64_t e0 = (int64_t)(((uint64_t)hi << 32) | lo);
@@ -357,18 +374,17 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     if (lane <= kWChunk) buf[lane] = rel > 0x3fffffff ? 0x3fffffff : (int)rel;
     if (lane == 1) { buf[52] = (int)(uint32_t)e0; buf[53] = (int)(uint32_t)((uint64_t)e0 >> 32); }
   };
-  // bounds of mini-block g: first edge (relative to the chunk's e0) and edge count
-  auto bounds = [&](int64_t g, int& eb, int& ne) {
-    const int64_t c = g / kMini;
-    const int m = (int)(g - c * kMini);
-    const int* buf = s_ptr + (int)(c & 1) * kWPtr;
+  // bounds of mini-block m of the chunk in buffer `which`: first edge (relative to the chunk's e0)
+  // and edge count
+  auto bounds = [&](int which, int m, int& eb, int& ne) {
+    const int* buf = s_ptr + which * kWPtr;
     eb = uni(buf[m * RPM]);
     const int ee = uni(buf[m * RPM + RPM]);
     ne = ee - eb;
     ne = ne < 0 ? 0 : ne;
   };
-  auto chunk_e0 = [&](int64_t c) {
-    const int* buf = s_ptr + (int)(c & 1) * kWPtr;
+  auto chunk_e0 = [&](int which) {
+    const int* buf = s_ptr + which * kWPtr;
     const uint32_t lo = (uint32_t)uni(buf[52]), hi = (uint32_t)uni(buf[53]);
     return (int64_t)(((uint64_t)hi << 32) | lo);
   };
@@ -383,11 +399,12 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   if (K_FITS_ONE_PASS && stage_codebook_vec_ok(a.codebooks, a.w, tile_cols)) {
     float4 cbv[8];
     stage_codebook_load<kThreads>(cbv, a.codebooks, a.K, a.w, tile, tile_cols);
+    if (threadIdx.x == 0) *s_next = kWaves;   // chunks 0 .. 15 are the waves' first ones
     if (has_rows) {
-      issue_P(0);
+      issue_P(base_cur);
       park_P(0);
       if (n_mini > 0) {
-        bounds(0, eb1, ne1);
+        bounds(0, 0, eb1, ne1);
         const int64_t e0 = chunk_e0(0);
         const bool on = ne1 <= kWEdges && lane < ne1;
         const Idx* src = on ? indices + e0 + eb1 + lane : indptr;
@@ -400,9 +417,10 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     if (!has_rows) return;
   } else {
     stage_codebook_tile<kThreads, H == 2>(s_cb, a.codebooks, a.K, a.w, tile, tile_cols);
+    if (threadIdx.x == 0) *s_next = kWaves;
     __syncthreads();
     if (!has_rows) return;
-    issue_P(0);
+    issue_P(base_cur);
     park_P(0);
   }
   CW Creg = {};
@@ -428,13 +446,25 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       pend_on[j] = false;
     }
   };
+  unsigned long long t_first = 0;
+  if constexpr (TRACE) t_first = wall_clock64();
+  int m = (int)g_first;   // position of g inside its chunk (negative during the two start-up steps)
   for (int64_t g = g_first; g < n_mini; ++g) {
     // chunk-level P stage, driven by the position of g inside its chunk
     if (g >= 0) {
-      const int64_t c = g / kMini;
-      const int m = (int)(g - c * kMini);
-      if (m == 0 && c + 1 < n_chunks) issue_P(c + 1);
-      if (m == kMini / 2 && c + 1 < n_chunks) park_P(c + 1);
+      if (m == 0) {
+        // take the next free chunk of the workgroup and request its row offsets
+        int id = 0;
+        if (lane == 0) id = atomicAdd(s_next, 1);
+        id = uni(id);
+        have_next = id < wg_chunks;
+        if (have_next) {
+          base_next = wg_row0 + (int64_t)id * kWChunk;
+          n_mini += minis_of(base_next);
+          issue_P(base_next);
+        }
+      }
+      if (m == kMini / 2 && have_next) park_P(par ^ 1);
     }
     // park C(g)
     if (g >= 0 && ne0 <= kWEdges && lane < ne0) *reinterpret_cast<CW*>(s_codes + lane * BT) = Creg;
@@ -451,23 +481,23 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       const bool v = g + 2 < n_mini;
       int64_t e0 = 0;
       if (v) {
-        bounds(g + 2, eb2, ne2);
-        e0 = chunk_e0((g + 2) / kMini);
+        const bool over = m + 2 >= kMini;   // in the next chunk
+        const int which = over ? par ^ 1 : par;
+        bounds(which, over ? m + 2 - kMini : m + 2, eb2, ne2);
+        e0 = chunk_e0(which);
       }
       const bool on = v && ne2 <= kWEdges && lane < ne2;
       const Idx* src = on ? indices + e0 + eb2 + lane : indptr;
       Ireg = (int64_t)*src;
     }
-    if constexpr (LATE >= 2) {
+    if constexpr (LATE == 2 || LATE == 3) {
       flush_stores();   // results of mini-block g - 1
       if (LATE == 3) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     // compute mini-block g
     if (g >= 0) {
-      const int64_t c = g / kMini;
-      const int m = (int)(g - c * kMini);
-      const int* buf = s_ptr + (int)(c & 1) * kWPtr + m * RPM;
-      const int64_t row0 = chunk_row0 + c * chunk_stride + m * RPM;
+      const int* buf = s_ptr + par * kWPtr + m * RPM;
+      const int64_t row0 = base_cur + m * RPM;
       const int64_t left = row_end - row0;
       const int nr = (int)(left < RPM ? left : RPM);
       const bool staged = ne0 <= kWEdges;
@@ -475,7 +505,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       // them takes the row's edges s, s + SPR, ... and the partial sums are added across the slots
       constexpr int SPR = kRowsPerPass / (RPM < kRowsPerPass ? RPM : kRowsPerPass);
       constexpr int kPasses = RPM * SPR / kRowsPerPass;
-      static_assert(LATE == 0 || H * kPasses == 2, "two pending stores per lane");
+      static_assert(!HELD || H * kPasses == 2, "two pending stores per lane");
       // sum of the codebook entries of this slot's share of row `row` (all of it when SPR == 1),
       // in edge order; returns the row's edge count
       auto row_sum = [&](int row, int sub, float (&acc)[H][4]) -> int {
@@ -518,7 +548,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
           }
         } else {
           n = re - rb;
-          const int64_t e0 = chunk_e0(c) + eb0;
+          const int64_t e0 = chunk_e0(par) + eb0;
           for (int k = sub; k < n; k += SPR) {
             const int64_t id = clamp_idx(indices[e0 + rb + k], a.N);
             const uint32_t code = a.codes[id * a.n_cb + tile * BT + byte_idx];
@@ -571,7 +601,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
           __builtin_amdgcn_wave_barrier();
           const float4 v = stg[row * 16 + c4];
           const int col = 64 * p + 4 * c4;
-          if constexpr (LATE) {
+          if constexpr (HELD) {
             pend_v[p] = v;
             pend_p[p] = obase + col;
             pend_on[p] = row < nr && col < tile_cols;
@@ -604,7 +634,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
 #endif
 #pragma unroll
           for (int h = 0; h < H; ++h) {
-            if constexpr (LATE) {
+            if constexpr (HELD) {
               pend_v[pass * H + h] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
               pend_p[pass * H + h] = orow + (int64_t)row * a.feat_dim + 4 * h;
               pend_on[pass * H + h] = true;
@@ -618,8 +648,20 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     if constexpr (LATE == 1) flush_stores();
     eb0 = eb1; ne0 = ne1;
     eb1 = eb2; ne1 = ne2;
+    if (++m == kMini) {   // on to the next chunk (the loop ends here when there is none)
+      m = 0;
+      par ^= 1;
+      base_cur = base_next;
+      have_next = false;
+    }
   }
-  if constexpr (LATE) flush_stores();
+  if constexpr (HELD) flush_stores();
+  if constexpr (TRACE) {
+    if (lane == 0) {
+      unsigned long long* t = a.trace + ((size_t)blockIdx.x * kWaves + wave) * 4;
+      t[0] = t_start; t[1] = t_first; t[2] = wall_clock64(); t[3] = (unsigned long long)n_mini;
+    }
+  }
 }
 
 #ifdef F2CGT_EXPERIMENTS
@@ -969,6 +1011,8 @@ int launch_strip_w(const VqArgs& a, int ke, const void* indptr, const void* indi
 #endif  // F2CGT_EXPERIMENTS
 
 #ifdef F2CGT_EXPERIMENTS
+unsigned long long* g_trace = nullptr;   // device buffer for the time stamps of F2CGT_VQ_DEFER=9
+
 // the 4-row, int64 form of the wave kernel with its stores held back (see LATE in the kernel)
 template <int BT, int LATE>
 int launch_wave_late(const VqArgs& a, const void* indptr, const void* indices, float* out, hipStream_t st,
@@ -994,6 +1038,7 @@ int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int id
     if (a.store_late == 1) return launch_wave_late<BT, 1>(a, indptr, indices, out, st, what, grid, wlds);
     if (a.store_late == 2) return launch_wave_late<BT, 2>(a, indptr, indices, out, st, what, grid, wlds);
     if (a.store_late == 3) return launch_wave_late<BT, 3>(a, indptr, indices, out, st, what, grid, wlds);
+    if (a.store_late == 9 && a.trace) return launch_wave_late<BT, 9>(a, indptr, indices, out, st, what, grid, wlds);
   }
 #endif
   const void* kern = idx_dtype == F2CGT_DT_I32 ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t>)
@@ -1040,6 +1085,7 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
 #ifdef F2CGT_EXPERIMENTS
   {
     if (const char* d = getenv("F2CGT_VQ_DEFER")) a.store_late = atoi(d);
+    a.trace = g_trace;
     if (const char* d = getenv("F2CGT_VQ_DENSE")) a.dense_store = atoi(d) != 0;   // results through LDS at any degree
     const char* v = getenv("F2CGT_VQ_STRIP");
     const int mode = v ? atoi(v) : 0;     // 0 off; tens: 0 plain, 1 non-temporal, 2 no stores; units: 2 = KE by degree, 6 = KE 16
@@ -1083,6 +1129,10 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
 
 }  // namespace
 
+#ifdef F2CGT_EXPERIMENTS
+void set_trace(unsigned long long* p) { g_trace = p; }
+#endif
+
 bool vq_pipe_eligible(const void* codes, const float* codebooks, const float* out, int64_t R, int64_t E,
                       int64_t N, int feat_dim, int n_cb, int K, int w) {
   if (E < 1 || N < 1 || codes == nullptr) return false;  // idle lanes read row 0 / indptr[0]
@@ -1113,3 +1163,9 @@ int vq_pipe_run(const uint8_t* codes, const float* codebooks, const void* indptr
 }
 
 }  // namespace f2cgt
+
+#ifdef F2CGT_EXPERIMENTS
+// Experiments build only: device buffer of 4 x 64-bit words per wave (workgroups x 16 waves) that
+// the time-stamped form of vq_wave_kernel (F2CGT_VQ_DEFER=9) fills; nullptr switches it off.
+extern "C" void f2cgt_experiment_set_trace(unsigned long long* device_buffer) { f2cgt::set_trace(device_buffer); }
+#endif
