@@ -328,17 +328,25 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   // each SIMD, which the hardware serves first, finished 25 % earlier than the youngest and the CU
   // ran its last quarter with ever fewer waves (16 x 8 codebooks: waves 0-3 done at 69 us, 12-15 at
   // 92 us); uneven degrees add to that.
-  const int64_t rows_per_wg = ((a.R + a.n_stripes - 1) / a.n_stripes + kWChunk - 1) / kWChunk * kWChunk;
+  // A launch too small to give every wave a 16-row chunk is cut into one piece per wave instead
+  // (nothing is left to deal then, and no wave walks four mini-blocks while others idle).
+  const int64_t wg_share = (a.R + a.n_stripes - 1) / a.n_stripes;
+  const bool dealt = wg_share >= (int64_t)kWaves * kWChunk;
+  const int64_t piece = dealt ? (int64_t)kWChunk : ((wg_share + kWaves - 1) / kWaves + RPM - 1) / RPM * RPM;
+  const int64_t rows_per_wg = dealt ? (wg_share + kWChunk - 1) / kWChunk * kWChunk : piece * kWaves;
   const int64_t wg_row0 = (int64_t)stripe * rows_per_wg;
-  const int64_t row_end = wg_row0 + rows_per_wg < a.R ? wg_row0 + rows_per_wg : a.R;   // of the workgroup
-  const int64_t wg_chunks = row_end > wg_row0 ? (row_end - wg_row0 + kWChunk - 1) / kWChunk : 0;
-  const bool has_rows = wave < wg_chunks;
+  const int64_t wg_end = wg_row0 + rows_per_wg < a.R ? wg_row0 + rows_per_wg : a.R;
+  const int64_t wg_chunks = !dealt ? 0 : (wg_end > wg_row0 ? (wg_end - wg_row0 + kWChunk - 1) / kWChunk : 0);
+  // rows of this wave end here: the workgroup's range when chunks are dealt, else the wave's own piece
+  const int64_t my_row0 = wg_row0 + (int64_t)wave * piece;
+  const int64_t row_end = dealt ? wg_end : (my_row0 + piece < wg_end ? my_row0 + piece : wg_end);
+  const bool has_rows = my_row0 < row_end;
   int* s_next = reinterpret_cast<int*>(smem + (size_t)a.K * 128 * 4 + (size_t)kWaves * kStage) + 55;
   auto minis_of = [&](int64_t base) {   // mini-blocks of the chunk that starts at row `base`
     const int64_t left = row_end - base;
     return (int64_t)(((left < kWChunk ? left : (int64_t)kWChunk) + RPM - 1) / RPM);
   };
-  int64_t base_cur = wg_row0 + (int64_t)wave * kWChunk;   // first row of the chunk being worked on
+  int64_t base_cur = my_row0;                              // first row of the chunk being worked on
   int64_t base_next = 0;
   bool have_next = false;
   int par = 0;                                             // offset buffer of the current chunk
@@ -389,32 +397,49 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     return (int64_t)(((uint64_t)hi << 32) | lo);
   };
 
-  // The codebook tile and the wave's first row offsets travel together, and the source ids of the
-  // first mini-block are on their way while the tile is written to LDS: a launch over few rows is
-  // mostly this start-up (128 KB per CU, then three dependent round trips before the first sum).
+  // Start-up.  A launch over few rows is mostly this: 128 KB of codebook per CU and three dependent
+  // round trips (row offsets -> source ids -> code bytes) before the first sum.  The wave's first
+  // row offsets and the source ids of its first mini-block are requested and waited for on their
+  // own; the eight codebook loads of a thread go out behind them and are still in flight while the
+  // code bytes of the first and the source ids of the second mini-block are requested, so the tile
+  // and the chain arrive together instead of one after the other.
   int eb0 = 0, ne0 = 0;      // mini-block g
   int eb1 = 0, ne1 = 0;      // g + 1
   int64_t Ireg = 0;
+  CW Creg = {};
   int64_t g_first = -2;
   if (K_FITS_ONE_PASS && stage_codebook_vec_ok(a.codebooks, a.w, tile_cols)) {
-    float4 cbv[8];
-    stage_codebook_load<kThreads>(cbv, a.codebooks, a.K, a.w, tile, tile_cols);
     if (threadIdx.x == 0) *s_next = kWaves;   // chunks 0 .. 15 are the waves' first ones
+    int64_t e0 = 0;
     if (has_rows) {
       issue_P(base_cur);
       park_P(0);
-      if (n_mini > 0) {
-        bounds(0, 0, eb1, ne1);
-        const int64_t e0 = chunk_e0(0);
-        const bool on = ne1 <= kWEdges && lane < ne1;
-        const Idx* src = on ? indices + e0 + eb1 + lane : indptr;
-        Ireg = (int64_t)*src;
-        g_first = -1;
-      }
+      bounds(0, 0, eb0, ne0);
+      e0 = chunk_e0(0);
+    }
+    bool on = has_rows && ne0 <= kWEdges && lane < ne0;
+    {
+      const Idx* src = on ? indices + e0 + eb0 + lane : indptr;
+      Ireg = (int64_t)*src;                                   // I(0)
+    }
+    float4 cbv[8];
+    stage_codebook_load<kThreads>(cbv, a.codebooks, a.K, a.w, tile, tile_cols);
+    {
+      const uint64_t raw = (uint64_t)Ireg;
+      const uint32_t id = (raw >> 32) ? n_last : ((uint32_t)raw < n_last ? (uint32_t)raw : n_last);
+      Creg = *reinterpret_cast<const CW*>(code_base + (uint64_t)(on ? id : 0u) * (uint32_t)a.n_cb);   // C(0)
+    }
+    {
+      const bool v = has_rows && 1 < n_mini;
+      if (v) bounds(0, 1, eb1, ne1);
+      on = v && ne1 <= kWEdges && lane < ne1;
+      const Idx* src = on ? indices + e0 + eb1 + lane : indptr;
+      Ireg = (int64_t)*src;                                   // I(1)
     }
     stage_codebook_store<kThreads, H == 2>(s_cb, cbv, a.K);
     __syncthreads();
     if (!has_rows) return;
+    g_first = 0;
   } else {
     stage_codebook_tile<kThreads, H == 2>(s_cb, a.codebooks, a.K, a.w, tile, tile_cols);
     if (threadIdx.x == 0) *s_next = kWaves;
@@ -423,7 +448,6 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     issue_P(base_cur);
     park_P(0);
   }
-  CW Creg = {};
   // The two 16-byte stores of a lane and step are issued where the results are ready, at the end of
   // the step, back to back from one base register.  In the direct (not LDS-staged) form they are
   // the two halves of the lane's 32 bytes, and they have to reach the L1 together: issued a few
