@@ -270,12 +270,12 @@ __global__ __launch_bounds__(kThreads) void vq_pipe_kernel(VqArgs a, const Idx* 
 // pipeline, with wave-private staging in LDS.  After the codebook is staged no workgroup barrier
 // is left: a wave that waits for its loads does not hold the other fifteen, and the LDS
 // operations of one wave execute in order, so its own stage hand-overs need no synchronisation.
-// A wave takes chunks of 16 consecutive destination rows from its workgroup's range (dealt through
+// A wave takes chunks of 12 consecutive destination rows from its workgroup's range (dealt through
 // a counter in LDS) and walks them as mini-blocks of RPM rows (<= 64 edges: one edge per lane in the
 // I and C stages; larger ones are summed straight from HBM).  RPM follows the average degree: 4 up
 // to 15 edges per row, and 2 or 1 above, where the lane groups left over in a pass share a row's
 // edges and add their partial sums:
-//     P  the 17 row offsets of a chunk     one load per chunk, issued while the previous chunk
+//     P  the 13 row offsets of a chunk     one load per chunk, issued while the previous chunk
 //                                          starts, parked half a chunk later (two LDS buffers)
 //     I  source id of edge `lane`          issued two mini-blocks ahead, stays in the register
 //     C  code bytes of edge `lane`         issued one mini-block ahead, parked in LDS when due
@@ -284,9 +284,9 @@ __global__ __launch_bounds__(kThreads) void vq_pipe_kernel(VqArgs a, const Idx* 
 // block-synchronous version of this kernel.
 constexpr int kWRows = 4;
 constexpr int kWEdges = 64;
-constexpr int kWMini = 4;                     // 4-row mini-blocks per chunk
+constexpr int kWMini = 3;                     // 4-row mini-blocks per chunk
 constexpr int kWChunk = kWRows * kWMini;      // rows per chunk
-constexpr int kWPtr = 56;                     // ints per offset buffer: [0..16] offsets, [52..53] first edge, [55] of the first buffer: next chunk
+constexpr int kWPtr = 56;                     // ints per offset buffer: [0..12] offsets, [52..53] first edge, [55] of the first buffer: next chunk
 
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
@@ -321,14 +321,16 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   }
   const int tile_cols = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
 
-  // A workgroup owns one contiguous range of rows, cut into chunks of 16 rows.  The waves deal the
+  // A workgroup owns one contiguous range of rows, cut into chunks of 12 rows.  The waves deal the
   // chunks among themselves through a counter in LDS: wave w starts with chunk w and takes the next
   // free one whenever it starts a chunk (the one after the chunk it is working on, so that its row
   // offsets and source ids are loaded a chunk ahead).  With equal fixed shares the oldest wave of
   // each SIMD, which the hardware serves first, finished 25 % earlier than the youngest and the CU
   // ran its last quarter with ever fewer waves (16 x 8 codebooks: waves 0-3 done at 69 us, 12-15 at
-  // 92 us); uneven degrees add to that.
-  // A launch too small to give every wave a 16-row chunk is cut into one piece per wave instead
+  // 92 us); uneven degrees add to that.  Twelve rows (three 4-row mini-blocks) is the smallest chunk
+  // whose offsets can still be requested a chunk ahead with two offset buffers; the tail of a
+  // workgroup is one chunk long (16 rows: 79.3 us, 12 rows: 77.8 us at that shape).
+  // A launch too small to give every wave a 12-row chunk is cut into one piece per wave instead
   // (nothing is left to deal then, and no wave walks four mini-blocks while others idle).
   const int64_t wg_share = (a.R + a.n_stripes - 1) / a.n_stripes;
   const bool dealt = wg_share >= (int64_t)kWaves * kWChunk;
