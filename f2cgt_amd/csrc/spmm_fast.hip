@@ -17,6 +17,7 @@
 #include "spmm_fast.hpp"
 
 #include <cstdlib>
+#include <cstring>
 
 namespace f2cgt {
 namespace {
@@ -280,6 +281,10 @@ struct AccArgs {
   int64_t R, E, N;
   int src_dim, feat_dim;
   int rows_per_block;  // destination rows per workgroup
+#ifdef F2CGT_EXPERIMENTS
+  int64_t n_first;     // workgroups [0, n_first) take rows_per_block rows, the ones after them rows_tail
+  int rows_tail;
+#endif
   int sub_rows;        // rows that go through the accumulators at a time
   int edge_batch;
   int eff_bytes;     // leading bytes of a code row that hold output columns
@@ -292,7 +297,20 @@ struct AccArgs {
   int fin_slots;     // finalize: rows per pass
   uint32_t fin_magic;  // ceil(2^16 / fin_group)
   int nt_out;        // output larger than the last-level cache: non-temporal stores
+#ifdef F2CGT_EXPERIMENTS
+  unsigned long long* trace;   // 8 words per workgroup: time stamps of its phases (100 MHz) and where it ran
+#endif
 };
+
+#ifdef F2CGT_EXPERIMENTS
+unsigned long long* g_acc_trace = nullptr;
+#define ACC_STAMP(a, slot)                                                                  \
+  do {                                                                                      \
+    if ((a).trace && threadIdx.x == 0) (a).trace[(size_t)blockIdx.x * 8 + (slot)] = wall_clock64(); \
+  } while (0)
+#else
+#define ACC_STAMP(a, slot) do {} while (0)
+#endif
 
 template <int TB, int BITS>
 __device__ __forceinline__ void acc_direct_block(const AccArgs& a, const int* s_ptr, int64_t e0, int64_t row0,
@@ -491,10 +509,12 @@ __device__ __forceinline__ void acc_block(const AccArgs& a, const FinParams& fir
     acc_tag<TB>(a, s_ptr, nrows, 0, ne, e0, indices, s_edge);
     acc_zero<TB>(s_acc, (nrows < sub ? nrows : sub) * pitch);
     __syncthreads();
+    ACC_STAMP(a, 2);
     for (int sb = 0; sb < nrows; sb += sub) {
       const int nr = (nrows - sb) < sub ? (nrows - sb) : sub;
       acc_gather<TB, BITS, NW>(a, s_acc, s_edge, s_ptr[sb], s_ptr[sb + nr], sb, pitch);
       __syncthreads();
+      if (sb == 0) ACC_STAMP(a, 3);
       acc_finalize<TB, BITS, NW>(a, first, s_acc, s_rdeg, row0, sb, nr, pitch, out);
       if (sb + sub < nrows) {
         __syncthreads();
@@ -535,8 +555,17 @@ __global__ __launch_bounds__(TB) void sq_affine_acc_kernel(AccArgs a, const Idx*
   uint2* s_edge = reinterpret_cast<uint2*>(s_wflag + 4);          // [edge_batch]
 
   const int t = threadIdx.x;
+  ACC_STAMP(a, 0);
+#ifdef F2CGT_EXPERIMENTS
+  const bool tail_block = (int64_t)blockIdx.x >= a.n_first;
+  const int row_cap = tail_block ? a.rows_tail : a.rows_per_block;
+  const int64_t row0 = tail_block ? a.n_first * a.rows_per_block + ((int64_t)blockIdx.x - a.n_first) * a.rows_tail
+                                  : (int64_t)blockIdx.x * a.rows_per_block;
+#else
+  const int row_cap = a.rows_per_block;
   const int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block;
-  const int nrows = (int)((a.R - row0) < a.rows_per_block ? (a.R - row0) : a.rows_per_block);
+#endif
+  const int nrows = (int)((a.R - row0) < row_cap ? (a.R - row0) : row_cap);
   const FinParams first = acc_fin_params(a);
   int64_t e0 = (int64_t)indptr[row0];
   e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
@@ -559,6 +588,7 @@ __global__ __launch_bounds__(TB) void sq_affine_acc_kernel(AccArgs a, const Idx*
     if ((t & (kWave - 1)) == 0) s_wflag[t / kWave] = wl;
   }
   __syncthreads();
+  ACC_STAMP(a, 1);
   uint32_t block_level = 0;
 #pragma unroll
   for (int w = 0; w < TB / kWave; ++w) block_level |= s_wflag[w];
@@ -573,6 +603,13 @@ __global__ __launch_bounds__(TB) void sq_affine_acc_kernel(AccArgs a, const Idx*
     acc_block<TB, BITS, 4, Idx>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
   else
     acc_block<TB, BITS, 2, Idx>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
+  ACC_STAMP(a, 4);
+#ifdef F2CGT_EXPERIMENTS
+  if (a.trace && threadIdx.x == 0) {
+    a.trace[(size_t)blockIdx.x * 8 + 5] = __builtin_amdgcn_s_getreg((31 << 11) | 4);    // HW_ID
+    a.trace[(size_t)blockIdx.x * 8 + 6] = __builtin_amdgcn_s_getreg((31 << 11) | 20);   // XCC_ID
+  }
+#endif
 }
 
 #ifdef F2CGT_EXPERIMENTS
@@ -733,6 +770,9 @@ int launch_acc_tb(AccArgs a, size_t lds, int64_t grid, const void* indptr, const
   a.fin_slots = TB / a.fin_group;
   a.fin_magic = (uint32_t)((65536 + a.fin_group - 1) / a.fin_group);
   a.nt_out = stream_output(a.R * (int64_t)a.feat_dim * 4) ? 1 : 0;
+#ifdef F2CGT_EXPERIMENTS
+  a.trace = g_acc_trace;
+#endif
   if (plan_only()) {
     plan_record("sq_affine_acc_kernel", grid, TB, (int64_t)lds, a.rows_per_block, a.fin_slots, TB >> a.lane_shift,
                 a.sub_rows, a.edge_batch);
@@ -786,11 +826,30 @@ int launch_acc_sized(AccArgs a, double dg, size_t acc_row, const void* indptr, c
     const int want = atoi(v);
     if (want >= 8) { sub = want / 8 * 8; rb = sub; }
   }
+  if (const char* v = getenv("F2CGT_ACC_SUB")) {   // rows through the accumulators at a time; F2CGT_ACC_RB then a multiple of it
+    const int want = atoi(v);
+    const char* r = getenv("F2CGT_ACC_RB");
+    if (want >= 8 && r) { sub = want / 8 * 8; rb = atoi(r) / sub * sub; if (rb < sub) rb = sub; }
+  }
 #endif
   a.rows_per_block = rb;
   a.sub_rows = sub;
   const size_t lds = sub * acc_row + (size_t)(rb + 4) * 4 + (size_t)rb * 4 + 16 + (size_t)a.edge_batch * 8 + 16;
-  const int64_t grid = ceil_div(a.R, rb);
+  int64_t grid = ceil_div(a.R, rb);
+#ifdef F2CGT_EXPERIMENTS
+  a.n_first = grid;
+  a.rows_tail = rb;
+  if (const char* v = getenv("F2CGT_ACC_TAIL")) {   // "<n_first>:<rows_tail>"
+    const long long nf = atoll(v);
+    const char* c = strchr(v, ':');
+    const int rt = c ? atoi(c + 1) / 8 * 8 : 0;
+    if (nf > 0 && nf < grid && rt >= 8 && rt <= rb) {
+      a.n_first = nf;
+      a.rows_tail = rt;
+      grid = nf + ceil_div(a.R - nf * rb, rt);
+    }
+  }
+#endif
   if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
   return launch_acc_tb<TB, BITS>(a, lds, grid, indptr, indices, idx_dtype, out, st, what);
 }
@@ -1511,3 +1570,9 @@ int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float*
 }
 
 }  // namespace f2cgt
+
+#ifdef F2CGT_EXPERIMENTS
+// Experiments build only: device buffer of 8 x 64-bit words per workgroup that sq_affine_acc_kernel
+// fills with the time stamps of its phases; nullptr switches it off.
+extern "C" void f2cgt_experiment_set_acc_trace(unsigned long long* device_buffer) { f2cgt::g_acc_trace = device_buffer; }
+#endif

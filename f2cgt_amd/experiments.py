@@ -1,0 +1,120 @@
+"""Time-stamp traces of two kernels, for the library built with `python -m f2cgt_amd.build --experiments`
+(the shipped build has neither the time-stamped kernel forms nor the entry points used here).
+
+    python3 -m f2cgt_amd.experiments wave-age c3|c5      per-wave start / first step / end of vq_wave_kernel
+    python3 -m f2cgt_amd.experiments block-phases c1|c2  per-workgroup phase times of sq_affine_acc_kernel
+
+Both run the workload of `bench.py --workload <w>` warm, switch the trace buffer on for a few launches and
+print percentiles of the last one (times in us from the earliest stamp of the launch; the stamps are
+`wall_clock64()`, 100 MHz).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _q(x):
+    return " ".join("%7.2f" % v for v in np.percentile(x, [0, 5, 25, 50, 75, 95, 100]))
+
+
+def _setup(name):
+    import torch
+
+    sys.path.insert(0, ROOT)
+    import bench
+    from f2cgt_amd import capi, synth
+
+    lib = capi.lib()
+    wl = synth.WORKLOADS[name](device="cuda", idx_dtype=torch.int64)
+    out = torch.empty((wl["R"], wl["feat_dim"]), dtype=torch.float32, device="cuda")
+    return torch, lib, wl, bench._launcher(capi, wl, out), out
+
+
+def wave_age(name):
+    os.environ["F2CGT_VQ_DEFER"] = "9"   # selects the time-stamped form of vq_wave_kernel
+    torch, lib, wl, step, _ = _setup(name)
+    if not hasattr(lib, "f2cgt_experiment_set_trace"):
+        raise SystemExit("the library in tree was built without --experiments")
+    lib.f2cgt_experiment_set_trace.argtypes = [ctypes.c_void_p]
+    lib.f2cgt_experiment_set_trace.restype = None
+    trace = torch.zeros((4096 * 4,), dtype=torch.int64, device="cuda")   # 256 workgroups x 16 waves x 4 words
+    for _ in range(50):
+        step()
+    torch.cuda.synchronize()
+    lib.f2cgt_experiment_set_trace(ctypes.c_void_p(trace.data_ptr()))
+    for _ in range(20):
+        step()
+    torch.cuda.synchronize()
+    lib.f2cgt_experiment_set_trace(None)
+    full = trace.cpu().numpy().reshape(-1, 4).astype(np.float64)
+    valid = full[:, 2] > 0
+    t = full[valid]
+    t0 = t[:, 0].min()
+    start, first, end = (t[:, 0] - t0) / 100.0, (t[:, 1] - t0) / 100.0, (t[:, 2] - t0) / 100.0
+    print(name, "waves with rows:", len(t), " steps per wave: %d .. %d" % (t[:, 3].min(), t[:, 3].max()))
+    print("  percentiles                0      5     25     50     75     95    100")
+    print("  wave start us        :", _q(start))
+    print("  first step us        :", _q(first))
+    print("  wave end us          :", _q(end))
+    print("  busy fraction of the wave slots (mean wave lifetime / launch): %.3f" % ((end - start).mean() / end.max()))
+    ends = np.where(valid, (full[:, 2] - t0) / 100.0, np.nan).reshape(-1, 16)
+    rows = ~np.isnan(ends).all(axis=1)
+    wg_end, wg_min = np.nanmax(ends[rows], axis=1), np.nanmin(ends[rows], axis=1)
+    print("  workgroup end us     :", _q(wg_end))
+    print("  spread in a workgroup:", _q(wg_end - wg_min))
+    print("  mean end by wave index in the workgroup:", " ".join("%.0f" % v for v in np.nanmean(ends[rows], axis=0)))
+    for x in range(8):
+        sub = ends[x::8]
+        sub = sub[~np.isnan(sub).all(axis=1)]
+        print("   workgroups with id %% 8 == %d (one XCD): mean wave end %.1f, last %.1f" % (x, np.nanmean(sub), np.nanmax(sub)))
+
+
+def block_phases(name):
+    torch, lib, wl, step, _ = _setup(name)
+    if not hasattr(lib, "f2cgt_experiment_set_acc_trace"):
+        raise SystemExit("the library in tree was built without --experiments")
+    lib.f2cgt_experiment_set_acc_trace.argtypes = [ctypes.c_void_p]
+    lib.f2cgt_experiment_set_acc_trace.restype = None
+    trace = torch.zeros((65536 * 8,), dtype=torch.int64, device="cuda")   # 8 words per workgroup
+    for _ in range(3000):
+        step()
+    torch.cuda.synchronize()
+    lib.f2cgt_experiment_set_acc_trace(ctypes.c_void_p(trace.data_ptr()))
+    for _ in range(50):
+        step()
+    torch.cuda.synchronize()
+    lib.f2cgt_experiment_set_acc_trace(None)
+    t = trace.cpu().numpy().reshape(-1, 8)
+    t = t[t[:, 4] > 0].astype(np.float64)
+    T = (t[:, :5] - t[:, 0].min()) / 100.0
+    print(name, "workgroups:", len(t), " launch length %.2f us (first stamp to last)" % T[:, 4].max())
+    print("  percentiles                        0      5     25     50     75     95    100")
+    print("  workgroup start us           :", _q(T[:, 0]))
+    print("  workgroup end us             :", _q(T[:, 4]))
+    print("  workgroup duration us        :", _q(T[:, 4] - T[:, 0]))
+    print("  phase: row offsets           :", _q(T[:, 1] - T[:, 0]))
+    print("  phase: source ids and tags   :", _q(T[:, 2] - T[:, 1]))
+    print("  phase: gather of the code rows:", _q(T[:, 3] - T[:, 2]))
+    print("  phase: finalize and store    :", _q(T[:, 4] - T[:, 3]))
+    for lo in np.arange(0.0, T[:, 4].max(), 1.0):
+        hi = lo + 1.0
+        print("  t = %2.0f .. %2.0f us: %5d workgroups resident, %5d started, %5d ended"
+              % (lo, hi, ((T[:, 0] < hi) & (T[:, 4] > lo)).sum(), ((T[:, 0] >= lo) & (T[:, 0] < hi)).sum(),
+                 ((T[:, 4] >= lo) & (T[:, 4] < hi)).sum()))
+    hw, xcc = t[:, 5].astype(np.int64), t[:, 6].astype(np.int64) & 0xf
+    key = xcc * 4096 + ((hw >> 13) & 7) * 512 + ((hw >> 12) & 1) * 16 + ((hw >> 8) & 0xf)
+    _, count = np.unique(key, return_counts=True)
+    print("  distinct CUs: %d, workgroups per CU min / mean / max: %d / %.1f / %d" % (len(count), count.min(), count.mean(), count.max()))
+
+
+if __name__ == "__main__":
+    if len(sys.argv) != 3 or sys.argv[1] not in ("wave-age", "block-phases"):
+        print(__doc__)
+        sys.exit(2)
+    (wave_age if sys.argv[1] == "wave-age" else block_phases)(sys.argv[2])
