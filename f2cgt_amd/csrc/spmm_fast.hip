@@ -867,6 +867,12 @@ int launch_acc(AccArgs a, const void* indptr, const void* indices, int idx_dtype
   const int skew = lanes2 % 32;
   a.pitch_n = ((4 * a.lanes + 31) / 32 * 32 + skew + 3) & ~3;
   a.pitch_w = ((8 * a.lanes + 31) / 32 * 32 + skew + 3) & ~3;
+#ifdef F2CGT_EXPERIMENTS
+  if (getenv("F2CGT_ACC_PITCH")) {   // rows packed: the 64 banks spread them as long as the pitch is not a multiple of 16 words
+    a.pitch_n = 4 * a.lanes + ((4 * a.lanes) % 16 == 0 ? 4 : 0);
+    a.pitch_w = 8 * a.lanes + ((8 * a.lanes) % 16 == 0 ? 4 : 0);
+  }
+#endif
   a.f4_per_row = a.feat_dim / 4;
   const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 1.0;
   const double dg = avg_deg > 0.5 ? avg_deg : 0.5;
