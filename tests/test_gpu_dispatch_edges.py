@@ -1,4 +1,4 @@
-"""Shapes on either side of the thresholds that pick a workgroup size: the two-table kernel runs
+"""Shapes on either side of the thresholds that pick a workgroup size or a row partition: the two-table kernel runs
 one wave per workgroup at 8-32 edges per row and up to 128 columns and 256 threads otherwise, the
 staged-rows kernel of the log-domain SQ runs 128 threads for 1/2-bit rows and 256 for 4/8-bit
 ones.  Every side of every threshold must give the oracle's result."""
@@ -101,3 +101,70 @@ def test_fused_sq_on_both_sides_of_the_rows_per_block_steps(rows):
     np.add.at(sums, np.repeat(np.arange(rows), deg), dec[indices].astype(np.float64))
     want = (sums / np.maximum(deg, 1)[:, None]).astype(np.float32)
     assert np.allclose(got.cpu().numpy(), want, rtol=RTOL, atol=RTOL * np.abs(dec).max())
+
+
+@pytest.mark.parametrize("mean_deg", [22, 45])
+def test_fused_vq_chunk_dealing_with_shared_rows(mean_deg):
+    """Above 15 edges per row on average the lane groups of a pass share a row (two or one row per
+    mini-block); the same chunk dealing, sums no longer in edge order: rtol 1e-5."""
+    rng = np.random.default_rng(mean_deg)
+    rows, n_src, n_cb, width, feat_dim = 256 * 200 + 9, 20000, 16, 8, 128
+    codes = rng.integers(0, 256, size=(n_src, n_cb), dtype=np.uint8)
+    cbs = rng.standard_normal((n_cb, 256, width)).astype(np.float32)
+    deg = rng.integers(0, 2 * mean_deg + 1, size=rows)
+    indptr = np.zeros(rows + 1, dtype=np.int64)
+    indptr[1:] = np.cumsum(deg)
+    indices = rng.integers(0, n_src, size=int(indptr[-1]))
+    got = capi.vq_decompress_spmm_csr(dev(codes), dev(cbs), dev(indptr), dev(indices), feat_dim)
+    full = capi.spmm_csr(capi.vq_decompress(dev(codes), dev(cbs), feat_dim), dev(indptr), dev(indices))
+    torch.cuda.synchronize()
+    scale = float(full.abs().max())
+    assert torch.allclose(got, full, rtol=RTOL, atol=RTOL * scale)
+    sample = np.unique(np.concatenate([np.arange(30), np.arange(rows - 30, rows), rng.integers(0, rows, size=200)]))
+    sub_ptr = np.zeros(len(sample) + 1, dtype=np.int64)
+    sub_ptr[1:] = np.cumsum(deg[sample])
+    sub_idx = np.concatenate([indices[indptr[r]:indptr[r + 1]] for r in sample]).astype(np.int64)
+    want = oc.vq_decompress_spmm_csr(codes, cbs, sub_ptr, sub_idx, feat_dim)
+    assert np.allclose(got.cpu().numpy()[sample], want, rtol=RTOL, atol=RTOL * np.abs(want).max())
+
+
+@pytest.mark.parametrize("idx", [np.int64, np.int32])
+@pytest.mark.parametrize("rows", [256 * 191 + 3, 256 * 192, 256 * 192 + 1, 256 * 205 + 7, 256 * 12 * 17 + 5])
+def test_fused_vq_on_both_sides_of_the_chunk_dealing_threshold(rows, idx):
+    """The fused VQ kernel gives every wave one piece of its workgroup's rows while a workgroup has
+    fewer than 16 x 12 rows and deals 12-row chunks among the waves from there on: row counts on
+    either side of that step, last chunks of one to twelve rows, empty rows, and rows with more
+    edges than a wave stages (summed straight from memory).  Edge order is kept, so the result is the
+    oracle's bit for bit."""
+    rng = np.random.default_rng(rows % 100003)
+    n_src, n_cb, width, feat_dim = 20000, 16, 8, 128
+    codes = rng.integers(0, 256, size=(n_src, n_cb), dtype=np.uint8)
+    cbs = rng.standard_normal((n_cb, 256, width)).astype(np.float32)
+    deg = rng.integers(0, 11, size=rows)
+    heavy = rng.integers(0, rows, size=40)
+    deg[heavy] = rng.integers(65, 120, size=40)          # more than the 64 staged edges of a mini-block
+    deg[rng.integers(0, rows, size=rows // 20)] = 0
+    indptr = np.zeros(rows + 1, dtype=idx)
+    indptr[1:] = np.cumsum(deg)
+    indices = rng.integers(0, n_src, size=int(indptr[-1])).astype(idx)
+    got = capi.vq_decompress_spmm_csr(dev(codes), dev(cbs), dev(indptr), dev(indices), feat_dim)
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    tag = capi.DT_I64 if idx == np.int64 else capi.DT_I32
+    rc, plan = capi.dry_run("f2cgt_vq_decompress_spmm_csr", 16, capi.DT_U8, 16, 16, 16, tag, 16, rows, int(indptr[-1]),
+                            n_src, feat_dim, n_cb, 256, width, None)
+    assert rc == 0 and plan.kernel == b"vq_wave_kernel"
+    # the oracle on a sample of rows (first, last, around every workgroup boundary, the heavy ones)
+    per_wg = -(-rows // 256)
+    sample = np.unique(np.clip(np.concatenate([
+        np.arange(0, 40), np.arange(rows - 40, rows), heavy,
+        (np.arange(1, 256)[:, None] * (-(-per_wg // 12) * 12) + np.arange(-2, 3)[None, :]).ravel(),
+        rng.integers(0, rows, size=400)]), 0, rows - 1))
+    sub_ptr = np.zeros(len(sample) + 1, dtype=np.int64)
+    sub_ptr[1:] = np.cumsum(deg[sample])
+    sub_idx = np.concatenate([indices[indptr[r]:indptr[r + 1]] for r in sample]).astype(np.int64)
+    want = oc.vq_decompress_spmm_csr(codes, cbs, sub_ptr, sub_idx, feat_dim)
+    assert np.array_equal(got[sample], want)
+    # every row against the unfused composition on the device
+    full = capi.spmm_csr(capi.vq_decompress(dev(codes), dev(cbs), feat_dim), dev(indptr), dev(indices))
+    assert torch.equal(torch.from_numpy(got).cuda(), full)
