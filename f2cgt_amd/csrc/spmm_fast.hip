@@ -1196,7 +1196,8 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
   float* s_par = reinterpret_cast<float*>(s_acc + (size_t)a.rows_per_block * acc_pitch);  // [chunks][8]
   int* s_ptr = reinterpret_cast<int*>(s_par + (size_t)a.chunks * 8);         // [RB + 1]
   int* s_nvq = s_ptr + a.rows_per_block + 4;                                 // [RB] VQ edges per row
-  uint32_t* s_row = reinterpret_cast<uint32_t*>(s_nvq + a.rows_per_block);   // [edge_batch] table row | flag
+  uint32_t* s_mask = reinterpret_cast<uint32_t*>(s_nvq + a.rows_per_block);  // [RB][2] which of a row's first 64 edges are not in the accumulators
+  uint32_t* s_row = s_mask + 2 * a.rows_per_block;                           // [edge_batch] table row | flag
   uint16_t* s_erow = reinterpret_cast<uint16_t*>(s_row + a.edge_batch);      // [edge_batch] local row
 
   const int t = threadIdx.x;
@@ -1210,7 +1211,11 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
     s_ptr[i] = (int)(v - e0 > 0x7fffffff ? 0x7fffffff : v - e0);
   }
   for (int i = t; i < nrows * acc_pitch; i += TB) s_acc[i] = 0u;
-  for (int i = t; i < nrows; i += TB) s_nvq[i] = 0;
+  for (int i = t; i < nrows; i += TB) {
+    s_nvq[i] = 0;
+    s_mask[2 * i] = 0u;
+    s_mask[2 * i + 1] = 0u;
+  }
   for (int i = t; i < a.feat_dim; i += TB) {
     const int c4 = i >> 2, q = i & 3;
     s_par[c4 * 8 + q] = a.sq_params[i];
@@ -1235,22 +1240,23 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
         const int64_t r = -m - 1;
         v = (uint32_t)(r < a.n_vq ? r : a.n_vq - 1) | kVqFlag;
       }
-      s_row[i] = v;
-      s_erow[i] = 0;
-    }
-    __syncthreads();
-    for (int r = t; r < nrows; r += TB) {
-      int b = s_ptr[r] - eb, e = s_ptr[r + 1] - eb;
-      const bool direct = s_ptr[r + 1] - s_ptr[r] > LIMIT;
-      b = b < 0 ? 0 : b;
-      e = e > nb ? nb : e;
-      int nvq = 0;
-      for (int k = b; k < e; ++k) {
-        s_erow[k] = (uint16_t)r;
-        if (direct) s_row[k] |= 0x40000000u;  // keep out of the integer accumulators
-        nvq += (s_row[k] >> 30) != 0;
+      // the edge's destination row: the last r with s_ptr[r] <= position (empty rows share a
+      // start and are skipped that way); the same number of steps in every lane
+      const int pos = eb + i;
+      int lo = 0, hi = nrows;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (s_ptr[mid] <= pos) lo = mid; else hi = mid;
       }
-      if (e > b) s_nvq[r] += nvq;
+      const int first = s_ptr[lo];
+      if (s_ptr[lo + 1] - first > LIMIT) v |= 0x40000000u;   // rows beyond the field capacity stay out of the accumulators
+      if (v >> 30) {   // added in the epilogue, in edge order: counted, and marked among the row's first 64 edges
+        atomicAdd(s_nvq + lo, 1);
+        const int bit = pos - first;
+        if (bit >= 0 && bit < 64) atomicOr(s_mask + 2 * lo + (bit >> 5), 1u << (bit & 31));
+      }
+      s_row[i] = v;
+      s_erow[i] = (uint16_t)lo;
     }
     __syncthreads();
     if (VEC == 4) {
@@ -1354,17 +1360,7 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
       const int sub = col / a.w;
       const int off = col - sub * a.w;
       const bool in_lds = ne <= a.edge_batch;  // one batch: s_row still describes every edge of the block
-      for (int k = b; k < e; ++k) {
-        int64_t m;
-        if (in_lds) {
-          const uint32_t v = s_row[k];
-          if ((v >> 30) == 0) continue;  // SQ edge already in the integer accumulators
-          m = (v & kVqFlag) ? -(int64_t)(v & 0x3fffffffu) - 1 : (int64_t)(v & 0x3fffffffu);
-        } else {
-          const int64_t id = clamp_idx(indices[e0 + k], a.N);
-          m = (int64_t)a.row_map[id];
-          if (m >= 0 && deg <= LIMIT) continue;
-        }
+      auto add_edge = [&](int64_t m) {
         if (m >= 0) {
           const int64_t row = m < a.n_sq ? m : a.n_sq - 1;
           const uint32_t wv = codes32[row * dwords_per_row + c4];
@@ -1379,6 +1375,29 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
           code = code < a.K ? code : a.K - 1;
           const float4 x = *reinterpret_cast<const float4*>(a.vq_codebooks + ((int64_t)sub * a.K + code) * a.w + off);
           v0 += x.x; v1 += x.y; v2 += x.z; v3 += x.w;
+        }
+      };
+      if (in_lds && deg <= 64) {
+        // only the marked edges (one or two of a dozen, typically), lowest first
+        uint64_t mask = (uint64_t)s_mask[2 * r] | ((uint64_t)s_mask[2 * r + 1] << 32);
+        while (mask) {
+          const uint32_t v = s_row[b + __builtin_ctzll(mask)];
+          mask &= mask - 1;
+          add_edge((v & kVqFlag) ? -(int64_t)(v & 0x3fffffffu) - 1 : (int64_t)(v & 0x3fffffffu));
+        }
+      } else {
+        for (int k = b; k < e; ++k) {
+          int64_t m;
+          if (in_lds) {
+            const uint32_t v = s_row[k];
+            if ((v >> 30) == 0) continue;  // SQ edge already in the integer accumulators
+            m = (v & kVqFlag) ? -(int64_t)(v & 0x3fffffffu) - 1 : (int64_t)(v & 0x3fffffffu);
+          } else {
+            const int64_t id = clamp_idx(indices[e0 + k], a.N);
+            m = (int64_t)a.row_map[id];
+            if (m >= 0 && deg <= LIMIT) continue;
+          }
+          add_edge(m);
         }
       }
     }
@@ -1512,7 +1531,7 @@ int launch_hybrid(HybArgs a, const void* indptr, const void* indices, int idx_dt
   }
 #endif
   a.rows_per_block = rb;
-  const size_t lds = rb * acc_row + (size_t)a.chunks * 32 + (size_t)(rb + 4) * 4 + (size_t)rb * 4 +
+  const size_t lds = rb * acc_row + (size_t)a.chunks * 32 + (size_t)(rb + 4) * 4 + (size_t)rb * 4 + (size_t)rb * 8 +
                      (size_t)a.edge_batch * 6 + 16;
   const int64_t grid = ceil_div(a.R, rb);
   if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
