@@ -1183,18 +1183,22 @@ struct HybArgs {
 
 constexpr uint32_t kVqFlag = 0x80000000u;
 
-template <typename Idx, int VEC, int TB>
+// CH: the number of 4-column chunks per row when it is known at compile time (32 for 128 columns,
+// the common width: the accumulator offsets of the gather then fold into the instructions), else 0.
+template <typename Idx, int VEC, int TB, int CH = 0>
 __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __restrict__ indptr,
                                                             const Idx* __restrict__ indices,
                                                             float* __restrict__ out) {
   constexpr int LIMIT = 257;
+  const int chunks = CH ? CH : a.chunks;
+  const int ch2 = CH ? CH : a.ch2;   // CH is a power of two
   extern __shared__ __align__(16) unsigned char smem[];
   // integer accumulators: [RB][plane 0: bytes 0,2 | plane 1: bytes 1,3][chunk], rows 8 words apart
   // in bank space so that the lane groups of a wave (different rows) spread over all 32 banks
-  const int acc_pitch = 2 * a.chunks + 8;
+  const int acc_pitch = 2 * chunks + 8;
   uint32_t* s_acc = reinterpret_cast<uint32_t*>(smem);
   float* s_par = reinterpret_cast<float*>(s_acc + (size_t)a.rows_per_block * acc_pitch);  // [chunks][8]
-  int* s_ptr = reinterpret_cast<int*>(s_par + (size_t)a.chunks * 8);         // [RB + 1]
+  int* s_ptr = reinterpret_cast<int*>(s_par + (size_t)chunks * 8);         // [RB + 1]
   int* s_nvq = s_ptr + a.rows_per_block + 4;                                 // [RB] VQ edges per row
   uint32_t* s_mask = reinterpret_cast<uint32_t*>(s_nvq + a.rows_per_block);  // [RB][2] which of a row's first 64 edges are not in the accumulators
   uint32_t* s_row = s_mask + 2 * a.rows_per_block;                           // [edge_batch] table row | flag
@@ -1261,7 +1265,7 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
     __syncthreads();
     if (VEC == 4) {
       // a lane takes 16 bytes (4 chunks) of an edge's code row: chunks / 4 lanes per edge
-      const int lanes = a.ch2 >> 2;
+      const int lanes = ch2 >> 2;
       const int j = t & (lanes - 1);
       const int gslot = t / lanes;
       const int gslots = TB / lanes;
@@ -1273,7 +1277,7 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
       const int per = (nb + gslots - 1) / gslots;
       const int e_begin = gslot * per;
       const int e_end = (e_begin + per) < nb ? (e_begin + per) : nb;
-      const int q = a.chunks >> 2;   // dwords per lane stride (chunks is a multiple of 4 here)
+      const int q = chunks >> 2;   // dwords per lane stride (chunks is a multiple of 4 here)
       const bool lane_on = j < q;
       for (int e = e_begin; e < e_end; e += U) {
         uint32_t w[U][4];
@@ -1299,16 +1303,17 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
             uint32_t* acc = s_acc + er[u] * acc_pitch + j;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-              atomicAdd(acc + c * q, w[u][c] & 0x00ff00ffu);
-              atomicAdd(acc + a.chunks + c * q, (w[u][c] >> 8) & 0x00ff00ffu);
+              // bytes 0 and 2, then bytes 1 and 3, each widened to a 16-bit field
+              atomicAdd(acc + c * q, __builtin_amdgcn_perm(0u, w[u][c], 0x0c020c00u));
+              atomicAdd(acc + chunks + c * q, __builtin_amdgcn_perm(0u, w[u][c], 0x0c030c01u));
             }
           }
         }
       }
     } else {
-    const int j = t & (a.ch2 - 1);
-    const int gslot = t / a.ch2;
-    const int gslots = TB / a.ch2;
+    const int j = t & (ch2 - 1);
+    const int gslot = t / ch2;
+    const int gslots = TB / ch2;
     constexpr int U = 4;
     for (int e = gslot; e < nb; e += gslots * U) {
       uint32_t w[U], row[U], er[U];
@@ -1319,15 +1324,15 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
         row[u] = s_row[ee];
         er[u] = s_erow[ee];
         w[u] = 0;
-        if (j < a.chunks && (row[u] >> 30) == 0) w[u] = codes32[(int64_t)row[u] * dwords_per_row + j];
+        if (j < chunks && (row[u] >> 30) == 0) w[u] = codes32[(int64_t)row[u] * dwords_per_row + j];
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int ee = e + u * gslots;
-        if (ee < nb && j < a.chunks && (row[u] >> 30) == 0) {
+        if (ee < nb && j < chunks && (row[u] >> 30) == 0) {
           uint32_t* acc = s_acc + er[u] * acc_pitch + j;
-          atomicAdd(acc, w[u] & 0x00ff00ffu);
-          atomicAdd(acc + a.chunks, (w[u] >> 8) & 0x00ff00ffu);
+          atomicAdd(acc, __builtin_amdgcn_perm(0u, w[u], 0x0c020c00u));
+          atomicAdd(acc + chunks, __builtin_amdgcn_perm(0u, w[u], 0x0c030c01u));
         }
       }
     }
@@ -1335,16 +1340,16 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
   }
   __syncthreads();
   // finalize: lane <-> one float4 of the block's contiguous output span
-  const int items = nrows * a.chunks;
+  const int items = nrows * chunks;
   float* ob = out + row0 * (int64_t)a.feat_dim;
   for (int it = t; it < items; it += TB) {
-    const int r = (int)__umulhi((uint32_t)it, a.magic);
-    const int c4 = it - r * a.chunks;
+    const int r = CH ? it / CH : (int)__umulhi((uint32_t)it, a.magic);
+    const int c4 = it - r * chunks;
     uint2 q;
     // (the 16-byte gather stores dword c4 of a row at word (c4 % 4) * chunks / 4 + c4 / 4)
-    const int pos = VEC == 4 ? (c4 & 3) * (a.chunks >> 2) + (c4 >> 2) : c4;
+    const int pos = VEC == 4 ? (c4 & 3) * (chunks >> 2) + (c4 >> 2) : c4;
     q.x = s_acc[r * acc_pitch + pos];
-    q.y = s_acc[r * acc_pitch + a.chunks + pos];
+    q.y = s_acc[r * acc_pitch + chunks + pos];
     const int b = s_ptr[r], e = s_ptr[r + 1];
     const int deg = e - b;
     const int nvq = s_nvq[r];
@@ -1546,10 +1551,12 @@ int launch_hybrid(HybArgs a, const void* indptr, const void* indices, int idx_dt
   const int64_t* ip64 = static_cast<const int64_t*>(indptr);
   const int64_t* ix64 = static_cast<const int64_t*>(indices);
   if (idx_dtype == F2CGT_DT_I32) {
-    if (vec4) hybrid_acc_kernel<int32_t, 4, TB><<<(unsigned)grid, TB, lds, st>>>(a, ip32, ix32, out);
+    if (vec4 && a.chunks == 32) hybrid_acc_kernel<int32_t, 4, TB, 32><<<(unsigned)grid, TB, lds, st>>>(a, ip32, ix32, out);
+    else if (vec4) hybrid_acc_kernel<int32_t, 4, TB><<<(unsigned)grid, TB, lds, st>>>(a, ip32, ix32, out);
     else hybrid_acc_kernel<int32_t, 1, TB><<<(unsigned)grid, TB, lds, st>>>(a, ip32, ix32, out);
   } else {
-    if (vec4) hybrid_acc_kernel<int64_t, 4, TB><<<(unsigned)grid, TB, lds, st>>>(a, ip64, ix64, out);
+    if (vec4 && a.chunks == 32) hybrid_acc_kernel<int64_t, 4, TB, 32><<<(unsigned)grid, TB, lds, st>>>(a, ip64, ix64, out);
+    else if (vec4) hybrid_acc_kernel<int64_t, 4, TB><<<(unsigned)grid, TB, lds, st>>>(a, ip64, ix64, out);
     else hybrid_acc_kernel<int64_t, 1, TB><<<(unsigned)grid, TB, lds, st>>>(a, ip64, ix64, out);
   }
   return launch_status(what);
