@@ -10,6 +10,18 @@ average launch duration measured with HIP events on the launch stream; `cpu_base
 is the reference's unfused CPU flow (torch dequantise + torch sparse mm) timed on this
 box's host cores on a bounded sample of the same workload.
 
+Every benchmark configuration is in that one line: next to the headline workload's `roofline`,
+`configs` holds the other fused workloads (C1, C3, C3 with scattered ids, C4, C5) and the C5 encode
+step, each with its own launch count, `launch_us`, `edges_per_s`, `algorithmic_bytes`,
+`compulsory_bytes`, measured HBM `traffic` and three fractions of the 8 TB/s peak:
+`frac_algorithmic` (every edge charged its source row), `frac_compulsory` (every distinct source
+row charged once: a bound no cache can beat, so it cannot exceed 1) and `frac`, which is
+`min(frac_algorithmic, 1)` when the launch really moves >= 0.9 of the algorithmic bytes through
+HBM and `frac_compulsory` otherwise.  The headline's `roofline.frac_cold` is the same kernel
+with six CSC blocks and six outputs in rotation (> 600 MB pass before a buffer comes round again,
+more than the 256 MB last-level cache).  `--workload X` measures X alone (what the rocprofv3
+runs use); `--configs off` drops the extra objects.
+
     python bench.py --all            adds the other workloads and the streaming/encode ops
                                      under "others" (same JSON line)
     python bench.py --calibrate-copy runs plain device copies of a known size (for scaling the
@@ -110,6 +122,83 @@ def _run_workload(name, idx, steps, warmup):
     out = torch.empty((wl["R"], wl["feat_dim"]), dtype=torch.float32, device="cuda")
     ms_step, ms_launch = _time_steps(_launcher(capi, wl, out), steps, warmup)
     return wl, ms_step, ms_launch
+
+
+def _fractions(wl, launch_ms, traffic):
+    """The three fractions of the HBM peak for one fused launch (see the module docstring)."""
+    from f2cgt_amd import synth
+
+    secs = launch_ms * 1e-3
+    algo, comp = wl["algo_bytes"], synth.compulsory_bytes(wl)
+    f_algo = algo / secs / 1e9 / HBM_PEAK_GBS
+    f_comp = comp / secs / 1e9 / HBM_PEAK_GBS
+    # how much of the algorithmic bytes really moves: the measured traffic where there is a figure
+    # for these kernel sources, else what the distinct rows say
+    moved = (traffic if traffic is not None else comp) / algo
+    frac = min(f_algo, 1.0) if moved >= 0.9 else f_comp
+    return {"algorithmic_bytes": algo, "compulsory_bytes": comp, "traffic": traffic,
+            "frac_algorithmic": f_algo, "frac_compulsory": f_comp, "frac": frac}
+
+
+def _cold_launch_ms(name, idx, wl, blocks=6, rounds=40, warm_rounds=10):
+    """Launch time with `blocks` CSC blocks and as many outputs in rotation: between two uses of
+    the same graph or output buffer the other launches write blocks-1 whole outputs, so neither
+    is still in the last-level cache (the tables' hot rows are, as they are in use)."""
+    import torch
+    from f2cgt_amd import capi, synth
+
+    graphs = [wl] + synth.extra_blocks(wl, blocks - 1)
+    steps = []
+    for g in graphs:
+        out = torch.empty((g["R"], g["feat_dim"]), dtype=torch.float32, device="cuda")
+        steps.append(_launcher(capi, g, out))
+
+    def one_round():
+        for st in steps:
+            st()
+
+    _, ms = _time_steps(one_round, rounds, warm_rounds)
+    algo = sum(g["algo_bytes"] for g in graphs) / len(graphs)
+    return ms / len(graphs), algo, len(graphs)
+
+
+# the other configurations in the default line: (workload, timed launches, warm-up launches, scattered ids)
+CONFIG_RUNS = (("c1", 2000, 2000, False), ("c3", 300, 300, False), ("c3", 300, 300, True),
+               ("c4", 100, 100, False), ("c5", 60, 60, False))
+
+
+def _configs(idx):
+    import torch
+    from f2cgt_amd import capi, synth
+
+    idx_dtype = torch.int64 if idx == "int64" else torch.int32
+    res = {}
+    for name, steps, warmup, scattered in CONFIG_RUNS:
+        key = name + ("_scattered" if scattered else "")
+        try:        # a failure here is reported in its entry; the headline line is printed regardless
+            wl = synth.WORKLOADS[name](device="cuda", idx_dtype=idx_dtype)
+            if scattered:
+                wl = synth.scatter_ids(wl)
+            key = wl["name"]
+            out = torch.empty((wl["R"], wl["feat_dim"]), dtype=torch.float32, device="cuda")
+            ms_step, ms_launch = _time_steps(_launcher(capi, wl, out), steps, warmup)
+            entry = {"steps": steps, "warmup": warmup, "launch_us": ms_launch * 1e3,
+                     "edges_per_s": wl["E"] / (ms_launch * 1e-3), "bound": "hbm"}
+            entry.update(_fractions(wl, ms_launch, _measured_traffic(wl["name"], idx)))
+            res[key] = entry
+            del wl, out
+        except RuntimeError as exc:
+            res[key] = {"error": str(exc)[:200]}
+        torch.cuda.empty_cache()
+    enc = synth.c5_encode(device="cuda")
+    labels = torch.empty((enc["m"],), dtype=torch.uint8, device="cuda")
+    _, ms = _time_steps(lambda: capi.kmeans_predict(enc["x"], enc["centers"], "l2", u8=True, out=labels), 50, 20)
+    tf = enc["flops"] / (ms * 1e-3) / 1e12
+    res["c5_encode_l2_argmin"] = {
+        "steps": 50, "warmup": 20, "launch_us": ms * 1e3, "vectors_per_s": enc["m"] / (ms * 1e-3), "bound": "mfma",
+        "algorithmic_flops": enc["flops"], "algorithmic_TFLOPps": tf, "executed_bf16_mfma_TFLOPps": 6 * tf,
+        "frac": 6 * tf / MFMA_BF16_PEAK_TFLOPS, "algorithmic_over_f32_mfma_peak": tf / MFMA_F32_PEAK_TFLOPS}
+    return res
 
 
 def _others(idx):
@@ -319,7 +408,10 @@ def main():
     # 5000 launches of ~25 us: the card's clocks and caches settle over ~100 ms, and a warm-up of
     # 100 launches (2.5 ms) leaves the timed region ~2 % slower on the same box.
     ap.add_argument("--warmup", type=int, default=5000)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default=None, choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--configs", default="auto", choices=["auto", "on", "off"],
+                    help="the other configurations and the cold-cache headline in the same line "
+                         "(auto: on unless --workload is given)")
     ap.add_argument("--idx", default="int64", choices=["int64", "int32"])
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the cpu_baseline leg (0 = skip)")
     ap.add_argument("--all", action="store_true", help="also measure the other workloads and ops")
@@ -345,9 +437,12 @@ def main():
               % (src.numel(), src.numel(), src.numel()))
         return
 
+    with_configs = args.configs == "on" or (args.configs == "auto" and args.workload is None)
+    args.workload = args.workload or "c2"
     wl, ms_per_step, launch_ms = _run_workload(args.workload, args.idx, args.steps, args.warmup)
     achieved = wl["algo_bytes"] / (launch_ms * 1e-3) / 1e9
     traffic = _measured_traffic(wl["name"], args.idx)
+    fr = _fractions(wl, launch_ms, traffic)
     result = {
         "metric": "edges aggregated/sec, fused decompress-SpMM",
         "value": wl["E"] / (ms_per_step * 1e-3),
@@ -364,10 +459,16 @@ def main():
         "config": {"workload": wl["name"], "index_dtype": args.idx, "dst_rows": wl["R"], "edges": wl["E"],
                    "src_rows": wl["N"], "feat_dim": wl["feat_dim"], "algorithmic_bytes": wl["algo_bytes"]},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "launch_us": launch_ms * 1e3},
+                     "frac": fr["frac"], "traffic": traffic, "launch_us": launch_ms * 1e3,
+                     "frac_algorithmic": fr["frac_algorithmic"], "frac_compulsory": fr["frac_compulsory"],
+                     "compulsory_bytes": fr["compulsory_bytes"]},
         "cpu_baseline": None,
     }
+    if with_configs:
+        cold_ms, cold_bytes, nblk = _cold_launch_ms(args.workload, args.idx, wl)
+        result["roofline"]["frac_cold"] = cold_bytes / (cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+        result["roofline"]["cold"] = {"launch_us": cold_ms * 1e3, "blocks_in_rotation": nblk,
+                                      "algorithmic_bytes": cold_bytes}
 
     if args.cpu_seconds > 0:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
@@ -390,9 +491,11 @@ def main():
                       "median of %d; unique+relabel (%.3f s) timed separately and excluded"
                       % (rows, wl["R"], edges, reps, relabel_secs),
         }
+    del wl
+    torch.cuda.empty_cache()
+    if with_configs:
+        result["configs"] = _configs(args.idx)
     if args.all:
-        del wl
-        torch.cuda.empty_cache()
         result["others"] = _others(args.idx)
     print(json.dumps(result))
 

@@ -12,6 +12,10 @@ edge counts are reproducible:
 
 Every workload is a dict with the operator inputs, `E` (edges), `R` (rows) and
 `algo_bytes` = E*(B_row + b_idx [+ 4 map]) + (R+1)*b_idx + R*D*4 + codebook bytes.
+
+`compulsory_bytes(wl)` is the same sum with every *distinct* source row (and row-map entry)
+counted once: what a launch must move through HBM at least, however well its caches work.
+`algo_bytes` charges a hot row once per edge and can therefore exceed what moves.
 """
 from __future__ import annotations
 
@@ -200,6 +204,64 @@ def scatter_ids(wl, mult=2_654_435_761):
         src = torch.arange(n, device=idx.device, dtype=torch.int64)
         inv[(src * (mult % n)) % n] = wl["row_map"]
         out["row_map"] = inv
+    return out
+
+
+def compulsory_bytes(wl):
+    """Bytes a launch cannot avoid moving: distinct source rows (and distinct row-map entries)
+    once each, plus indices, row offsets, output and codebooks / column parameters."""
+    idx = wl["indices"]
+    b = _idx_bytes(idx.dtype)
+    R, E, D = wl["R"], wl["E"], wl["feat_dim"]
+    uniq = torch.unique(idx)
+    if wl["kind"] == "hybrid":
+        hot = int((wl["row_map"][uniq.to(torch.int64)] >= 0).sum().item())
+        cb = wl["vq_codebooks"]
+        rows = hot * D + (uniq.numel() - hot) * cb.shape[0] + uniq.numel() * 4
+        fixed = cb.numel() * 4 + 2 * D * 4
+    elif wl["kind"] == "vq":
+        rows = uniq.numel() * wl["codes"].shape[1]
+        fixed = wl["codebooks"].numel() * 4
+    else:
+        rows = uniq.numel() * wl["codes"].shape[1]
+        fixed = 2 * D * 4
+    return int(rows + E * b + (R + 1) * b + R * D * 4 + fixed)
+
+
+def extra_blocks(wl, count, seed=1000):
+    """`count` further CSC blocks over the same tables, drawn like the workload's own (same degree
+    law, same id distribution, other seeds): lets a benchmark rotate graphs and outputs so that
+    nothing but the tables' hot rows is still cached when a buffer comes round again."""
+    dev = wl["indices"].device
+    out = []
+    for i in range(count):
+        g = _gen(seed + i, dev)
+        nb = dict(wl)
+        if wl["name"].startswith("c2"):
+            deg = powerlaw_degrees(wl["R"], 2.1, 12, g, dev)
+            zs = 1.1
+        else:
+            deg = torch.full((wl["R"],), wl["E"] // wl["R"], dtype=torch.int64, device=dev)
+            zs = 1.2 if wl["kind"] == "hybrid" else 1.1
+        nb["indptr"] = csc_from_degrees(deg, wl["indptr"].dtype)
+        nb["E"] = int(deg.sum().item())
+        if wl["name"].startswith("c1"):
+            nb["indices"] = torch.randint(0, wl["N"], (nb["E"],), generator=g, device=dev).to(wl["indices"].dtype)
+        else:
+            nb["indices"] = zipf_ids(wl["N"], (nb["E"],), zs, g, dev, wl["indices"].dtype)
+        row_b = wl["codes"].shape[1] if "codes" in wl else None
+        if row_b is not None:
+            b = _idx_bytes(wl["indices"].dtype)
+            fixed = wl["codebooks"].numel() * 4 if "codebooks" in wl else 2 * wl["feat_dim"] * 4
+            nb["algo_bytes"] = nb["E"] * (row_b + b) + (wl["R"] + 1) * b + wl["R"] * wl["feat_dim"] * 4 + fixed
+        elif wl["kind"] == "hybrid":
+            b = _idx_bytes(wl["indices"].dtype)
+            cb, D = wl["vq_codebooks"], wl["feat_dim"]
+            hot = int((nb["indices"] < wl["sq_codes"].shape[0]).sum().item())
+            nb["hot_edges"] = hot
+            nb["algo_bytes"] = (hot * D + (nb["E"] - hot) * cb.shape[0] + nb["E"] * (b + 4) + (wl["R"] + 1) * b
+                                + wl["R"] * D * 4 + cb.numel() * 4 + 2 * D * 4)
+        out.append(nb)
     return out
 
 
