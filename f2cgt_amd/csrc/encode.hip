@@ -78,7 +78,10 @@ __device__ int exact_argmin_row(const float* __restrict__ xrow, const float* __r
     const int oi = __shfl_xor(besti, off);
     if (ov < bestv || (ov == bestv && oi < besti)) { bestv = ov; besti = oi; }
   }
-  return besti;
+  // a row without a single comparable distance (NaN or infinite entries) goes to centre 0, where the
+  // callers' trainer sends it (examples/my_kmeans.py:92-94 turns such distances into 1 before the
+  // arg-min); the label must be a valid index whatever the data
+  return besti == INT_MAX ? 0 : besti;
 }
 
 // LDS layout of the MFMA A operands: [pair of 32-centre tiles][step][half][centre % 32][tile of pair].
@@ -114,7 +117,10 @@ __device__ int exact_argmin_row_l2_lds(const float* __restrict__ xrow, const flo
     const int oi = __shfl_xor(besti, off);
     if (ov < bestv || (ov == bestv && oi < besti)) { bestv = ov; besti = oi; }
   }
-  return besti;
+  // a row without a single comparable distance (NaN or infinite entries) goes to centre 0, where the
+  // callers' trainer sends it (examples/my_kmeans.py:92-94 turns such distances into 1 before the
+  // arg-min); the label must be a valid index whatever the data
+  return besti == INT_MAX ? 0 : besti;
 }
 
 // ---- general fallback: one wave per row, exact -------------------------------------------
@@ -492,7 +498,11 @@ __device__ int exact_argmin_row_l2_pieces(const float* __restrict__ xrow, float*
     bestv = m1; besti = i1; nextv = m2; nexti = i2; thirdv = m3;
   }
   const double margin = 4.9e-7 * ((double)xnorm2 + (double)cmax);
-  if (nextv - bestv > margin) return besti;              // also the only candidate (nextv = DBL_MAX)
+  // no candidate at all (a row with NaN or infinite entries: nothing compares below the limit), or one:
+  // the stages below index the centres with besti and nexti and must not see INT_MAX
+  if (besti == INT_MAX) return 0;
+  if (nexti == INT_MAX) return besti;
+  if (nextv - bestv > margin) return besti;
   if (thirdv - bestv <= margin) return -1 - besti;       // three or more: the caller takes every centre
   // exactly two centres can be the nearest one of the original row: decide between them there
   double da = 0.0, db = 0.0;
@@ -594,7 +604,10 @@ __device__ int exact_argmin_row_cosine_pieces(const float* __restrict__ xrow, fl
     const int oi = __shfl_xor(besti, off);
     if (ov < bestv || (ov == bestv && oi < besti)) { bestv = ov; besti = oi; }
   }
-  return besti;
+  // a row without a single comparable distance (NaN or infinite entries) goes to centre 0, where the
+  // callers' trainer sends it (examples/my_kmeans.py:92-94 turns such distances into 1 before the
+  // arg-min); the label must be a valid index whatever the data
+  return besti == INT_MAX ? 0 : besti;
 }
 
 // PW = false: labels of the nearest centre (KMeans.predict).  PW = true: the distance matrix itself

@@ -380,6 +380,8 @@ class KMeans {
       ++n_iter_;
       if ((it & 7) == 7 && stop.item<int>() != 0) break;   // later steps are no-ops once the flag is up
     }
+    // flag 2: the centre shift is not a number (NaN / infinite rows in the data); the centres are garbage
+    TORCH_CHECK(stop.item<int>() != 2, "KMeans.fit: the centre shift became NaN (non-finite input rows?)");
   }
 
   int64_t n_iter() const { return n_iter_; }
@@ -504,7 +506,7 @@ SideStream* side_stream_of(int device) {
 }
 
 // Aggregation followed by the dense layer that consumes it (the first layer of the GraphSAGE model,
-// examples/models/sage.py:62-70 with the mean aggregator: h = fc_neigh(mean over the neighbours)).
+// examples/conv.py:68-69, the layer examples/models.py:25-31 stacks, with the mean aggregator: h = fc_neigh(mean over the neighbours)).
 // At the reference's widest shape (768 features -> 256 units, 341k destination rows) the fp32 GEMM
 // takes 1.75 ms at 86 % of the matrix cores' fp32 peak and the aggregation 0.5 ms, so the multiply
 // is not moved into the aggregation kernel: it would slow the part that already dominates.

@@ -31,7 +31,7 @@ struct KmArgs {
   const uint8_t* labels_u8;
   float* centers;
   float* shift;         // [2]: sum_c |dc|, sum_c |dc|^2
-  int32_t* stop;        // may be null; nonzero = the centres are final, the step does nothing
+  int32_t* stop;        // may be null; nonzero = the centres are final, the step does nothing (1: rule met, 2: shift is NaN)
   float* sums;          // [n * k]
   uint32_t* counts;     // [n]
   int64_t m;
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(kKmThreads) void km_finalize_kernel(KmArgs a) {
   }
 #pragma unroll
   for (int off = kWave / 2; off > 0; off >>= 1) d2 += __shfl_xor(d2, off);
-  if (lane == 0 && d2 > 0.f) {
+  if (lane == 0 && !(d2 <= 0.f)) {   // a NaN shift is added too: the decide kernel has to see it
     add_f32<false>(a.shift, sqrtf(d2));
     add_f32<false>(a.shift + 1, d2);
   }
@@ -133,7 +133,10 @@ __global__ __launch_bounds__(kKmThreads) void km_finalize_kernel(KmArgs a) {
 __global__ void km_decide_kernel(KmArgs a) {
   if (a.stop == nullptr || *a.stop != 0 || a.rule == 0) return;
   const float s = a.rule == 1 ? a.shift[1] : a.shift[0] * a.shift[0];
-  if (s < a.tol) *a.stop = 1;
+  // a shift that is not a number never passes `s < tol`: flag it (2) so that the loop ends and the
+  // caller can tell (examples/my_kmeans.py:108-109 gives up on such a fit)
+  if (s != s) *a.stop = 2;
+  else if (s < a.tol) *a.stop = 1;
 }
 
 int km_check(const char* what, const float* x, const int64_t* l64, const uint8_t* l8, float* centers, float* shift,

@@ -39,7 +39,7 @@ struct VqArgs {
   int n_tiles, n_stripes;
   int stripes_per_xcd;  // > 0: the column tiles of a stripe share one XCD (see the kernel)
   int dense_store;      // sparse rows: results go through LDS so that every store instruction is dense
-  int store_late;       // experiments build only: selects the LATE form of the wave kernel (1..3; 9 = time stamps)
+  int store_late;       // experiments build only: 9 = the time-stamped form of the wave kernel
   unsigned long long* trace;   // experiments build only: per wave {start, first step, end} in 100 MHz ticks
 };
 
@@ -58,6 +58,15 @@ __device__ __forceinline__ float dpp_swap_pair(float v) {
 __device__ __forceinline__ float div_by(float a, float d, float r) {
   const float q = a * r;
   return __fmaf_rn(__fmaf_rn(-q, d, a), r, q);
+}
+
+// 1 / n for a row of n >= 2 edges, refined by one Newton step: within an ulp of the exact
+// reciprocal, so `sum * mean_scale(n)` is the mean to 2 ulp (relative 2.4e-7), where a correctly
+// rounded division costs three more vector instructions per output.
+__device__ __forceinline__ float mean_scale(int n) {
+  const float d = (float)n;
+  const float r = __builtin_amdgcn_rcpf(d);
+  return __fmaf_rn(__fmaf_rn(-d, r, 1.f), r, r);
 }
 
 template <int BT, typename Idx>
@@ -215,10 +224,8 @@ struct VqPipe {
         }
       }
       if (n > 1) {
-        const float d = (float)n;
-        float r = __builtin_amdgcn_rcpf(d);
-        r = __fmaf_rn(__fmaf_rn(-d, r, 1.f), r, r);
-        a0 = div_by(a0, d, r); a1 = div_by(a1, d, r); a2 = div_by(a2, d, r); a3 = div_by(a3, d, r);
+        const float r = mean_scale(n);
+        a0 *= r; a1 *= r; a2 *= r; a3 *= r;
       }
       store_nt4(out + (global_block(b) * kRows + row) * (int64_t)a.feat_dim + tile * 128 + c4 * 4, a0, a1, a2, a3);
     }
@@ -290,15 +297,14 @@ constexpr int kWPtr = 56;                     // ints per offset buffer: [0..12]
 
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
-template <int BT, int H, int RPM, typename Idx, int LATE = 0>
+template <int BT, int H, int RPM, typename Idx, bool DENSE = false, bool TRACE = false>
 __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* __restrict__ indptr,
                                                            const Idx* __restrict__ indices,
                                                            float* __restrict__ out) {
   using CW = typename code_word<BT>::type;
   constexpr int kWaves = kThreads / 64;
   constexpr int kMini = kWChunk / RPM;          // mini-blocks (RPM rows each) per chunk
-  constexpr bool HELD = LATE >= 1 && LATE <= 3; // results held in registers, stored later
-  constexpr bool TRACE = LATE == 9;             // time stamps per wave
+  // TRACE (experiments build): time stamps per wave
   unsigned long long t_start = 0;
   if constexpr (TRACE) t_start = wall_clock64();
   const bool K_FITS_ONE_PASS = a.K * 32 <= 8 * kThreads;
@@ -357,9 +363,14 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   // lanes per row: 32 lanes with one float4 each (H == 1) or 16 lanes with a whole 8-column code
   // each (H == 2); the wave then works on 2 or 4 rows at a time
   constexpr int kLanesPerRow = 32 / H, kRowsPerPass = 64 / kLanesPerRow;
-  const int c4 = lane & (kLanesPerRow - 1), half = lane / kLanesPerRow;
+  // A lane beyond the columns of a partial tile takes the tile's last column group again (it
+  // computes and stores what that group's own lane does), so that no lane ever skips a store: the
+  // number of memory operations of a step is then the same on every path, and the waits in front
+  // of the next step's loads can leave this step's stores in flight (see the main loop).
+  const int groups = tile_cols / (4 * H);      // column groups of this tile (tile_cols % (4 H) == 0)
+  const int c4 = (lane & (kLanesPerRow - 1)) < groups ? (lane & (kLanesPerRow - 1)) : groups - 1;
+  const int half = lane / kLanesPerRow;
   const int col0 = c4 * 4 * H;                 // first column of the lane inside the tile
-  const bool col_on = col0 < tile_cols;
   const int byte_idx = col0 / a.w;
   const float* cbp = s_cb + c4 * 4;
   const uint8_t* code_base = a.codes + tile * BT;
@@ -455,55 +466,30 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   // the two halves of the lane's 32 bytes, and they have to reach the L1 together: issued a few
   // instructions apart (separate predicated blocks) the halves are written to memory separately
   // and the kernel falls into a regime twice as slow (24 x 32 codebooks: 497 -> 870-960 us, L2 ->
-  // memory write-credit stalls up from 2e4 to 3.7e7 cycles per launch).  LATE (built with the
-  // experiments only, chosen by F2CGT_VQ_DEFER) holds the results in registers and stores them later:
-  // 1 = at the end of the step, 2 = behind the loads of the next step, so that the stores have that
-  // step's sums to complete, 3 = as 2 with a wait for them in front of the sums.  With whole-line
-  // stores (the LDS-staged form, F2CGT_VQ_DENSE=1) all placements run at the same speed (520 us),
-  // i.e. a wave does not lose time waiting for its own stores and there is nothing to gain by
-  // moving them; with the half-line pair every LATE form is in the slow regime.  Not adopted.
-  float4 pend_v[2] = {make_float4(0.f, 0.f, 0.f, 0.f), make_float4(0.f, 0.f, 0.f, 0.f)};
-  float* pend_p[2] = {out, out};
-  bool pend_on[2] = {false, false};
-  auto flush_stores = [&]() {
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      if (pend_on[j]) store_nt4(pend_p[j], pend_v[j].x, pend_v[j].y, pend_v[j].z, pend_v[j].w);
-      pend_on[j] = false;
-    }
-  };
+  // memory write-credit stalls up from 2e4 to 3.7e7 cycles per launch).
+  //
+  // Loads and stores complete in order on one counter.  A step issues its loads (code bytes of the
+  // next mini-block, source ids of the one after) in front of its sums and its stores behind them,
+  // and the next step waits for those loads only: it may leave the younger stores in flight if the
+  // compiler can count them, i.e. if every path through a step issues the same number of stores.
+  // Hence no store below sits under a condition: a lane group without a row of its own (the last
+  // mini-block of a range) takes the mini-block's last row again and stores the same values to the
+  // same place, as do the lane groups that shared a row's edges.  With conditional stores every
+  // step began by waiting for the stores of the one before, a full trip to memory per step and wave.
   unsigned long long t_first = 0;
   if constexpr (TRACE) t_first = wall_clock64();
-  int m = (int)g_first;   // position of g inside its chunk (negative during the two start-up steps)
-  for (int64_t g = g_first; g < n_mini; ++g) {
-    // chunk-level P stage, driven by the position of g inside its chunk
-    if (g >= 0) {
-      if (m == 0) {
-        // take the next free chunk of the workgroup and request its row offsets
-        int id = 0;
-        if (lane == 0) id = atomicAdd(s_next, 1);
-        id = uni(id);
-        have_next = id < wg_chunks;
-        if (have_next) {
-          base_next = wg_row0 + (int64_t)id * kWChunk;
-          n_mini += minis_of(base_next);
-          issue_P(base_next);
-        }
-      }
-      if (m == kMini / 2 && have_next) park_P(par ^ 1);
-    }
-    // park C(g)
+  int eb2 = 0, ne2 = 0;
+  // the load stages of step g at position m of its chunk: park C(g), issue C(g+1), issue I(g+2)
+  auto front = [&](int64_t g, int m) {
     if (g >= 0 && ne0 <= kWEdges && lane < ne0) *reinterpret_cast<CW*>(s_codes + lane * BT) = Creg;
-    // issue C(g+1): the id fetched one step ago is clamped only now
-    {
+    {  // C(g+1): the id fetched one step ago is clamped only now
       const bool on = g + 1 >= 0 && g + 1 < n_mini && ne1 <= kWEdges && lane < ne1;
       const uint64_t raw = (uint64_t)Ireg;
       const uint32_t id = (raw >> 32) ? n_last : ((uint32_t)raw < n_last ? (uint32_t)raw : n_last);
       Creg = *reinterpret_cast<const CW*>(code_base + (uint64_t)(on ? id : 0u) * (uint32_t)a.n_cb);
     }
-    // issue I(g+2)
-    int eb2 = 0, ne2 = 0;
-    {
+    eb2 = 0; ne2 = 0;
+    {  // I(g+2)
       const bool v = g + 2 < n_mini;
       int64_t e0 = 0;
       if (v) {
@@ -516,22 +502,46 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       const Idx* src = on ? indices + e0 + eb2 + lane : indptr;
       Ireg = (int64_t)*src;
     }
-    if constexpr (LATE == 2 || LATE == 3) {
-      flush_stores();   // results of mini-block g - 1
-      if (LATE == 3) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  };
+  // start-up without the early loads (large or unaligned codebooks): two steps that only load
+  for (int64_t g = g_first; g < 0; ++g) {
+    front(g, (int)g);
+    eb0 = eb1; ne0 = ne1;
+    eb1 = eb2; ne1 = ne2;
+  }
+  int m = 0;   // position of g inside its chunk
+  // One step.  The first step runs ahead of the loop on its own copy of the code, so that the loop
+  // is entered with the same memory operations in flight as after any of its own iterations (two
+  // loads, then two stores): the compiler's counts for the waits are the minimum over every way
+  // into the loop, and the start-up, which has no stores yet, would otherwise set them to "all".
+  auto step = [&](int64_t g) __attribute__((always_inline)) {
+    // chunk-level P stage, driven by the position of g inside its chunk
+    if (m == 0) {
+      // take the next free chunk of the workgroup and request its row offsets
+      int id = 0;
+      if (lane == 0) id = atomicAdd(s_next, 1);
+      id = uni(id);
+      have_next = id < wg_chunks;
+      if (have_next) {
+        base_next = wg_row0 + (int64_t)id * kWChunk;
+        n_mini += minis_of(base_next);
+        issue_P(base_next);
+      }
+    } else if (m == kMini / 2 && have_next) {   // `else`: never in the step that issued the load
+      park_P(par ^ 1);
     }
+    front(g, m);
     // compute mini-block g
-    if (g >= 0) {
+    {
       const int* buf = s_ptr + par * kWPtr + m * RPM;
       const int64_t row0 = base_cur + m * RPM;
       const int64_t left = row_end - row0;
-      const int nr = (int)(left < RPM ? left : RPM);
+      const int nr = (int)(left < RPM ? left : RPM);          // >= 1: the mini-block exists
       const bool staged = ne0 <= kWEdges;
       // RPM < 4 (H == 2 only): the 4 / RPM lane groups ("slots") of a pass share a row, slot s of
       // them takes the row's edges s, s + SPR, ... and the partial sums are added across the slots
       constexpr int SPR = kRowsPerPass / (RPM < kRowsPerPass ? RPM : kRowsPerPass);
       constexpr int kPasses = RPM * SPR / kRowsPerPass;
-      static_assert(!HELD || H * kPasses == 2, "two pending stores per lane");
       // sum of the codebook entries of this slot's share of row `row` (all of it when SPR == 1),
       // in edge order; returns the row's edge count
       auto row_sum = [&](int row, int sub, float (&acc)[H][4]) -> int {
@@ -589,59 +599,55 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       };
       auto mean = [&](int n, float (&acc)[H][4]) {
         if (n > 1) {
-          const float d = (float)n;
-          float r = __builtin_amdgcn_rcpf(d);
-          r = __fmaf_rn(__fmaf_rn(-d, r, 1.f), r, r);
+          const float r = mean_scale(n);
 #pragma unroll
           for (int h = 0; h < H; ++h)
 #pragma unroll
-            for (int t = 0; t < 4; ++t) acc[h][t] = div_by(acc[h][t], d, r);
+            for (int t = 0; t < 4; ++t) acc[h][t] *= r;
         }
       };
-      if (H == 2 && SPR == 1 && kPasses == 1 && a.dense_store == 1) {
+      if constexpr (DENSE) {
+        static_assert(H == 2 && SPR == 1 && kPasses == 1, "the LDS-turned stores are for 4-row steps of 16-lane rows");
         // Four rows, sixteen lanes each.  A lane's result is 32 consecutive bytes, which as two
         // stores would be 16 of every 32 bytes per instruction (half-written sectors on the way to
         // memory).  The wave's 1 KB staging area, free once the edge loops are done, turns them
         // around: the lanes of columns [64 p, 64 p + 64) write their two float4, every lane reads
         // back the float4 of its own lane index, and each store instruction covers 256 contiguous
-        // bytes of every row.
-        const int row = half;
-        const bool active = col_on && row < nr;
+        // bytes of every row.  (Lanes beyond a partial tile's columns hold a copy of its last
+        // column group and skip the write to the staging area; their stores repeat the last float4.)
+        const int lane_c = lane & (kLanesPerRow - 1);
+        const int row = half < nr ? half : nr - 1;
         float acc[H][4];
-#pragma unroll
-        for (int h = 0; h < H; ++h) acc[h][0] = acc[h][1] = acc[h][2] = acc[h][3] = 0.f;
-        if (active) {
-          const int n = row_sum(row, 0, acc);
-          mean(n, acc);
-        }
+        const int n = row_sum(row, 0, acc);
+        mean(n, acc);
         float4* stg = reinterpret_cast<float4*>(s_codes);
         float* obase = out + (row0 + row) * (int64_t)a.feat_dim + tile * 128;
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
           __builtin_amdgcn_wave_barrier();
-          if ((c4 >> 3) == p) {
+          if ((lane_c >> 3) == p && lane_c < groups) {
 #pragma unroll
             for (int h = 0; h < H; ++h)
-              stg[row * 16 + (c4 & 7) * 2 + h] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+              stg[half * 16 + (lane_c & 7) * 2 + h] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
           }
           __builtin_amdgcn_wave_barrier();
-          const float4 v = stg[row * 16 + c4];
-          const int col = 64 * p + 4 * c4;
-          if constexpr (HELD) {
-            pend_v[p] = v;
-            pend_p[p] = obase + col;
-            pend_on[p] = row < nr && col < tile_cols;
-          } else {
-            if (row < nr && col < tile_cols) store_nt4(obase + col, v.x, v.y, v.z, v.w);
-          }
+          // a lane beyond the tile's columns stores the tile's last float4 again; when that lies in
+          // the other half (tile_cols <= 64 p) nobody wrote to the staging area in this pass and it
+          // still holds that half
+          int col = 64 * p + 4 * lane_c;
+          const int last = tile_cols - 4;                  // first column of the tile's last float4
+          col = col < last ? col : last;
+          const float4 v = stg[half * 16 + ((col & 63) >> 2)];
+          store_nt4(obase + col, v.x, v.y, v.z, v.w);
         }
-      } else if (col_on) {
+      } else {
         float* orow = out + row0 * (int64_t)a.feat_dim + tile * 128 + col0;
 #pragma unroll
         for (int pass = 0; pass < kPasses; ++pass) {
           const int slot = pass * kRowsPerPass + half;
-          const int row = slot / SPR, sub = slot % SPR;
-          if (row >= nr) continue;
+          int row = slot / SPR;
+          const int sub = slot % SPR;
+          row = row < nr ? row : nr - 1;
           float acc[H][4];
           const int n = row_sum(row, sub, acc);
           if (SPR > 1) {
@@ -652,26 +658,17 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
                 acc[h][t] += __shfl_xor(acc[h][t], kLanesPerRow);
                 if (SPR > 2) acc[h][t] += __shfl_xor(acc[h][t], 2 * kLanesPerRow);
               }
-            if (sub != 0) continue;
           }
           mean(n, acc);
 #ifdef F2CGT_EXPERIMENTS
           if (a.dense_store == 2 && acc[0][0] != 12345.678f) continue;   // no stores: what the rest of the kernel costs
 #endif
 #pragma unroll
-          for (int h = 0; h < H; ++h) {
-            if constexpr (HELD) {
-              pend_v[pass * H + h] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
-              pend_p[pass * H + h] = orow + (int64_t)row * a.feat_dim + 4 * h;
-              pend_on[pass * H + h] = true;
-            } else {
-              store_nt4(orow + (int64_t)row * a.feat_dim + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
-            }
-          }
+          for (int h = 0; h < H; ++h)
+            store_nt4(orow + (int64_t)row * a.feat_dim + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
         }
       }
     }
-    if constexpr (LATE == 1) flush_stores();
     eb0 = eb1; ne0 = ne1;
     eb1 = eb2; ne1 = ne2;
     if (++m == kMini) {   // on to the next chunk (the loop ends here when there is none)
@@ -680,8 +677,11 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       base_cur = base_next;
       have_next = false;
     }
+  };
+  if (n_mini > 0) {
+    step(0);
+    for (int64_t g = 1; g < n_mini; ++g) step(g);
   }
-  if constexpr (HELD) flush_stores();
   if constexpr (TRACE) {
     if (lane == 0) {
       unsigned long long* t = a.trace + ((size_t)blockIdx.x * kWaves + wave) * 4;
@@ -1039,15 +1039,15 @@ int launch_strip_w(const VqArgs& a, int ke, const void* indptr, const void* indi
 #ifdef F2CGT_EXPERIMENTS
 unsigned long long* g_trace = nullptr;   // device buffer for the time stamps of F2CGT_VQ_DEFER=9
 
-// the 4-row, int64 form of the wave kernel with its stores held back (see LATE in the kernel)
-template <int BT, int LATE>
-int launch_wave_late(const VqArgs& a, const void* indptr, const void* indices, float* out, hipStream_t st,
-                     const char* what, unsigned grid, size_t wlds) {
-  const void* kern = reinterpret_cast<const void*>(vq_wave_kernel<BT, 2, 4, int64_t, LATE>);
+// the 4-row, int64 form of the wave kernel with time stamps per wave
+template <int BT>
+int launch_wave_trace(const VqArgs& a, const void* indptr, const void* indices, float* out, hipStream_t st,
+                      const char* what, unsigned grid, size_t wlds) {
+  const void* kern = reinterpret_cast<const void*>(vq_wave_kernel<BT, 2, 4, int64_t, false, true>);
   const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
   if (e != hipSuccess) return fail((int)e, "%s: cannot reserve %zu B of LDS", what, wlds);
-  vq_wave_kernel<BT, 2, 4, int64_t, LATE><<<grid, kThreads, wlds, st>>>(a, static_cast<const int64_t*>(indptr),
-                                                                         static_cast<const int64_t*>(indices), out);
+  vq_wave_kernel<BT, 2, 4, int64_t, false, true><<<grid, kThreads, wlds, st>>>(
+      a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
   return launch_status(what);
 }
 #endif
@@ -1061,22 +1061,24 @@ int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int id
   }
 #ifdef F2CGT_EXPERIMENTS
   if (H == 2 && RPM == 4 && idx_dtype == F2CGT_DT_I64) {
-    if (a.store_late == 1) return launch_wave_late<BT, 1>(a, indptr, indices, out, st, what, grid, wlds);
-    if (a.store_late == 2) return launch_wave_late<BT, 2>(a, indptr, indices, out, st, what, grid, wlds);
-    if (a.store_late == 3) return launch_wave_late<BT, 3>(a, indptr, indices, out, st, what, grid, wlds);
-    if (a.store_late == 9 && a.trace) return launch_wave_late<BT, 9>(a, indptr, indices, out, st, what, grid, wlds);
+    if (a.store_late == 9 && a.trace) return launch_wave_trace<BT>(a, indptr, indices, out, st, what, grid, wlds);
   }
 #endif
-  const void* kern = idx_dtype == F2CGT_DT_I32 ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t>)
-                                               : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t>);
+  // the sparse-row form (results turned round in LDS before they are stored) is its own instantiation
+  constexpr bool CAN_DENSE = H == 2 && RPM == 4;
+  const bool dense = CAN_DENSE && a.dense_store == 1;
+  const void* kern;
+  if (idx_dtype == F2CGT_DT_I32)
+    kern = dense ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, CAN_DENSE>)
+                 : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false>);
+  else
+    kern = dense ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t, CAN_DENSE>)
+                 : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t, false>);
   const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
   if (e != hipSuccess) return fail((int)e, "%s: cannot reserve %zu B of LDS", what, wlds);
-  if (idx_dtype == F2CGT_DT_I32)
-    vq_wave_kernel<BT, H, RPM, int32_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int32_t*>(indptr),
-                                                                      static_cast<const int32_t*>(indices), out);
-  else
-    vq_wave_kernel<BT, H, RPM, int64_t><<<grid, kThreads, wlds, st>>>(a, static_cast<const int64_t*>(indptr),
-                                                                      static_cast<const int64_t*>(indices), out);
+  void* params[] = {const_cast<VqArgs*>(&a), &indptr, &indices, &out};
+  const hipError_t le = hipLaunchKernel(kern, dim3(grid), dim3(kThreads), params, wlds, st);
+  if (le != hipSuccess) return fail((int)le, "%s: launch failed: %s", what, hipGetErrorString(le));
   return launch_status(what);
 }
 

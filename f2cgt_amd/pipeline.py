@@ -149,6 +149,13 @@ class KMeansTrainer:
             self.n_iter += 1
             if it % self.check_every == self.check_every - 1 and int(stop.item()):
                 break
+        if int(stop.item()) == 2:
+            # the centre shift is not a number (NaN or infinite input): the reference's trainer gives
+            # up on such a fit (examples/my_kmeans.py:108-109); so does this one, loudly
+            import warnings
+            warnings.warn("KMeansTrainer.fit: the centre shift became NaN; no centres were produced")
+            self.centers = None
+            return
         self.centers = centers
 
     def get_centers(self):
@@ -398,6 +405,8 @@ class CompressionManager:
         side = self.seeds_task_stream
         side.wait_stream(torch.cuda.current_stream())      # seeds_key may still be in the making
         with torch.cuda.stream(side):
+            # the caller may drop seeds_key as soon as this returns: tie its memory to the side stream
+            seeds_key.record_stream(side)
             slots = self.seed_slot[seeds_key.long()].long()
             if self.check_seed_keys and bool((slots < 0).any()):
                 raise KeyError("a requested id is not a seed row")

@@ -244,7 +244,9 @@ int f2cgt_kmeans_update(const float* x, const int64_t* labels_i64, const uint8_t
  * inside the library (272 KB per device, kept until the process ends), so the problem is limited to
  * n * k <= 65536 sums and n <= 4096 centres; larger ones return F2CGT_E_UNSUPPORTED.  Same arguments,
  * results and stop-flag behaviour as f2cgt_kmeans_update.  Every call on a device uses that device's
- * one array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not. */
+ * one array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.
+ * The first call on each device looks the array's address up (hipGetSymbolAddress, which may load
+ * the code object): make that first call outside any stream capture; later calls only launch kernels. */
 int f2cgt_kmeans_update_static(const float* x, const int64_t* labels_i64, const uint8_t* labels_u8,
                                float* centers, float* shift, int32_t* stop, int stop_rule, float tol,
                                int64_t m, int64_t n, int64_t k, void* stream);

@@ -11,6 +11,7 @@ import pytest
 import torch
 
 import f2cgt_oracle as oc
+from parity_bars import assert_mean_aggregate
 from f2cgt_amd import capi, synth
 
 pytestmark = pytest.mark.gpu
@@ -66,7 +67,7 @@ def _oracle_rows(wl, rows):
         if (~hot).any():
             vq = wl["vq_codes"][torch.from_numpy(-m[~hot] - 1).to(tu.device)].cpu().numpy()
             dec[~hot] = oc.vq_decompress(vq, wl["vq_codebooks"].cpu().numpy(), wl["feat_dim"])
-    return oc.spmm_csr(dec, sub_ptr, inv), float(np.abs(dec).max())
+    return oc.spmm_csr(dec, sub_ptr, inv), oc.spmm_csr(dec.astype(np.float64), sub_ptr, inv), float(np.abs(dec).max())
 
 
 @pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
@@ -81,17 +82,18 @@ def test_full_size_workload(name, idx):
     # sampled rows against the CPU oracle
     rng = np.random.default_rng(0)
     rows = np.unique(np.concatenate([rng.integers(0, R, size=300), [0, R - 1]]))
-    want, scale = _oracle_rows(wl, rows)
+    want, exact, scale = _oracle_rows(wl, rows)
     got = out[torch.from_numpy(rows).cuda()].cpu().numpy()
-    assert np.allclose(got, want, rtol=RTOL, atol=RTOL * scale)
+    # 1e-5 of each row's magnitude, and no further from the float64 mean than the reference's fp32 sum
+    assert_mean_aggregate(got, want, exact, scale)
 
     # fused == unfused on the GPU: decode the unique source rows, aggregate with the plain kernel
     uniq, inv = torch.unique(wl["indices"].long(), return_inverse=True)
     dec = _decode_rows(wl, uniq)
     unfused = capi.spmm_csr(dec, wl["indptr"].long(), inv)
     torch.cuda.synchronize()
-    tol = RTOL * float(dec.abs().max())
-    assert float((out - unfused).abs().max()) <= tol + RTOL * float(unfused.abs().max())
+    row_scale = unfused.abs().amax(dim=1, keepdim=True).clamp_min(1e-30)
+    assert bool(((out - unfused).abs() <= RTOL * row_scale).all())
 
     # checksum of checksums in fp64: sum_r deg_r * out[r] == sum_e decoded[index_e]
     deg = (wl["indptr"][1:] - wl["indptr"][:-1]).double()

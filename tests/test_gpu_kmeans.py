@@ -108,7 +108,7 @@ def test_kmeans_fit_reaches_a_fixed_point(metric):
     torch.manual_seed(3)
     quick = lib.KMeans(12, 8, metric, max_iter=300, tol=1e-1)
     quick.fit(x)
-    assert quick.n_iter <= km.n_iter and quick.n_iter % 8 == 0 or quick.n_iter == 300
+    assert quick.n_iter <= km.n_iter and (quick.n_iter % 8 == 0 or quick.n_iter == 300)
 
 
 def test_kmeans_warns_about_ignored_arguments():
@@ -153,3 +153,45 @@ def test_pipeline_trainer_follows_the_reference_rule(metric, width):
     assert np.allclose(runs[0].get_centers().cpu().numpy(), centers, rtol=1e-3, atol=1e-3)
     labels = runs[0].predict(x)
     assert labels.shape == (len(pts),)
+
+
+def test_nan_shift_raises_the_flag_and_ends_the_fit():
+    """A centre shift that is not a number never satisfies `shift < tol`: the update kernel flags it
+    (stop == 2), the trainer ends without centres like the reference's (examples/my_kmeans.py:108-109)
+    and KMeans.fit raises."""
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((2000, 8)).astype(np.float32)
+    x[17, 3] = np.nan
+    centers = rng.standard_normal((8, 8)).astype(np.float32)
+    labels = rng.integers(0, 8, size=2000)
+    c, stop = dev(centers), torch.zeros(1, dtype=torch.int32, device="cuda")
+    capi.kmeans_update(dev(x), dev(labels), c, stop=stop, rule=2, tol=1e-4)
+    assert int(stop.item()) == 2
+    frozen = c.clone()
+    capi.kmeans_update(dev(x), dev(labels), c, stop=stop, rule=2, tol=1e-4)      # a no-op once the flag is up
+    assert torch.equal(torch.nan_to_num(frozen), torch.nan_to_num(c)) and int(stop.item()) == 2
+    km = pipeline.KMeansTrainer(8, metric="euclidean", tol=1e-4, generator=torch.Generator().manual_seed(1))
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        km.fit(dev(x))
+    assert km.get_centers() is None and km.n_iter <= 8 and any("NaN" in str(w.message) for w in seen)
+    with pytest.raises(RuntimeError, match="NaN"):
+        f2cgt_amd.load().KMeans(8, 8, "l2", max_iter=50).fit(dev(x))
+
+
+def test_cosine_fit_with_a_zero_row():
+    """A zero-norm row has no cosine distance (0 / 0): the reference's trainer sets such distances to 1
+    before the arg-min (examples/my_kmeans.py:92-94), so the row goes to centre 0; here all its scores
+    tie and the first centre wins as well, and nothing non-finite reaches the centres."""
+    rng = np.random.default_rng(12)
+    pts, _, _ = blobs(rng, 400, 8, spread=5.0)
+    pts[5] = 0.0
+    x = dev(pts)
+    km = pipeline.KMeansTrainer(6, metric="cosine", tol=5e-2, generator=torch.Generator().manual_seed(4))
+    km.fit(x)
+    centers = km.get_centers()
+    assert centers is not None and bool(torch.isfinite(centers).all())
+    labels = km.predict(x)
+    assert int(labels[5]) == 0
+    want = oc.kmeans_predict(pts, centers.cpu().numpy(), "cosine")[0]
+    assert int(want[5]) == 0

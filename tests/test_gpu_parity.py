@@ -7,6 +7,7 @@ import pytest
 import torch
 
 import f2cgt_oracle as oc
+from parity_bars import assert_mean_aggregate
 from f2cgt_amd import capi
 
 pytestmark = pytest.mark.gpu
@@ -338,18 +339,22 @@ def test_fused_vq_vs_oracle(idx, shape):
     indptr, indices = random_graph(rng, R, N, 20, idx)
     got = host(capi.vq_decompress_spmm_csr(dev(codes), dev(cb), dev(indptr), dev(indices), feat_dim))
     want = oc.vq_decompress_spmm_csr(codes, cb, indptr, indices, feat_dim)
-    assert close(got, want)
+    dec = oc.vq_decompress(codes, cb, feat_dim)
+    exact = oc.spmm_csr(dec.astype(np.float64), indptr.astype(np.int64), indices.astype(np.int64))
+    assert_mean_aggregate(got, want, exact, np.abs(dec).max(), np.diff(indptr.astype(np.int64)))
     unfused = host(capi.spmm_csr(capi.vq_decompress(dev(codes), dev(cb), feat_dim), dev(indptr), dev(indices)))
-    assert close(got, unfused)
+    assert np.array_equal(unfused, want)       # the unfused composition is the reference's order and division
 
 
 @pytest.mark.parametrize("max_deg,rows", [(50, 1500), (200, 700), (3, 4099)])
 def test_fused_vq_degree_regimes(max_deg, rows):
     # average degree up to 15: wave-granular pipeline with 4-row mini-blocks, with a row count that
     # leaves partial chunks and mini-blocks; above 60: block-synchronous pipeline (blocks above 1024
-    # edges summed from HBM).  Both keep the sequential edge order, so the result is bit-exact.  In
-    # between (max_deg 50: about 25 per row) two or four lane groups share a row and their partial
-    # sums are added, so the order differs and the bar is the 1e-5 relative one.
+    # edges summed from HBM).  Both keep the sequential edge order and take the mean as sum * (1 / n)
+    # with a refined reciprocal (within 2 ulp of the reference's division).  In between (max_deg 50:
+    # about 25 per row) two or four lane groups share a row and their partial sums are added, so the
+    # order differs as well.  The bar for all of them: 1e-5 of the row's magnitude, no further from
+    # the float64 mean than the reference's own fp32 evaluation, single-neighbour rows bit-exact.
     rng = np.random.default_rng(max_deg)
     N = 3000
     cb = rng.standard_normal((16, 256, 8)).astype(np.float32)
@@ -357,13 +362,9 @@ def test_fused_vq_degree_regimes(max_deg, rows):
     indptr, indices = random_graph(rng, rows, N, max_deg)
     got = host(capi.vq_decompress_spmm_csr(dev(codes), dev(cb), dev(indptr), dev(indices), 128))
     want = oc.vq_decompress_spmm_csr(codes, cb, indptr, indices, 128)
-    avg = indices.size / rows
-    if 15 < avg <= 60:
-        assert close(got, want)
-        single = np.diff(indptr) == 1
-        assert np.array_equal(got[single], want[single])
-    else:
-        assert np.array_equal(got, want)
+    dec = oc.vq_decompress(codes, cb, 128)
+    exact = oc.spmm_csr(dec.astype(np.float64), indptr, indices)
+    assert_mean_aggregate(got, want, exact, np.abs(dec).max(), np.diff(indptr))
 
 
 @pytest.mark.parametrize("fanout,rows", [(20, 1003), (27, 515), (45, 300), (60, 130)])
@@ -378,10 +379,9 @@ def test_fused_vq_shared_rows(fanout, rows):
     indices = rng.integers(0, N, size=rows * fanout).astype(np.int32)
     got = host(capi.vq_decompress_spmm_csr(dev(codes), dev(cb), dev(indptr), dev(indices), 256))
     want = oc.vq_decompress_spmm_csr(codes, cb, indptr.astype(np.int64), indices.astype(np.int64), 256)
-    assert close(got, want)
-    exact = oc.spmm_csr(oc.vq_decompress(codes, cb, 256).astype(np.float64), indptr.astype(np.int64),
-                        indices.astype(np.int64))
-    assert np.abs(got - exact).max() <= 1e-5 * np.abs(exact).max() + 1e-6
+    dec = oc.vq_decompress(codes, cb, 256)
+    exact = oc.spmm_csr(dec.astype(np.float64), indptr.astype(np.int64), indices.astype(np.int64))
+    assert_mean_aggregate(got, want, exact, np.abs(dec).max())
 
 
 @pytest.mark.parametrize("w,n_cb,feat_dim", [(8, 32, 200), (16, 16, 248), (32, 8, 160)])
@@ -396,7 +396,9 @@ def test_fused_vq_sparse_rows_partial_tiles(w, n_cb, feat_dim):
     got = host(capi.vq_decompress_spmm_csr(dev(codes), dev(cb), dev(indptr), dev(indices), feat_dim))
     want = oc.vq_decompress_spmm_csr(codes, cb, indptr, indices, feat_dim)
     assert got.shape == (rows, feat_dim)
-    assert np.array_equal(got, want)        # sequential edge order: bit-exact
+    dec = oc.vq_decompress(codes, cb, feat_dim)
+    exact = oc.spmm_csr(dec.astype(np.float64), indptr, indices)
+    assert_mean_aggregate(got, want, exact, np.abs(dec).max(), np.diff(indptr))
 
 
 def test_fused_vq_int16_codes_big_codebook():
@@ -623,6 +625,32 @@ def test_kmeans_predict_vs_oracle(metric, m, n, k):
     got = host(capi.kmeans_predict(dev(x), dev(c), metric))
     assert np.array_equal(got[~near], want[~near])
     assert near.mean() < 0.01
+    if n <= 256:
+        got8 = host(capi.kmeans_predict(dev(x), dev(c), metric, u8=True))
+        assert np.array_equal(got8.astype(np.int64), got)
+
+
+@pytest.mark.parametrize("metric", ["l2", "cosine"])
+@pytest.mark.parametrize("m,n,k", [(2000, 8, 8), (3000, 256, 32), (500, 1000, 24), (300, 50, 200)])
+def test_kmeans_predict_rows_that_are_not_numbers(metric, m, n, k):
+    """Rows with NaN or infinite entries have no nearest centre.  Their labels must still be valid
+    indices (centre 0: the callers' trainer turns NaN distances into 1 before its arg-min,
+    examples/my_kmeans.py:92-94, which sends such a row to the first centre) and the other rows must
+    not notice: an arg-min stage that found no comparable distance used to keep its "none yet" index."""
+    rng = np.random.default_rng(m + k)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    c = rng.standard_normal((n, k)).astype(np.float32)
+    clean, near = oc.kmeans_predict(x, c, metric)
+    bad = rng.choice(m, size=25, replace=False)
+    x[bad[:10], rng.integers(0, k, size=10)] = np.nan
+    x[bad[10:18]] = np.nan
+    x[bad[18:], rng.integers(0, k, size=7)] = np.inf
+    got = host(capi.kmeans_predict(dev(x), dev(c), metric))
+    assert got.min() >= 0 and got.max() < n
+    assert np.all(got[bad[:18]] == 0)
+    keep = np.ones(m, dtype=bool)
+    keep[bad] = False
+    assert np.array_equal(got[keep & ~near], clean[keep & ~near])
     if n <= 256:
         got8 = host(capi.kmeans_predict(dev(x), dev(c), metric, u8=True))
         assert np.array_equal(got8.astype(np.int64), got)
