@@ -25,8 +25,9 @@ def lib_dir() -> str:
 
 
 def capi_path() -> str:
-    """Path of the C-ABI shared library (see include/f2cgt.h)."""
-    return os.path.join(_LIB, "libf2cgt_hip.so")
+    """Path of the C-ABI shared library (see include/f2cgt.h); F2CGT_AMD_CAPI_LIB names another build of it
+    (same ABI), e.g. to compare two builds in one session."""
+    return os.environ.get("F2CGT_AMD_CAPI_LIB") or os.path.join(_LIB, "libf2cgt_hip.so")
 
 
 def load():

@@ -311,7 +311,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   extern __shared__ __align__(16) unsigned char smem[];
   float* s_cb = reinterpret_cast<float*>(smem);
   const int wave = uni((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
-  constexpr int kStage = kWEdges * BT > 1024 ? kWEdges * BT : 1024;   // code bytes of a mini-block, or 64 float4
+  constexpr int kStage = kWEdges * BT > 1024 ? kWEdges * BT : 1024;     // code bytes of a mini-block, or 64 float4
   unsigned char* s_codes = smem + (size_t)a.K * 128 * 4 + (size_t)wave * kStage;
   int* s_ptr = reinterpret_cast<int*>(smem + (size_t)a.K * 128 * 4 + (size_t)kWaves * kStage) + wave * 2 * kWPtr;
 
@@ -383,6 +383,13 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     const int nr = (int)(left < kWChunk ? left : kWChunk);
     Preg = (int64_t)indptr[row0 + (lane < nr ? lane : nr)];
   };
+  // With 4-row mini-blocks the four mini-block boundaries of a chunk and its first edge are also
+  // kept in scalar registers, one set per offset buffer (read out of the lanes when the offsets
+  // are parked), so that the bounds of a mini-block cost no LDS read and no vector instruction in
+  // any step; with more mini-blocks per chunk they are read back from LDS.
+  constexpr bool SCALAR_BOUNDS = RPM == 4;
+  int sb0[4] = {0, 0, 0, 0}, sb1[4] = {0, 0, 0, 0};
+  int64_t se0[2] = {0, 0};
   auto park_P = [&](int which) {
     int* buf = s_ptr + which * kWPtr;
     const uint32_t lo = (uint32_t)uni((int)(uint32_t)Preg);
@@ -392,22 +399,42 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     int64_t v = Preg;
     v = v < e0 ? e0 : (v > a.E ? a.E : v);
     const int64_t rel = v - e0;
-    if (lane <= kWChunk) buf[lane] = rel > 0x3fffffff ? 0x3fffffff : (int)rel;
-    if (lane == 1) { buf[52] = (int)(uint32_t)e0; buf[53] = (int)(uint32_t)((uint64_t)e0 >> 32); }
+    const int rel32 = rel > 0x3fffffff ? 0x3fffffff : (int)rel;
+    if (lane <= kWChunk) buf[lane] = rel32;
+    if constexpr (SCALAR_BOUNDS) {
+      const int b0 = __builtin_amdgcn_readlane(rel32, 0), b1 = __builtin_amdgcn_readlane(rel32, 4);
+      const int b2 = __builtin_amdgcn_readlane(rel32, 8), b3 = __builtin_amdgcn_readlane(rel32, 12);
+      if (which) { sb1[0] = b0; sb1[1] = b1; sb1[2] = b2; sb1[3] = b3; se0[1] = e0; }
+      else { sb0[0] = b0; sb0[1] = b1; sb0[2] = b2; sb0[3] = b3; se0[0] = e0; }
+    } else {
+      if (lane == 1) { buf[52] = (int)(uint32_t)e0; buf[53] = (int)(uint32_t)((uint64_t)e0 >> 32); }
+    }
   };
   // bounds of mini-block m of the chunk in buffer `which`: first edge (relative to the chunk's e0)
   // and edge count
   auto bounds = [&](int which, int m, int& eb, int& ne) {
-    const int* buf = s_ptr + which * kWPtr;
-    eb = uni(buf[m * RPM]);
-    const int ee = uni(buf[m * RPM + RPM]);
+    int ee;
+    if constexpr (SCALAR_BOUNDS) {
+      const int c0 = which ? sb1[0] : sb0[0], c1 = which ? sb1[1] : sb0[1];
+      const int c2 = which ? sb1[2] : sb0[2], c3 = which ? sb1[3] : sb0[3];
+      eb = m == 0 ? c0 : (m == 1 ? c1 : c2);
+      ee = m == 0 ? c1 : (m == 1 ? c2 : c3);
+    } else {
+      const int* buf = s_ptr + which * kWPtr;
+      eb = uni(buf[m * RPM]);
+      ee = uni(buf[m * RPM + RPM]);
+    }
     ne = ee - eb;
     ne = ne < 0 ? 0 : ne;
   };
   auto chunk_e0 = [&](int which) {
-    const int* buf = s_ptr + which * kWPtr;
-    const uint32_t lo = (uint32_t)uni(buf[52]), hi = (uint32_t)uni(buf[53]);
-    return (int64_t)(((uint64_t)hi << 32) | lo);
+    if constexpr (SCALAR_BOUNDS) {
+      return which ? se0[1] : se0[0];
+    } else {
+      const int* buf = s_ptr + which * kWPtr;
+      const uint32_t lo = (uint32_t)uni(buf[52]), hi = (uint32_t)uni(buf[53]);
+      return (int64_t)(((uint64_t)hi << 32) | lo);
+    }
   };
 
   // Start-up.  A launch over few rows is mostly this: 128 KB of codebook per CU and three dependent
@@ -433,7 +460,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     bool on = has_rows && ne0 <= kWEdges && lane < ne0;
     {
       const Idx* src = on ? indices + e0 + eb0 + lane : indptr;
-      Ireg = (int64_t)*src;                                   // I(0)
+      Ireg = (int64_t)*src;                                // I(0)
     }
     float4 cbv[8];
     stage_codebook_load<kThreads>(cbv, a.codebooks, a.K, a.w, tile, tile_cols);
@@ -447,7 +474,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       if (v) bounds(0, 1, eb1, ne1);
       on = v && ne1 <= kWEdges && lane < ne1;
       const Idx* src = on ? indices + e0 + eb1 + lane : indptr;
-      Ireg = (int64_t)*src;                                   // I(1)
+      Ireg = (int64_t)*src;                                // I(1)
     }
     stage_codebook_store<kThreads, H == 2>(s_cb, cbv, a.K);
     __syncthreads();
@@ -480,13 +507,17 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   if constexpr (TRACE) t_first = wall_clock64();
   int eb2 = 0, ne2 = 0;
   // the load stages of step g at position m of its chunk: park C(g), issue C(g+1), issue I(g+2)
+  // Every lane always loads: a lane beyond the mini-block's edges reads its last edge again (and
+  // with no mini-block to load for, the first row offset, which is a valid id once clamped), so the
+  // id a lane holds is always one whose code row may be read, and neither load needs a per-lane
+  // choice of address: the ids come from a uniform base plus a 32-bit lane offset, the code bytes of
+  // every lane are parked whether the mini-block uses them or not.
   auto front = [&](int64_t g, int m) {
-    if (g >= 0 && ne0 <= kWEdges && lane < ne0) *reinterpret_cast<CW*>(s_codes + lane * BT) = Creg;
-    {  // C(g+1): the id fetched one step ago is clamped only now
-      const bool on = g + 1 >= 0 && g + 1 < n_mini && ne1 <= kWEdges && lane < ne1;
+    if (g >= 0) *reinterpret_cast<CW*>(s_codes + lane * BT) = Creg;
+    {  // C(g+1): the id fetched one step ago is clamped only now (ids outside [0, N) read row N - 1)
       const uint64_t raw = (uint64_t)Ireg;
       const uint32_t id = (raw >> 32) ? n_last : ((uint32_t)raw < n_last ? (uint32_t)raw : n_last);
-      Creg = *reinterpret_cast<const CW*>(code_base + (uint64_t)(on ? id : 0u) * (uint32_t)a.n_cb);
+      Creg = *reinterpret_cast<const CW*>(code_base + (uint64_t)id * (uint32_t)a.n_cb);
     }
     eb2 = 0; ne2 = 0;
     {  // I(g+2)
@@ -498,9 +529,11 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
         bounds(which, over ? m + 2 - kMini : m + 2, eb2, ne2);
         e0 = chunk_e0(which);
       }
-      const bool on = v && ne2 <= kWEdges && lane < ne2;
-      const Idx* src = on ? indices + e0 + eb2 + lane : indptr;
-      Ireg = (int64_t)*src;
+      const bool ok = v && ne2 <= kWEdges && ne2 > 0;
+      const char* base = reinterpret_cast<const char*>(ok ? indices + e0 + eb2 : indptr);
+      const uint32_t last = ok ? (uint32_t)(ne2 - 1) : 0u;
+      const uint32_t li = (uint32_t)lane < last ? (uint32_t)lane : last;
+      Ireg = (int64_t)*reinterpret_cast<const Idx*>(base + li * (uint32_t)sizeof(Idx));
     }
   };
   // start-up without the early loads (large or unaligned codebooks): two steps that only load
@@ -546,16 +579,40 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       // in edge order; returns the row's edge count
       auto row_sum = [&](int row, int sub, float (&acc)[H][4]) -> int {
         int rb = buf[row] - eb0, re = buf[row + 1] - eb0;
-#pragma unroll
-        for (int h = 0; h < H; ++h) acc[h][0] = acc[h][1] = acc[h][2] = acc[h][3] = 0.f;
         int n;
         if (staged) {
-          rb = rb < 0 ? 0 : (rb > ne0 ? ne0 : rb);
-          re = re < 0 ? 0 : (re > ne0 ? ne0 : re);
+          rb = min(max(rb, 0), ne0);
+          re = min(max(re, 0), ne0);
           n = re - rb;
           const int ns = n > sub ? (n - sub + SPR - 1) / SPR : 0;   // edges of this slot
           const unsigned char* cp = s_codes + (rb + sub) * BT + byte_idx;
           int k = 0;
+          if (ns >= kGroup) {
+            // the first group starts the sums (0 + x is x: the same values as adding to zero)
+            uint32_t code[kGroup];
+            float4 x[kGroup][H];
+#pragma unroll
+            for (int u = 0; u < kGroup; ++u) code[u] = cp[u * SPR * BT];
+            cp += kGroup * SPR * BT;
+#pragma unroll
+            for (int u = 0; u < kGroup; ++u)
+#pragma unroll
+              for (int h = 0; h < H; ++h) x[u][h] = *reinterpret_cast<const float4*>(cbp + code[u] * 128 + h * 64);
+#pragma unroll
+            for (int h = 0; h < H; ++h) {
+              acc[h][0] = x[0][h].x; acc[h][1] = x[0][h].y; acc[h][2] = x[0][h].z; acc[h][3] = x[0][h].w;
+            }
+#pragma unroll
+            for (int u = 1; u < kGroup; ++u)
+#pragma unroll
+              for (int h = 0; h < H; ++h) {
+                acc[h][0] += x[u][h].x; acc[h][1] += x[u][h].y; acc[h][2] += x[u][h].z; acc[h][3] += x[u][h].w;
+              }
+            k = kGroup;
+          } else {
+#pragma unroll
+            for (int h = 0; h < H; ++h) acc[h][0] = acc[h][1] = acc[h][2] = acc[h][3] = 0.f;
+          }
           for (; k + kGroup <= ns; k += kGroup) {
             uint32_t code[kGroup];
             float4 x[kGroup][H];
@@ -583,6 +640,8 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
             }
           }
         } else {
+#pragma unroll
+          for (int h = 0; h < H; ++h) acc[h][0] = acc[h][1] = acc[h][2] = acc[h][3] = 0.f;
           n = re - rb;
           const int64_t e0 = chunk_e0(par) + eb0;
           for (int k = sub; k < n; k += SPR) {
@@ -621,7 +680,8 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
         const int n = row_sum(row, 0, acc);
         mean(n, acc);
         float4* stg = reinterpret_cast<float4*>(s_codes);
-        float* obase = out + (row0 + row) * (int64_t)a.feat_dim + tile * 128;
+        char* obase = reinterpret_cast<char*>(out + row0 * (int64_t)a.feat_dim + tile * 128);   // uniform
+        const uint32_t orow_b = (uint32_t)row * ((uint32_t)a.feat_dim * 4u);
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
           __builtin_amdgcn_wave_barrier();
@@ -638,10 +698,11 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
           const int last = tile_cols - 4;                  // first column of the tile's last float4
           col = col < last ? col : last;
           const float4 v = stg[half * 16 + ((col & 63) >> 2)];
-          store_nt4(obase + col, v.x, v.y, v.z, v.w);
+          store_nt4(reinterpret_cast<float*>(obase + (orow_b + 4u * (uint32_t)col)), v.x, v.y, v.z, v.w);
         }
       } else {
-        float* orow = out + row0 * (int64_t)a.feat_dim + tile * 128 + col0;
+        // uniform base + 32-bit byte offset of the lane: no 64-bit address arithmetic per lane
+        char* obase = reinterpret_cast<char*>(out + row0 * (int64_t)a.feat_dim + tile * 128);
 #pragma unroll
         for (int pass = 0; pass < kPasses; ++pass) {
           const int slot = pass * kRowsPerPass + half;
@@ -663,9 +724,12 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
 #ifdef F2CGT_EXPERIMENTS
           if (a.dense_store == 2 && acc[0][0] != 12345.678f) continue;   // no stores: what the rest of the kernel costs
 #endif
+          // the lane's two 16-byte stores: one address, the second 16 bytes on as an immediate offset,
+          // so that they are issued back to back (see above)
+          const uint32_t off_b = (uint32_t)row * ((uint32_t)a.feat_dim * 4u) + 4u * (uint32_t)col0;
+          float* dst = reinterpret_cast<float*>(obase + off_b);
 #pragma unroll
-          for (int h = 0; h < H; ++h)
-            store_nt4(orow + (int64_t)row * a.feat_dim + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+          for (int h = 0; h < H; ++h) store_nt4(dst + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
         }
       }
     }
