@@ -22,6 +22,7 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 HIP_SOURCES = ["runtime.hip", "packbits.hip", "sq.hip", "vq.hip", "spmm.hip", "spmm_fast.hip",
                "vq_fast.hip", "encode.hip", "fetch.hip", "kmeans.hip"]
+EXPERIMENT_SOURCES = ["overlap_probe.hip"]   # compiled into the --experiments build only
 HIP_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -71,6 +72,8 @@ def build_capi(verbose=True, experiments=False):
     os.makedirs(OBJ, exist_ok=True)
     hipcc = shutil.which("hipcc") or os.path.join(ROCM, "bin", "hipcc")
     sources = [s for s in HIP_SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    if experiments:
+        sources += [s for s in EXPERIMENT_SOURCES if os.path.exists(os.path.join(CSRC, s))]
     optional = _optional_flags(hipcc, verbose)
 
     def compile_one(src):

@@ -3,6 +3,7 @@
 
     python3 -m f2cgt_amd.experiments wave-age c3|c5      per-wave start / first step / end of vq_wave_kernel
     python3 -m f2cgt_amd.experiments block-phases c1|c2  per-workgroup phase times of sq_affine_acc_kernel
+    python3 -m f2cgt_amd.experiments mfma-overlap x      fp32 MFMA and LDS-gather work on one SIMD: side by side or one after the other?
 
 Both run the workload of `bench.py --workload <w>` warm, switch the trace buffer on for a few launches and
 print percentiles of the last one (times in us from the earliest stamp of the launch; the stamps are
@@ -113,8 +114,52 @@ def block_phases(name):
     print("  distinct CUs: %d, workgroups per CU min / mean / max: %d / %.1f / %d" % (len(count), count.min(), count.mean(), count.max()))
 
 
+def mfma_overlap(_):
+    """Times the four arrangements of csrc/overlap_probe.hip on every CU and prints what each costs."""
+    import torch
+
+    sys.path.insert(0, ROOT)
+    from f2cgt_amd import capi
+
+    lib = capi.lib()
+    if not hasattr(lib, "f2cgt_experiment_overlap_probe"):
+        raise SystemExit("the library in tree was built without --experiments")
+    fn = lib.f2cgt_experiment_overlap_probe
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    fn.restype = ctypes.c_int
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    out = torch.zeros((cus,), device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    iters = 4000
+    names = ["mfma        (4 waves: 8 x v_mfma_f32_32x32x2_f32 per trip)", "gather      (4 waves: 8 x ds_read_b128 + 32 adds per trip)",
+             "split       (8 waves: 4 mfma + 4 gather, sharing the SIMDs)", "mixed       (4 waves, both kinds from one loop)",
+             "lds         (4 waves: the 8 reads alone)", "adds        (4 waves: the 32 adds alone)",
+             "split-lds   (8 waves: 4 mfma + 4 lds)", "split-adds  (8 waves: 4 mfma + 4 adds)"]
+    times = []
+    for arr in range(8):
+        for _ in range(3):
+            assert fn(out.data_ptr(), cus, iters, arr, stream) == 0
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+            assert fn(out.data_ptr(), cus, iters, arr, stream) == 0
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1) / 5 * 1e3)
+    for name, t in zip(names, times):
+        print("  %-62s %8.1f us  (%.0f ns per trip)" % (name, t, t * 1e3 / iters))
+    print("  sum of mfma and gather %.1f us, larger of the two %.1f us: split is %.2f of the sum, mixed %.2f"
+          % (times[0] + times[1], max(times[0], times[1]), times[2] / (times[0] + times[1]), times[3] / (times[0] + times[1])))
+    print("  mfma + lds: %.2f of the sum; mfma + adds: %.2f of the sum"
+          % (times[6] / (times[0] + times[4]), times[7] / (times[0] + times[5])))
+    flops = 2.0 * 32 * 32 * 2 * 8 * iters * 4 * cus
+    print("  mfma alone: %.1f TFLOP/s fp32; in split: %.1f" % (flops / times[0] / 1e6, flops / times[2] / 1e6))
+
+
 if __name__ == "__main__":
-    if len(sys.argv) != 3 or sys.argv[1] not in ("wave-age", "block-phases"):
+    modes = {"wave-age": wave_age, "block-phases": block_phases, "mfma-overlap": mfma_overlap}
+    if len(sys.argv) != 3 or sys.argv[1] not in modes:
         print(__doc__)
         sys.exit(2)
-    (wave_age if sys.argv[1] == "wave-age" else block_phases)(sys.argv[2])
+    modes[sys.argv[1]](sys.argv[2])
