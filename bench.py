@@ -1,6 +1,6 @@
 """Benchmark of the fused decompress + mean-aggregation hot path on one MI355X.
 
-    python bench.py [--steps K] [--warmup W] [--workload c2|c1|c3|c4|c5] [--idx int64|int32]
+    python bench.py [--steps K] [--warmup W] [--workload c2|c1|c3|c4|c5 [--scatter]] [--idx int64|int32]
 
 Prints ONE JSON line.  A step is one launch of the fused operator over one synthetic CSC
 block, inputs resident in HBM, through the C ABI (caller-allocated output).  `value` is
@@ -113,12 +113,14 @@ def _time_steps(step, steps, warmup):
     return wall * 1e3 / steps, ev0.elapsed_time(ev1) / steps
 
 
-def _run_workload(name, idx, steps, warmup):
+def _run_workload(name, idx, steps, warmup, scattered=False):
     import torch
     from f2cgt_amd import capi, synth
 
     idx_dtype = torch.int64 if idx == "int64" else torch.int32
     wl = synth.WORKLOADS[name](device="cuda", idx_dtype=idx_dtype)
+    if scattered:
+        wl = synth.scatter_ids(wl)
     out = torch.empty((wl["R"], wl["feat_dim"]), dtype=torch.float32, device="cuda")
     ms_step, ms_launch = _time_steps(_launcher(capi, wl, out), steps, warmup)
     return wl, ms_step, ms_launch
@@ -412,6 +414,8 @@ def main():
     ap.add_argument("--configs", default="auto", choices=["auto", "on", "off"],
                     help="the other configurations and the cold-cache headline in the same line "
                          "(auto: on unless --workload is given)")
+    ap.add_argument("--scatter", action="store_true",
+                    help="with --workload: pass the source ids through a fixed bijection (hot rows no longer neighbours)")
     ap.add_argument("--idx", default="int64", choices=["int64", "int32"])
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the cpu_baseline leg (0 = skip)")
     ap.add_argument("--all", action="store_true", help="also measure the other workloads and ops")
@@ -438,8 +442,10 @@ def main():
         return
 
     with_configs = args.configs == "on" or (args.configs == "auto" and args.workload is None)
+    if args.scatter and args.workload is None:
+        ap.error("--scatter needs --workload (the headline line is measured on the workload as generated)")
     args.workload = args.workload or "c2"
-    wl, ms_per_step, launch_ms = _run_workload(args.workload, args.idx, args.steps, args.warmup)
+    wl, ms_per_step, launch_ms = _run_workload(args.workload, args.idx, args.steps, args.warmup, args.scatter)
     achieved = wl["algo_bytes"] / (launch_ms * 1e-3) / 1e9
     traffic = _measured_traffic(wl["name"], args.idx)
     fr = _fractions(wl, launch_ms, traffic)

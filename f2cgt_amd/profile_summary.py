@@ -3,7 +3,8 @@ HBM-traffic record profiles/traffic.json that bench.py reads.
 
     python3 -m f2cgt_amd.profile_summary <rocprof_out_dir> [<profiles_dir>]
 
-Nothing is run here.  <rocprof_out_dir> is expected to hold, per workload w in c1..c5, the output
+Nothing is run here.  <rocprof_out_dir> is expected to hold, per workload w in c1..c5 and c3s (c3 with
+`--scatter`), the output
 directories of these runs (`cd /tmp && export TMPDIR=/tmp` first, every run on its own, from the
 repository root; B = `python3 bench.py --workload <w> --steps 2000 --warmup 200 --cpu-seconds 0`,
 with 300 steps for c4 and c5 (30 and 100 warm-up launches); T = B except for c2, where T = `python3 bench.py --workload c2
@@ -45,19 +46,23 @@ WORKLOADS = {
     "c3": ("vq_wave_kernel", "c3_vq_16x8"),
     "c4": ("hybrid_acc_kernel", "c4_hybrid"),
     "c5": ("vq_wave_kernel", "c5_vq_24x32"),
+    "c3s": ("vq_wave_kernel", "c3_vq_16x8_scattered"),
 }
-STEPS = {"c1": (2000, 200), "c2": (2000, 200), "c3": (2000, 200), "c4": (300, 30), "c5": (300, 100)}
+STEPS = {"c1": (2000, 200), "c2": (2000, 200), "c3": (2000, 200), "c4": (300, 30), "c5": (300, 100),
+         "c3s": (2000, 200)}
 N_SIMD, N_XCD, N_CU = 1024, 8, 256
 
 
+FUSED_SOURCES = ("common.hpp", "spmm.hip", "spmm_fast.hip", "spmm_fast.hpp", "vq_fast.hip")
+
+
 def csrc_sha16():
-    """Content hash of the kernel sources (*.hip, *.hpp): a traffic figure belongs to the kernels it was
-    measured on."""
+    """Content hash of the sources of the fused aggregation kernels and their dispatch: a traffic
+    figure belongs to the kernels it was measured on."""
     h = hashlib.sha256()
-    for path in sorted(glob.glob(os.path.join(PKG, "csrc", "*"))):
-        if os.path.isfile(path) and path.endswith((".hip", ".hpp")):
-            h.update(os.path.basename(path).encode())
-            h.update(open(path, "rb").read())
+    for name in FUSED_SOURCES:
+        h.update(name.encode())
+        h.update(open(os.path.join(PKG, "csrc", name), "rb").read())
     return h.hexdigest()[:16]
 
 
@@ -65,7 +70,8 @@ def bench_cmd(w, short=False):
     if w == "c2" and short:
         return "python3 bench.py --workload c2 --steps 20 --warmup 5 --cpu-seconds 0"
     steps, warm = STEPS[w]
-    return "python3 bench.py --workload %s --steps %d --warmup %d --cpu-seconds 0" % (w, steps, warm)
+    name = "c3 --scatter" if w == "c3s" else w
+    return "python3 bench.py --workload %s --steps %d --warmup %d --cpu-seconds 0" % (name, steps, warm)
 
 
 def kstats(d, match):
@@ -150,11 +156,12 @@ def write_workload(O, P, w, scales, traffic_out):
                 fh.write("Short run (`--warmup 5 --steps 20`, what a fresh process sees): the 20 timed dispatches avg %.2f us, "
                          "min %.2f, max %.2f" % (sum(last) / len(last), min(last), max(last)))
                 if b20:
-                    fh.write("; bench.py in that run: launch %.2f us, frac %.3f" % (b20["roofline"]["launch_us"], b20["roofline"]["frac"]))
+                    fh.write("; bench.py in that run: launch %.2f us" % b20["roofline"]["launch_us"])
                 fh.write(".\n\n")
         if b:
             fh.write("bench.py in the same run (HIP events on the launch stream): launch %.2f us, %.0f GB/s algorithmic, "
-                     "frac %.3f\n\n" % (b["roofline"]["launch_us"], b["roofline"]["achieved"], b["roofline"]["frac"]))
+                     "%.3f of the 8 TB/s peak\n\n" % (b["roofline"]["launch_us"], b["roofline"]["achieved"],
+                                                      b["roofline"]["achieved"] / 8000.0))
         if fc and wc and b:
             algo = b["config"]["algorithmic_bytes"]
             traffic = (fc[0] * fs + wc[0] * ws) * 1024
