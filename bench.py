@@ -13,11 +13,14 @@ box's host cores on a bounded sample of the same workload.
 Every benchmark configuration is in that one line: next to the headline workload's `roofline`,
 `configs` holds the other fused workloads (C1, C3, C3 with scattered ids, C4, C5) and the C5 encode
 step, each with its own launch count, `launch_us`, `edges_per_s`, `algorithmic_bytes`,
-`compulsory_bytes`, measured HBM `traffic` and three fractions of the 8 TB/s peak:
-`frac_algorithmic` (every edge charged its source row), `frac_compulsory` (every distinct source
-row charged once: a bound no cache can beat, so it cannot exceed 1) and `frac`, which is
-`min(frac_algorithmic, 1)` when the launch really moves >= 0.9 of the algorithmic bytes through
-HBM and `frac_compulsory` otherwise.  The headline's `roofline.frac_cold` is the same kernel
+`compulsory_bytes`, measured HBM `traffic` and four fractions of the 8 TB/s peak:
+`frac_algorithmic` (every edge charged its source row), `frac_traffic` (the bytes the counters saw
+move through HBM in such a launch: a physical rate, so it cannot exceed 1), `frac_compulsory` (every
+distinct source row charged once: what no cache can avoid) and `frac`, the lesser of
+`frac_algorithmic` and `frac_traffic` (a launch whose hot rows hit in cache is not credited with
+bytes it never moved; one that re-reads is not credited with its re-reads).  Without a traffic
+figure for these kernel sources `frac` is `min(frac_algorithmic, 1)` when the distinct rows make up
+>= 0.9 of the algorithmic bytes and `frac_compulsory` otherwise.  The headline's `roofline.frac_cold` is the same kernel
 with six CSC blocks and six outputs in rotation (> 600 MB pass before a buffer comes round again,
 more than the 256 MB last-level cache).  `--workload X` measures X alone (what the rocprofv3
 runs use); `--configs off` drops the extra objects.
@@ -127,19 +130,20 @@ def _run_workload(name, idx, steps, warmup, scattered=False):
 
 
 def _fractions(wl, launch_ms, traffic):
-    """The three fractions of the HBM peak for one fused launch (see the module docstring)."""
+    """The fractions of the HBM peak for one fused launch (see the module docstring)."""
     from f2cgt_amd import synth
 
     secs = launch_ms * 1e-3
     algo, comp = wl["algo_bytes"], synth.compulsory_bytes(wl)
     f_algo = algo / secs / 1e9 / HBM_PEAK_GBS
     f_comp = comp / secs / 1e9 / HBM_PEAK_GBS
-    # how much of the algorithmic bytes really moves: the measured traffic where there is a figure
-    # for these kernel sources, else what the distinct rows say
-    moved = (traffic if traffic is not None else comp) / algo
-    frac = min(f_algo, 1.0) if moved >= 0.9 else f_comp
+    f_traffic = traffic / secs / 1e9 / HBM_PEAK_GBS if traffic is not None else None
+    if f_traffic is not None:
+        frac = min(f_algo, f_traffic)
+    else:
+        frac = min(f_algo, 1.0) if comp / algo >= 0.9 else f_comp
     return {"algorithmic_bytes": algo, "compulsory_bytes": comp, "traffic": traffic,
-            "frac_algorithmic": f_algo, "frac_compulsory": f_comp, "frac": frac}
+            "frac_algorithmic": f_algo, "frac_traffic": f_traffic, "frac_compulsory": f_comp, "frac": frac}
 
 
 def _cold_launch_ms(name, idx, wl, blocks=6, rounds=40, warm_rounds=10):
@@ -400,6 +404,37 @@ def _others(idx):
     fetch_case("fetch_rows_50B_pinned_host_1M", host_table, count=1_000_000)
     fetch_case("fetch_rows_50B_pinned_host_1M_quarter_cached", host_table, packed[hot_ids].contiguous(), slot,
                count=1_000_000)
+    del host_table, feats, packed, slot, hot_ids
+    torch.cuda.empty_cache()
+    # a minibatch as the training loop sees it (examples/tensor_cache.py:49-58 then the fused operator):
+    # the block's distinct source ids are fetched into a gathered copy and aggregated through block-local
+    # ids, against the fused operator reading the device-resident table through global ids
+    for name in ("c2", "c3"):
+        wl = synth.WORKLOADS[name](device="cuda", idx_dtype=torch.int64)
+        input_nodes, local = torch.unique(wl["indices"], return_inverse=True)
+        codes = wl["codes"]
+        gathered = torch.empty((input_nodes.numel(), codes.shape[1]), dtype=codes.dtype, device="cuda")
+        out = torch.empty((wl["R"], wl["feat_dim"]), dtype=torch.float32, device="cuda")
+        local_wl = dict(wl, codes=gathered, indices=local.contiguous(), N=int(input_nodes.numel()))
+        fused_local, fused_global = _launcher(capi, local_wl, out), _launcher(capi, wl, out)
+        ids = torch.empty_like(wl["indices"])
+
+        def two_step():
+            capi.fetch_rows(codes, input_nodes, None, None, out=gathered)
+            fused_local()
+
+        def on_global_ids():
+            torch.index_select(input_nodes, 0, local, out=ids)      # compose block-local ids into global ones
+            fused_global()
+
+        _, t2 = _time_steps(two_step, 200, 50)
+        _, tg = _time_steps(on_global_ids, 200, 50)
+        _, t0 = _time_steps(fused_global, 200, 50)
+        res[wl["name"] + "_minibatch_flow"] = {
+            "distinct_source_rows": int(input_nodes.numel()), "fetch_then_aggregate_us": t2 * 1e3,
+            "compose_ids_then_aggregate_global_us": tg * 1e3, "aggregate_on_given_global_ids_us": t0 * 1e3}
+        del wl, local_wl, gathered, out, ids, local, input_nodes, codes
+        torch.cuda.empty_cache()
     return res
 
 
@@ -466,7 +501,8 @@ def main():
                    "src_rows": wl["N"], "feat_dim": wl["feat_dim"], "algorithmic_bytes": wl["algo_bytes"]},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": fr["frac"], "traffic": traffic, "launch_us": launch_ms * 1e3,
-                     "frac_algorithmic": fr["frac_algorithmic"], "frac_compulsory": fr["frac_compulsory"],
+                     "frac_algorithmic": fr["frac_algorithmic"], "frac_traffic": fr["frac_traffic"],
+                     "frac_compulsory": fr["frac_compulsory"],
                      "compulsory_bytes": fr["compulsory_bytes"]},
         "cpu_baseline": None,
     }

@@ -22,7 +22,7 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 HIP_SOURCES = ["runtime.hip", "packbits.hip", "sq.hip", "vq.hip", "spmm.hip", "spmm_fast.hip",
                "vq_fast.hip", "encode.hip", "fetch.hip", "kmeans.hip"]
-EXPERIMENT_SOURCES = ["overlap_probe.hip"]   # compiled into the --experiments build only
+EXPERIMENT_SOURCES = ["overlap_probe.hip", "lds_rate_probe.hip"]   # compiled into the --experiments build only
 HIP_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -4,8 +4,9 @@
     python3 -m f2cgt_amd.experiments wave-age c3|c5      per-wave start / first step / end of vq_wave_kernel
     python3 -m f2cgt_amd.experiments block-phases c1|c2  per-workgroup phase times of sq_affine_acc_kernel
     python3 -m f2cgt_amd.experiments mfma-overlap x      fp32 MFMA and LDS-gather work on one SIMD: side by side or one after the other?
+    python3 -m f2cgt_amd.experiments lds-rate x          bytes per clock and CU that conflict-free LDS reads return
 
-Both run the workload of `bench.py --workload <w>` warm, switch the trace buffer on for a few launches and
+The first two run the workload of `bench.py --workload <w>` warm, switch the trace buffer on for a few launches and
 print percentiles of the last one (times in us from the earliest stamp of the launch; the stamps are
 `wall_clock64()`, 100 MHz).
 """
@@ -157,8 +158,44 @@ def mfma_overlap(_):
     print("  mfma alone: %.1f TFLOP/s fp32; in split: %.1f" % (flops / times[0] / 1e6, flops / times[2] / 1e6))
 
 
+def lds_rate(_):
+    """Bytes per clock that the LDS of a CU returns to conflict-free reads of 16, 8 and 4 bytes per lane
+    (csrc/lds_rate_probe.hip: 16 waves per CU, the aggregation kernel's access shape)."""
+    import torch
+
+    sys.path.insert(0, ROOT)
+    from f2cgt_amd import capi
+
+    lib = capi.lib()
+    if not hasattr(lib, "f2cgt_experiment_lds_rate_probe"):
+        raise SystemExit("the library in tree was built without --experiments")
+    fn = lib.f2cgt_experiment_lds_rate_probe
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    fn.restype = ctypes.c_int
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    out = torch.zeros((cus,), dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    iters = 2000
+    for width, name in ((16, "ds_read_b128"), (8, "ds_read_b64"), (4, "ds_read_b32")):
+        for _ in range(2):
+            assert fn(out.data_ptr(), cus, iters, width, stream) == 0
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        assert fn(out.data_ptr(), cus, iters, width, stream) == 0
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3
+        clocks = out.cpu().numpy().astype("int64")
+        nbytes = 16 * 8 * iters * 64 * width                      # per CU: 16 waves x 8 reads per trip x 64 lanes
+        print("  %-13s launch %8.1f us; workgroup loop %d .. %d shader clocks (median %d): %.1f bytes per clock and CU, "
+              "%.2f clocks per wave instruction"
+              % (name, us, clocks.min(), clocks.max(), int(sorted(clocks)[len(clocks) // 2]),
+                 nbytes / float(sorted(clocks)[len(clocks) // 2]), float(sorted(clocks)[len(clocks) // 2]) / (16 * 8 * iters)))
+
+
 if __name__ == "__main__":
-    modes = {"wave-age": wave_age, "block-phases": block_phases, "mfma-overlap": mfma_overlap}
+    modes = {"wave-age": wave_age, "block-phases": block_phases, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate}
     if len(sys.argv) != 3 or sys.argv[1] not in modes:
         print(__doc__)
         sys.exit(2)
