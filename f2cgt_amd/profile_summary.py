@@ -193,7 +193,8 @@ def write_workload(O, P, w, scales, traffic_out):
                     fh.write("; vector ALU busy %.2f (4 clk per wave instruction on %d SIMDs)" % (v[0] * 4 / N_SIMD / clk, N_SIMD))
                 l = merged.get("SQ_LDS_IDX_ACTIVE")
                 if l:
-                    fh.write("; LDS busy %.2f (SQ_LDS_IDX_ACTIVE / %d CUs)" % (l[0] / N_CU / clk, N_CU))
+                    fh.write("; LDS address pipeline busy %.2f (SQ_LDS_IDX_ACTIVE / %d CUs; a `ds_read_b128` counts 4 clocks there "
+                             "and occupies the data return for 8, `profiles/lds_rate_probe_kernel_ds_read_widths.md`)" % (l[0] / N_CU / clk, N_CU))
                 fh.write(".\n")
     print(w, wl, "written")
 
