@@ -22,7 +22,9 @@ bytes it never moved; one that re-reads is not credited with its re-reads).  Wit
 figure for these kernel sources `frac` is `min(frac_algorithmic, 1)` when the distinct rows make up
 >= 0.9 of the algorithmic bytes and `frac_compulsory` otherwise.  The headline's `roofline.frac_cold` is the same kernel
 with six CSC blocks and six outputs in rotation (> 600 MB pass before a buffer comes round again,
-more than the 256 MB last-level cache).  `--workload X` measures X alone (what the rocprofv3
+more than the 256 MB last-level cache); `frac_cold_streaming` is that rotation with the output
+written by non-temporal stores (`f2cgt_set_store_mode(F2CGT_STORE_STREAM)`), which also takes the
+same time on one buffer (`cold.streaming_stores.one_buffer_launch_us`).  `--workload X` measures X alone (what the rocprofv3
 runs use); `--configs off` drops the extra objects.
 
     python bench.py --all            adds the other workloads and the streaming/encode ops
@@ -507,10 +509,24 @@ def main():
         "cpu_baseline": None,
     }
     if with_configs:
+        from f2cgt_amd import capi
+
         cold_ms, cold_bytes, nblk = _cold_launch_ms(args.workload, args.idx, wl)
         result["roofline"]["frac_cold"] = cold_bytes / (cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
         result["roofline"]["cold"] = {"launch_us": cold_ms * 1e3, "blocks_in_rotation": nblk,
                                       "algorithmic_bytes": cold_bytes}
+        # the same rotation, and the one-buffer loop, with the output streamed past the caches
+        was = capi.set_store_mode(capi.STORE_STREAM)
+        try:
+            s_cold_ms, _, _ = _cold_launch_ms(args.workload, args.idx, wl)
+            out = torch.empty((wl["R"], wl["feat_dim"]), dtype=torch.float32, device="cuda")
+            _, s_warm_ms = _time_steps(_launcher(capi, wl, out), 1000, 300)
+            del out
+        finally:
+            capi.set_store_mode(was)
+        result["roofline"]["frac_cold_streaming"] = cold_bytes / (s_cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+        result["roofline"]["cold"]["streaming_stores"] = {"launch_us": s_cold_ms * 1e3,
+                                                          "one_buffer_launch_us": s_warm_ms * 1e3}
 
     if args.cpu_seconds > 0:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))

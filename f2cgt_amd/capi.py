@@ -22,6 +22,7 @@ SIGNATURES = {
     "f2cgt_last_error": ([], c_char_p),
     "f2cgt_num_cus": ([], c_int),
     "f2cgt_set_plan_only": ([I], c_int),
+    "f2cgt_set_store_mode": ([I], c_int),
     "f2cgt_last_plan": ([P], c_int),
     "f2cgt_packbits": ([P, P, L, L, I, P], c_int),
     "f2cgt_unpackbits": ([P, P, L, L, L, I, P], c_int),
@@ -85,6 +86,18 @@ def dry_run(entry, *args):
 
 class F2CGTError(RuntimeError):
     pass
+
+
+STORE_AUTO, STORE_STREAM, STORE_CACHED = 0, 1, 2
+
+
+def set_store_mode(mode):
+    """Output store policy of the row-block SQ aggregation kernels (f2cgt_set_store_mode): returns the
+    previous mode."""
+    was = lib().f2cgt_set_store_mode(int(mode))
+    if was < 0:
+        raise F2CGTError("set_store_mode failed (%d): %s" % (was, lib().f2cgt_last_error().decode()))
+    return was
 
 
 def _check(rc, name):

@@ -85,7 +85,12 @@ __device__ __forceinline__ void row_range(const Idx* __restrict__ indptr, int64_
 // streamed past the caches with non-temporal stores: 4-bit affine aggregation, 400-byte rows,
 // 1e6 rows: 124 us plain, 94 us non-temporal; 5e5 rows: 48 us plain, 51 us non-temporal.
 // The crossover measured with dense 16-byte-per-lane stores lies between 200 and 240 MB.
-inline bool stream_output(int64_t out_bytes) { return out_bytes > 220000000ll; }
+// That holds for a buffer that is written again while its lines are still cached.  With six
+// 100 MB outputs in rotation (nothing of a buffer left in the cache when its turn comes) the plain
+// form takes 32.7 us per launch and the non-temporal one 27.7 us, which is also what it takes on
+// one buffer: the streamed form does not depend on the cache state.  The size rule is therefore
+// only the default (F2CGT_STORE_AUTO); f2cgt_set_store_mode overrides it either way.
+bool stream_output(int64_t out_bytes);
 
 // Non-temporal stores: the aggregation output is written once and never re-read by
 // the kernel, so it should not displace gathered code rows from L2 / MALL.

@@ -701,6 +701,19 @@ torch::Tensor vq_encode(torch::Tensor x, torch::Tensor centers, std::string metr
 
 }  // namespace
 
+// Output store policy of the SQ aggregation operators: "auto" (by output size), "stream"
+// (non-temporal stores whatever the size) or "cached" (plain stores); returns the previous one.
+std::string set_store_mode(const std::string& mode) {
+  static const char* names[] = {"auto", "stream", "cached"};
+  int want = -1;
+  for (int i = 0; i < 3; ++i)
+    if (mode == names[i]) want = i;
+  TORCH_CHECK(want >= 0, "set_store_mode: mode must be \"auto\", \"stream\" or \"cached\", got \"", mode, "\"");
+  const int was = f2cgt_set_store_mode(want);
+  TORCH_CHECK(was >= 0, f2cgt_last_error());
+  return names[was];
+}
+
 PYBIND11_MODULE(F2CGTLib, m) {
   m.doc() = "MI355X-native drop-in for F2CGT's F2CGTLib operator module";
   m.def("packbits", &packbits, py::arg("unpack"), py::arg("target_bits"))
@@ -741,7 +754,8 @@ PYBIND11_MODULE(F2CGTLib, m) {
       .def("fetch_rows", &fetch_rows, py::arg("table"), py::arg("index"), py::arg("hot") = py::none(),
            py::arg("slot_map") = py::none())
       .def("kmeans_update", &kmeans_update, py::arg("data"), py::arg("labels"), py::arg("centers"),
-           py::arg("stop") = py::none(), py::arg("rule") = 0, py::arg("tol") = 0.0);
+           py::arg("stop") = py::none(), py::arg("rule") = 0, py::arg("tol") = 0.0)
+      .def("set_store_mode", &set_store_mode, py::arg("mode"));
   py::class_<KMeans>(m, "KMeans")
       .def(py::init<int64_t, int64_t, std::string, int, double, int, double, int, int, bool>(),
            py::arg("n_cluster"), py::arg("feat_dim"), py::arg("metric"), py::arg("max_iter") = 300,

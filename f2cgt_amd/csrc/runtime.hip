@@ -27,6 +27,15 @@ void plan_record(const char* kernel, int64_t grid, int block, int64_t lds_bytes,
   t_plan.aux[0] = a0; t_plan.aux[1] = a1; t_plan.aux[2] = a2; t_plan.aux[3] = a3;
 }
 
+std::atomic<int> g_store_mode{F2CGT_STORE_AUTO};
+
+bool stream_output(int64_t out_bytes) {
+  const int mode = g_store_mode.load(std::memory_order_relaxed);
+  if (mode == F2CGT_STORE_STREAM) return true;
+  if (mode == F2CGT_STORE_CACHED) return false;
+  return out_bytes > 220000000ll;
+}
+
 int num_cus() {
   if (t_plan_only) return 256;   // a dry run must not depend on (or wake) a device
   static std::atomic<int> cached[64];   // 0 = not asked yet; callers may come from several threads
@@ -50,6 +59,13 @@ int f2cgt_version(void) { return 100; }
 const char* f2cgt_last_error(void) { return f2cgt::error_buffer(); }
 
 int f2cgt_num_cus(void) { return f2cgt::num_cus(); }
+
+int f2cgt_set_store_mode(int mode) {
+  if (mode != F2CGT_STORE_AUTO && mode != F2CGT_STORE_STREAM && mode != F2CGT_STORE_CACHED) {
+    return f2cgt::fail(F2CGT_E_INVALID, "set_store_mode: mode %d is none of AUTO, STREAM, CACHED", mode);
+  }
+  return f2cgt::g_store_mode.exchange(mode, std::memory_order_relaxed);
+}
 
 int f2cgt_set_plan_only(int on) {
   const int was = f2cgt::t_plan_only ? 1 : 0;

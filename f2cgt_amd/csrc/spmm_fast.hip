@@ -1179,6 +1179,9 @@ struct HybArgs {
   int rows_per_block, edge_batch;
   int chunks, ch2;   // 4-column chunks per row; gather lanes per edge = pow2 >= chunks
   uint32_t magic;
+#ifdef F2CGT_EXPERIMENTS
+  unsigned long long* trace;   // 8 words per workgroup: time stamps of its phases (100 MHz) and where it ran
+#endif
 };
 
 constexpr uint32_t kVqFlag = 0x80000000u;
@@ -1205,14 +1208,52 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
   uint16_t* s_erow = reinterpret_cast<uint16_t*>(s_row + a.edge_batch);      // [edge_batch] local row
 
   const int t = threadIdx.x;
+  ACC_STAMP(a, 0);
   const int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block;
   const int nrows = (int)((a.R - row0) < a.rows_per_block ? (a.R - row0) : a.rows_per_block);
+  // The column parameters are requested ahead of the row offsets, so that the two fetches of this
+  // phase share one round trip (issued behind the offsets' wait they made it two).
+  constexpr int NP = CH ? (CH * 4 + TB - 1) / TB : 1;
+  float par_min[NP], par_scale[NP];
+  if (CH) {
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int i = t + p * TB;
+      const int ic = i < CH * 4 ? i : CH * 4 - 1;
+      par_min[p] = a.sq_params[ic];
+      par_scale[p] = a.sq_params[a.param_stride + ic];
+    }
+  }
   int64_t e0 = (int64_t)indptr[row0];
   e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
+  // The source ids of the block's first PRE * TB edges are requested as soon as the block's first
+  // edge is known, next to the row offsets, and their row-map entries behind them, ahead of the
+  // barrier: the chain offsets -> ids -> row map of a block is then two round trips instead of
+  // three.  How many of these edges the block really has is known only after the barrier; a
+  // position beyond the edge array reads its last entry instead (nothing is read when it is empty).
+  constexpr int PRE = 2;
+  int64_t pre_id[PRE];
+#pragma unroll
+  for (int p = 0; p < PRE; ++p) pre_id[p] = 0;
+  if (a.E > 0) {   // one block around all of them: the loads go out back to back
+#pragma unroll
+    for (int p = 0; p < PRE; ++p) {
+      int64_t at = e0 + t + p * TB;
+      at = at < a.E ? at : a.E - 1;
+      pre_id[p] = (int64_t)indices[at];
+    }
+  }
   for (int i = t; i <= nrows; i += TB) {
     int64_t v = (int64_t)indptr[row0 + i];
     v = v < e0 ? e0 : (v > a.E ? a.E : v);
     s_ptr[i] = (int)(v - e0 > 0x7fffffff ? 0x7fffffff : v - e0);
+  }
+  int32_t pre_map[PRE];
+#pragma unroll
+  for (int p = 0; p < PRE; ++p) pre_map[p] = 0;
+  if (a.E > 0) {   // edges imply source rows
+#pragma unroll
+    for (int p = 0; p < PRE; ++p) pre_map[p] = a.row_map[clamp_idx(pre_id[p], a.N)];
   }
   for (int i = t; i < nrows * acc_pitch; i += TB) s_acc[i] = 0u;
   for (int i = t; i < nrows; i += TB) {
@@ -1220,23 +1261,41 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
     s_mask[2 * i] = 0u;
     s_mask[2 * i + 1] = 0u;
   }
-  for (int i = t; i < a.feat_dim; i += TB) {
-    const int c4 = i >> 2, q = i & 3;
-    s_par[c4 * 8 + q] = a.sq_params[i];
-    s_par[c4 * 8 + 4 + q] = a.sq_params[a.param_stride + i];
+  if (CH) {
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int i = t + p * TB;
+      if (i < CH * 4) {
+        const int c4 = i >> 2, q = i & 3;
+        s_par[c4 * 8 + q] = par_min[p];
+        s_par[c4 * 8 + 4 + q] = par_scale[p];
+      }
+    }
+  } else {
+    for (int i = t; i < a.feat_dim; i += TB) {
+      const int c4 = i >> 2, q = i & 3;
+      s_par[c4 * 8 + q] = a.sq_params[i];
+      s_par[c4 * 8 + 4 + q] = a.sq_params[a.param_stride + i];
+    }
   }
   __syncthreads();
+  ACC_STAMP(a, 1);
   const int ne = s_ptr[nrows];
   const uint32_t* codes32 = reinterpret_cast<const uint32_t*>(a.sq_codes);
-  const int dwords_per_row = a.feat_dim >> 2;
+  const int dwords_per_row = CH ? CH : a.feat_dim >> 2;   // CH chunks are CH dwords of 8-bit codes
 
   // rows longer than the field capacity are summed directly in the epilogue (flag: all edges "VQ-like")
   for (int eb = 0; eb < ne; eb += a.edge_batch) {
     const int nb = (ne - eb) < a.edge_batch ? (ne - eb) : a.edge_batch;
     if (eb) __syncthreads();
     for (int i = t; i < nb; i += TB) {
-      const int64_t id = clamp_idx(indices[e0 + eb + i], a.N);
-      const int64_t m = (int64_t)a.row_map[id];
+      int64_t m;
+      if (eb == 0 && i < PRE * TB) {
+        m = (int64_t)(i < TB ? pre_map[0] : pre_map[1]);
+      } else {
+        const int64_t id = clamp_idx(indices[e0 + eb + i], a.N);
+        m = (int64_t)a.row_map[id];
+      }
       uint32_t v;
       if (m >= 0) {
         v = (uint32_t)(m < a.n_sq ? m : a.n_sq - 1);
@@ -1263,6 +1322,7 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
       s_erow[i] = (uint16_t)lo;
     }
     __syncthreads();
+    if (eb == 0) ACC_STAMP(a, 2);
     if (VEC == 4) {
       // a lane takes 16 bytes (4 chunks) of an edge's code row: chunks / 4 lanes per edge
       const int lanes = ch2 >> 2;
@@ -1279,8 +1339,12 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
       const int e_end = (e_begin + per) < nb ? (e_begin + per) : nb;
       const int q = chunks >> 2;   // dwords per lane stride (chunks is a multiple of 4 here)
       const bool lane_on = j < q;
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      // every lane always loads: a lane without a row to fetch (an edge that is added in the epilogue,
+      // a lane beyond the row's chunks) reads the first 16 bytes of row 0, which the table has
+      const uint32_t* lane_codes = codes32 + (lane_on ? 4 * j : 0);
       for (int e = e_begin; e < e_end; e += U) {
-        uint32_t w[U][4];
+        u32x4 w[U];
         uint32_t row[U], er[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -1288,14 +1352,12 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
           ee = ee < e_end ? ee : e_end - 1;
           row[u] = s_row[ee];
           er[u] = s_erow[ee];
-          const bool on = lane_on && (row[u] >> 30) == 0;
-          typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-          const u32x4 zero4 = {0u, 0u, 0u, 0u};
-          const u32x4 v4 = on ? *reinterpret_cast<const u32x4*>(codes32 + (int64_t)row[u] * dwords_per_row + 4 * j)
-                              : zero4;
-#pragma unroll
-          for (int c = 0; c < 4; ++c) w[u][c] = v4[c];
+          const uint32_t r = (row[u] >> 30) == 0 ? row[u] : 0u;
+          w[u] = *reinterpret_cast<const u32x4*>(lane_codes + (uint64_t)r * (uint32_t)dwords_per_row);
         }
+        // the four loads are issued together and waited for together, whatever the adds below use
+#pragma unroll
+        for (int u = 0; u < U; ++u) asm volatile("" : "+v"(w[u]));
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const int ee = e + u;
@@ -1339,6 +1401,7 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
     }
   }
   __syncthreads();
+  ACC_STAMP(a, 3);
   // finalize: lane <-> one float4 of the block's contiguous output span
   const int items = nrows * chunks;
   float* ob = out + row0 * (int64_t)a.feat_dim;
@@ -1414,6 +1477,13 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
     if (deg <= 0) v0 = v1 = v2 = v3 = 0.f;
     store_nt4(ob + (int64_t)it * 4, v0, v1, v2, v3);
   }
+  ACC_STAMP(a, 4);
+#ifdef F2CGT_EXPERIMENTS
+  if (a.trace && threadIdx.x == 0) {
+    a.trace[(size_t)blockIdx.x * 8 + 5] = __builtin_amdgcn_s_getreg((31 << 11) | 4);    // HW_ID
+    a.trace[(size_t)blockIdx.x * 8 + 6] = __builtin_amdgcn_s_getreg((31 << 11) | 20);   // XCC_ID
+  }
+#endif
 }
 
 }  // namespace
@@ -1536,6 +1606,9 @@ int launch_hybrid(HybArgs a, const void* indptr, const void* indices, int idx_dt
   }
 #endif
   a.rows_per_block = rb;
+#ifdef F2CGT_EXPERIMENTS
+  a.trace = g_acc_trace;
+#endif
   const size_t lds = rb * acc_row + (size_t)a.chunks * 32 + (size_t)(rb + 4) * 4 + (size_t)rb * 4 + (size_t)rb * 8 +
                      (size_t)a.edge_batch * 6 + 16;
   const int64_t grid = ceil_div(a.R, rb);

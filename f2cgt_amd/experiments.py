@@ -2,7 +2,7 @@
 (the shipped build has neither the time-stamped kernel forms nor the entry points used here).
 
     python3 -m f2cgt_amd.experiments wave-age c3|c5      per-wave start / first step / end of vq_wave_kernel
-    python3 -m f2cgt_amd.experiments block-phases c1|c2  per-workgroup phase times of sq_affine_acc_kernel
+    python3 -m f2cgt_amd.experiments block-phases c1|c2|c4  per-workgroup phase times of sq_affine_acc_kernel / hybrid_acc_kernel
     python3 -m f2cgt_amd.experiments mfma-overlap x      fp32 MFMA and LDS-gather work on one SIMD: side by side or one after the other?
     python3 -m f2cgt_amd.experiments lds-rate x          bytes per clock and CU that conflict-free LDS reads return
 
@@ -83,12 +83,13 @@ def block_phases(name):
         raise SystemExit("the library in tree was built without --experiments")
     lib.f2cgt_experiment_set_acc_trace.argtypes = [ctypes.c_void_p]
     lib.f2cgt_experiment_set_acc_trace.restype = None
-    trace = torch.zeros((65536 * 8,), dtype=torch.int64, device="cuda")   # 8 words per workgroup
-    for _ in range(3000):
+    # 8 words per workgroup; the two-table kernel runs workgroups of at least 8 rows
+    trace = torch.zeros((max(65536, wl["R"] // 8 + 1) * 8,), dtype=torch.int64, device="cuda")
+    for _ in range(3000 if wl["R"] <= 300_000 else 100):
         step()
     torch.cuda.synchronize()
     lib.f2cgt_experiment_set_acc_trace(ctypes.c_void_p(trace.data_ptr()))
-    for _ in range(50):
+    for _ in range(50 if wl["R"] <= 300_000 else 5):
         step()
     torch.cuda.synchronize()
     lib.f2cgt_experiment_set_acc_trace(None)
@@ -104,9 +105,10 @@ def block_phases(name):
     print("  phase: source ids and tags   :", _q(T[:, 2] - T[:, 1]))
     print("  phase: gather of the code rows:", _q(T[:, 3] - T[:, 2]))
     print("  phase: finalize and store    :", _q(T[:, 4] - T[:, 3]))
-    for lo in np.arange(0.0, T[:, 4].max(), 1.0):
-        hi = lo + 1.0
-        print("  t = %2.0f .. %2.0f us: %5d workgroups resident, %5d started, %5d ended"
+    width = 1.0 if T[:, 4].max() < 60 else 10.0
+    for lo in np.arange(0.0, T[:, 4].max(), width):
+        hi = lo + width
+        print("  t = %3.0f .. %3.0f us: %5d workgroups resident, %5d started, %5d ended"
               % (lo, hi, ((T[:, 0] < hi) & (T[:, 4] > lo)).sum(), ((T[:, 0] >= lo) & (T[:, 0] < hi)).sum(),
                  ((T[:, 4] >= lo) & (T[:, 4] < hi)).sum()))
     hw, xcc = t[:, 5].astype(np.int64), t[:, 6].astype(np.int64) & 0xf

@@ -56,6 +56,22 @@ const char* f2cgt_last_error(void);
 /* Number of compute units of the current device (the kernels size their grids by it). */
 int f2cgt_num_cus(void);
 
+/* How the row-block aggregation kernels (the SQ and affine-SQ fused operators) write their output
+ * (no counterpart in the reference, whose kernels use plain stores, src/fusion_spmm.cu:173-236).
+ *   F2CGT_STORE_AUTO    (default) outputs above 220 MB are streamed past the caches with non-temporal
+ *                       stores, smaller ones are written with plain stores
+ *   F2CGT_STORE_STREAM  always streamed: the launch time no longer depends on what the caches hold
+ *   F2CGT_STORE_CACHED  never streamed
+ * Plain stores are fastest when the same output buffer is written again before the last-level cache
+ * (256 MB) has been turned over, as in a loop over one buffer; a caller whose outputs are written
+ * once and consumed later (a training step with other large kernels in between) is better off
+ * streaming.  Results are identical in every mode.  Process-wide; returns the previous mode, or
+ * F2CGT_E_INVALID for a value that is none of the three (the mode is then unchanged). */
+#define F2CGT_STORE_AUTO 0
+#define F2CGT_STORE_STREAM 1
+#define F2CGT_STORE_CACHED 2
+int f2cgt_set_store_mode(int mode);
+
 /* Dry runs of the fused aggregation entry points (no counterpart in the reference; for tests and
  * tools that want to know what a shape dispatches to, with or without a GPU).  While switched on
  * for the calling thread, f2cgt_spmm_csr and the f2cgt_*_spmm_csr operators validate their

@@ -57,6 +57,24 @@ def test_validation_rejects_before_device_work():
     assert lib.f2cgt_pairwise_distance(None, None, None, 5, 3, 8, 7, None) == E_INVALID
 
 
+def test_store_mode_setter_is_host_only_state():
+    lib = capi.lib()
+    was = capi.set_store_mode(capi.STORE_STREAM)
+    try:
+        assert was in (capi.STORE_AUTO, capi.STORE_STREAM, capi.STORE_CACHED)
+        assert capi.set_store_mode(capi.STORE_CACHED) == capi.STORE_STREAM
+        assert lib.f2cgt_set_store_mode(7) == -1 and b"store_mode" in lib.f2cgt_last_error()
+        assert capi.set_store_mode(capi.STORE_AUTO) == capi.STORE_CACHED       # a rejected value changes nothing
+        with pytest.raises(capi.F2CGTError):
+            capi.set_store_mode(-3)
+        module = f2cgt_amd.load()
+        assert module.set_store_mode("stream") == "auto" and module.set_store_mode("auto") == "stream"
+        with pytest.raises(RuntimeError, match="stream"):
+            module.set_store_mode("sometimes")
+    finally:
+        capi.set_store_mode(was)
+
+
 def test_extension_module_surface_matches_reference():
     lib = f2cgt_amd.load()
     import F2CGTLib  # registered under the reference's module name

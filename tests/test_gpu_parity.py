@@ -475,6 +475,33 @@ def test_fused_affine_vs_oracle(bits, d, idx):
         assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_store_mode_changes_no_result(bits):
+    """Plain, non-temporal and size-chosen output stores of the row-block SQ kernels write the same bits."""
+    rng = np.random.default_rng(bits)
+    N, R, d = 5000, 3000, 100
+    x = rng.standard_normal((N, d)).astype(np.float32)
+    params = oc.sq_affine_params(x, bits)
+    store = oc.sq_affine_compress(x, params, bits)
+    store = oc.packbits(store, bits) if bits < 8 else store
+    cbs = np.stack([oc.sq_codebook(x)])
+    log_store = oc.sq_codes_to_storage(oc.sq_compress(x, cbs, bits, d), bits)
+    indptr, indices = random_graph(rng, R, N, 12, np.int64)
+    s, p, ls, cb, ip, ix = dev(store), dev(params), dev(log_store), dev(cbs), dev(indptr), dev(indices)
+    was = capi.set_store_mode(capi.STORE_AUTO)
+    try:
+        results = []
+        for mode in (capi.STORE_AUTO, capi.STORE_STREAM, capi.STORE_CACHED):
+            capi.set_store_mode(mode)
+            results.append((host(capi.sq_affine_decompress_spmm_csr(s, p, ip, ix, bits, d)),
+                            host(capi.sq_decompress_spmm_csr(ls, cb, ip, ix, bits, d, d))))
+    finally:
+        capi.set_store_mode(was)
+    for affine, log_domain in results[1:]:
+        assert np.array_equal(affine, results[0][0]) and np.array_equal(log_domain, results[0][1])
+    assert np.array_equal(results[0][1], oc.sq_decompress_spmm_csr(log_store, cbs, indptr, indices, bits, d, d))
+
+
 @pytest.mark.parametrize("bits,d,max_deg", [(4, 100, 150), (8, 128, 120), (8, 64, 700), (4, 40, 5000)])
 def test_fused_affine_high_degree_rows(bits, d, max_deg):
     # many edge batches per row block, and rows beyond the 16-bit accumulator field capacity
