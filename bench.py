@@ -12,7 +12,8 @@ box's host cores on a bounded sample of the same workload.
 
 Every benchmark configuration is in that one line: next to the headline workload's `roofline`,
 `configs` holds the other fused workloads (C1, C3, C3 with scattered ids, C4, C5) and the C5 encode
-step, each with its own launch count, `launch_us`, `edges_per_s`, `algorithmic_bytes`,
+step, each with its own launch count, `launch_us` (and, for C3 / C4 / C5, `cold_launch_us` / `frac_cold`
+with three blocks and outputs in rotation), `edges_per_s`, `algorithmic_bytes`,
 `compulsory_bytes`, measured HBM `traffic` and four fractions of the 8 TB/s peak:
 `frac_algorithmic` (every edge charged its source row), `frac_traffic` (the bytes the counters saw
 move through HBM in such a launch: a physical rate, so it cannot exceed 1), `frac_compulsory` (every
@@ -193,6 +194,15 @@ def _configs(idx):
             entry = {"steps": steps, "warmup": warmup, "launch_us": ms_launch * 1e3,
                      "edges_per_s": wl["E"] / (ms_launch * 1e-3), "bound": "hbm"}
             entry.update(_fractions(wl, ms_launch, _measured_traffic(wl["name"], idx)))
+            if name in ("c3", "c4", "c5") and not scattered:
+                # three blocks and outputs in rotation (each output is 256 MB or more, so more than
+                # the last-level cache passes before a buffer comes round again)
+                del out
+                cold_ms, cold_bytes, nblk = _cold_launch_ms(name, idx, wl, blocks=3, rounds=max(4, steps // 6),
+                                                            warm_rounds=max(2, warmup // 6))
+                entry["cold_launch_us"] = cold_ms * 1e3
+                entry["frac_cold"] = cold_bytes / (cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+                out = None
             res[key] = entry
             del wl, out
         except RuntimeError as exc:
