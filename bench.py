@@ -201,7 +201,8 @@ def _configs(idx):
                 cold_ms, cold_bytes, nblk = _cold_launch_ms(name, idx, wl, blocks=3, rounds=max(4, steps // 6),
                                                             warm_rounds=max(2, warmup // 6))
                 entry["cold_launch_us"] = cold_ms * 1e3
-                entry["frac_cold"] = cold_bytes / (cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+                # the warm fraction scaled by the launch times (the blocks in rotation are the same size)
+                entry["frac_cold"] = entry["frac"] * ms_launch / cold_ms
                 out = None
             res[key] = entry
             del wl, out
