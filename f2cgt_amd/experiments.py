@@ -5,6 +5,7 @@
     python3 -m f2cgt_amd.experiments block-phases c1|c2|c4  per-workgroup phase times of sq_affine_acc_kernel / hybrid_acc_kernel
     python3 -m f2cgt_amd.experiments mfma-overlap x      fp32 MFMA and LDS-gather work on one SIMD: side by side or one after the other?
     python3 -m f2cgt_amd.experiments lds-rate x          bytes per clock and CU that conflict-free LDS reads return
+    python3 -m f2cgt_amd.experiments cold-parts c2|c3|c4|c5   launch time by what of the input is still cached (any build)
 
 The first two run the workload of `bench.py --workload <w>` warm, switch the trace buffer on for a few launches and
 print percentiles of the last one (times in us from the earliest stamp of the launch; the stamps are
@@ -196,8 +197,67 @@ def lds_rate(_):
                  nbytes / float(sorted(clocks)[len(clocks) // 2]), float(sorted(clocks)[len(clocks) // 2]) / (16 * 8 * iters)))
 
 
+def cold_parts(name):
+    """Which part of a launch's input has to be cached for the warm figure of a fused workload: the launch
+    with its graph in one or several copies of the index arrays, with other graphs, with other outputs, and
+    with a large unrelated read between two launches.  Needs no experiments build."""
+    import torch
+
+    sys.path.insert(0, ROOT)
+    import bench
+    from f2cgt_amd import capi, synth
+
+    wl = synth.WORKLOADS[name](device="cuda", idx_dtype=torch.int64)
+    outs = [torch.empty((wl["R"], wl["feat_dim"]), dtype=torch.float32, device="cuda") for _ in range(3)]
+
+    def timed(pairs, rounds=30, warm=8):
+        steps = [bench._launcher(capi, g, o) for g, o in pairs]
+
+        def one_round():
+            for st in steps:
+                st()
+
+        _, ms = bench._time_steps(one_round, rounds, warm)
+        return ms / len(steps) * 1e3
+
+    def copies(n, ids=True, ptr=True):
+        res = [wl]
+        for _ in range(n - 1):
+            g = dict(wl)
+            if ids:
+                g["indices"] = wl["indices"].clone()
+            if ptr:
+                g["indptr"] = wl["indptr"].clone()
+            res.append(g)
+        return res
+
+    timed([(wl, outs[0])] * 3, rounds=200)  # brings the clocks up before the first figure
+    print(name, "launch times in us")
+    print("  one graph, one output                          %7.1f" % timed([(wl, outs[0])] * 3))
+    print("  one graph, three outputs in rotation           %7.1f" % timed([(wl, o) for o in outs]))
+    for n in (2, 3, 4, 6):
+        print("  the graph in %d copies of indices and indptr     %7.1f" % (n, timed([(g, outs[0]) for g in copies(n)])))
+    print("  the graph in 6 copies of indptr only           %7.1f" % timed([(g, outs[0]) for g in copies(6, ids=False)]))
+    print("  the graph in 6 copies of indices only          %7.1f" % timed([(g, outs[0]) for g in copies(6, ptr=False)]))
+    others = synth.extra_blocks(wl, 2)
+    print("  three different graphs, one output             %7.1f" % timed([(g, outs[0]) for g in [wl] + others]))
+    print("  three different graphs, three outputs          %7.1f" % timed(list(zip([wl] + others, outs))))
+    del others
+    junk = torch.empty(512 * 1024 * 1024 // 4, dtype=torch.float32, device="cuda")
+    step = bench._launcher(capi, wl, outs[0])
+
+    def with_junk():
+        junk.sum()
+        step()
+
+    _, both = bench._time_steps(with_junk, 20, 5)
+    _, alone = bench._time_steps(lambda: junk.sum(), 20, 5)
+    print("  one graph, a 512 MB read between two launches  %7.1f" % ((both - alone) * 1e3))
+
+
 if __name__ == "__main__":
-    modes = {"wave-age": wave_age, "block-phases": block_phases, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate}
+    modes = {"wave-age": wave_age, "block-phases": block_phases, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
+             "cold-parts": cold_parts}
     if len(sys.argv) != 3 or sys.argv[1] not in modes:
         print(__doc__)
         sys.exit(2)
