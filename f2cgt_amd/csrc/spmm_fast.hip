@@ -311,6 +311,14 @@ unsigned long long* g_acc_trace = nullptr;
 #else
 #define ACC_STAMP(a, slot) do {} while (0)
 #endif
+// A wave is given its scalar registers in units of 16 plus 16 more (measured: a kernel of 84 runs 7 waves per
+// SIMD, one of 104 runs 6, one of 78 runs 8, out of 800 per SIMD).  The stamps cost about ten scalar registers;
+// the stamped build is held to the 80 of the shipped one so that it keeps the same 32 workgroups per CU.
+#ifdef F2CGT_EXPERIMENTS
+#define F2CGT_SGPR_AS_SHIPPED __attribute__((amdgpu_num_sgpr(80)))
+#else
+#define F2CGT_SGPR_AS_SHIPPED
+#endif
 
 template <int TB, int BITS>
 __device__ __forceinline__ void acc_direct_block(const AccArgs& a, const int* s_ptr, int64_t e0, int64_t row0,
@@ -772,6 +780,13 @@ int launch_acc_tb(AccArgs a, size_t lds, int64_t grid, const void* indptr, const
   a.nt_out = stream_output(a.R * (int64_t)a.feat_dim * 4) ? 1 : 0;
 #ifdef F2CGT_EXPERIMENTS
   a.trace = g_acc_trace;
+  if (const char* v = getenv("F2CGT_ACC_RESIDENT")) {   // at most this many workgroups per CU, by padding the LDS request
+    const int n = atoi(v);
+    if (n >= 1 && n <= 32) {
+      const size_t want = (size_t)(160 * 1024 / n / 1280) * 1280;
+      if (want > lds) lds = want;
+    }
+  }
 #endif
   if (plan_only()) {
     plan_record("sq_affine_acc_kernel", grid, TB, (int64_t)lds, a.rows_per_block, a.fin_slots, TB >> a.lane_shift,
@@ -1189,6 +1204,7 @@ struct HybArgs {
   int rows_per_block, edge_batch;
   int chunks, ch2;   // 4-column chunks per row; gather lanes per edge = pow2 >= chunks
   uint32_t magic;
+  uint32_t w_magic;  // ceil(2^32 / w), 0 for w == 1: column / w as one multiply
 #ifdef F2CGT_EXPERIMENTS
   unsigned long long* trace;   // 8 words per workgroup: time stamps of its phases (100 MHz) and where it ran
 #endif
@@ -1199,7 +1215,7 @@ constexpr uint32_t kVqFlag = 0x80000000u;
 // CH: the number of 4-column chunks per row when it is known at compile time (32 for 128 columns,
 // the common width: the accumulator offsets of the gather then fold into the instructions), else 0.
 template <typename Idx, int VEC, int TB, int CH = 0>
-__global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __restrict__ indptr,
+__global__ __launch_bounds__(TB) F2CGT_SGPR_AS_SHIPPED void hybrid_acc_kernel(HybArgs a, const Idx* __restrict__ indptr,
                                                             const Idx* __restrict__ indices,
                                                             float* __restrict__ out) {
   constexpr int LIMIT = 257;
@@ -1218,6 +1234,9 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
   uint16_t* s_erow = reinterpret_cast<uint16_t*>(s_row + a.edge_batch);      // [edge_batch] local row
 
   const int t = threadIdx.x;
+#ifdef F2CGT_EXPERIMENTS
+  if (a.trace == reinterpret_cast<unsigned long long*>(1)) return;   // the launch alone: what dispatching the grid costs
+#endif
   ACC_STAMP(a, 0);
   const int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block;
   const int nrows = (int)((a.R - row0) < a.rows_per_block ? (a.R - row0) : a.rows_per_block);
@@ -1265,7 +1284,11 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
 #pragma unroll
     for (int p = 0; p < PRE; ++p) pre_map[p] = a.row_map[clamp_idx(pre_id[p], a.N)];
   }
-  for (int i = t; i < nrows * acc_pitch; i += TB) s_acc[i] = 0u;
+  {   // all rows of the block's accumulator area, 16 bytes per lane (rows_per_block is a multiple of 8)
+    uint4* z = reinterpret_cast<uint4*>(s_acc);
+    const int n4 = (a.rows_per_block * acc_pitch) >> 2;
+    for (int i = t; i < n4; i += TB) z[i] = make_uint4(0u, 0u, 0u, 0u);
+  }
   for (int i = t; i < nrows; i += TB) {
     s_nvq[i] = 0;
     s_mask[2 * i] = 0u;
@@ -1294,6 +1317,12 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
   const uint32_t* codes32 = reinterpret_cast<const uint32_t*>(a.sq_codes);
   const int dwords_per_row = CH ? CH : a.feat_dim >> 2;   // CH chunks are CH dwords of 8-bit codes
 
+  // Blocks of eight rows find an edge's row by comparing its position with the seven inner row starts
+  // (read once, the same in every lane) instead of a search with one LDS round trip per step.
+  const bool eight = a.rows_per_block == 8;
+  int start_of[8];
+#pragma unroll
+  for (int k = 1; k < 8; ++k) start_of[k] = eight ? s_ptr[k < nrows ? k : nrows] : 0;
   // rows longer than the field capacity are summed directly in the epilogue (flag: all edges "VQ-like")
   for (int eb = 0; eb < ne; eb += a.edge_batch) {
     const int nb = (ne - eb) < a.edge_batch ? (ne - eb) : a.edge_batch;
@@ -1316,10 +1345,16 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
       // the edge's destination row: the last r with s_ptr[r] <= position (empty rows share a
       // start and are skipped that way); the same number of steps in every lane
       const int pos = eb + i;
-      int lo = 0, hi = nrows;
-      while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (s_ptr[mid] <= pos) lo = mid; else hi = mid;
+      int lo = 0;
+      if (eight) {
+#pragma unroll
+        for (int k = 1; k < 8; ++k) lo += start_of[k] <= pos ? 1 : 0;
+      } else {
+        int hi = nrows;
+        while (hi - lo > 1) {
+          const int mid = (lo + hi) >> 1;
+          if (s_ptr[mid] <= pos) lo = mid; else hi = mid;
+        }
       }
       const int first = s_ptr[lo];
       if (s_ptr[lo + 1] - first > LIMIT) v |= 0x40000000u;   // rows beyond the field capacity stay out of the accumulators
@@ -1435,7 +1470,7 @@ __global__ __launch_bounds__(TB) void hybrid_acc_kernel(HybArgs a, const Idx* __
     float v3 = __fadd_rn(__fmul_rn(nsq, mn.w), __fmul_rn((float)(q.y >> 16), sc.w));
     if (nvq > 0) {  // the row's remaining edges, in edge order, straight from the tables
       const int col = c4 * 4;
-      const int sub = col / a.w;
+      const int sub = a.w_magic ? (int)__umulhi((uint32_t)col, a.w_magic) : col;
       const int off = col - sub * a.w;
       const bool in_lds = ne <= a.edge_batch;  // one batch: s_row still describes every edge of the block
       auto add_edge = [&](int64_t m) {
@@ -1663,6 +1698,7 @@ int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float*
   a.vq_codes = vq_codes; a.vq_codebooks = vq_codebooks;
   a.R = R; a.E = E; a.N = N; a.n_sq = n_sq; a.n_vq = n_vq;
   a.feat_dim = feat_dim; a.n_cb = n_cb; a.K = K; a.w = w;
+  a.w_magic = w > 1 ? (uint32_t)((0x100000000ull + (uint64_t)w - 1) / (uint64_t)w) : 0u;
   a.chunks = feat_dim / 4;
   a.ch2 = pow2_ceil(a.chunks);
   a.magic = (uint32_t)((0x100000000ull + a.chunks - 1) / a.chunks);

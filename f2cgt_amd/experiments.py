@@ -4,6 +4,7 @@
     python3 -m f2cgt_amd.experiments wave-age c3|c5      per-wave start / first step / end of vq_wave_kernel
     python3 -m f2cgt_amd.experiments block-phases c1|c2|c4  per-workgroup phase times of sq_affine_acc_kernel / hybrid_acc_kernel
     python3 -m f2cgt_amd.experiments mfma-overlap x      fp32 MFMA and LDS-gather work on one SIMD: side by side or one after the other?
+    python3 -m f2cgt_amd.experiments dispatch-cost c4    the two-table kernel's grid with workgroups that return at once
     python3 -m f2cgt_amd.experiments lds-rate x          bytes per clock and CU that conflict-free LDS reads return
     python3 -m f2cgt_amd.experiments cold-parts c2|c3|c4|c5   launch time by what of the input is still cached (any build)
 
@@ -116,6 +117,46 @@ def block_phases(name):
     key = xcc * 4096 + ((hw >> 13) & 7) * 512 + ((hw >> 12) & 1) * 16 + ((hw >> 8) & 0xf)
     _, count = np.unique(key, return_counts=True)
     print("  distinct CUs: %d, workgroups per CU min / mean / max: %d / %.1f / %d" % (len(count), count.min(), count.mean(), count.max()))
+    # Residency per CU from the stamps themselves: time-weighted mean, the most ever resident, and how long a
+    # CU waits from the end of one workgroup to the start of its next one.
+    dur = T[:, 4] - T[:, 0]
+    print("  workgroups resident per CU, time-weighted mean over the launch: %.1f" % (dur.sum() / T[:, 4].max() / len(count)))
+    peak, refill, steady = [], [], []
+    for k in np.unique(key)[:: max(1, len(count) // 64)]:
+        sel = key == k
+        st, en = np.sort(T[sel, 0]), np.sort(T[sel, 4])
+        ev = np.concatenate([np.stack([st, np.ones_like(st)], 1), np.stack([en, -np.ones_like(en)], 1)])
+        ev = ev[np.lexsort((ev[:, 1], ev[:, 0]))]
+        level = np.cumsum(ev[:, 1])
+        peak.append(level.max())
+        mid = (ev[:-1, 0] > 0.2 * T[:, 4].max()) & (ev[:-1, 0] < 0.8 * T[:, 4].max())
+        steady.append((level[:-1][mid] * np.diff(ev[:, 0])[mid]).sum() / max(np.diff(ev[:, 0])[mid].sum(), 1e-9))
+        nxt = np.searchsorted(st, en, side="left")
+        ok = nxt < len(st)
+        refill.append(st[nxt[ok]] - en[ok])
+    refill = np.concatenate(refill)
+    print("  (every %d-th CU) most resident at once min / median / max: %d / %d / %d; mean resident in the middle 60 %% of the launch: %.1f"
+          % (max(1, len(count) // 64), min(peak), int(np.median(peak)), max(peak), float(np.mean(steady))))
+    print("  from a workgroup's last stamp to the next start on its CU, us:", _q(refill))
+
+
+def dispatch_cost(name):
+    """What the grid of the two-table kernel costs to dispatch: the same launch with workgroups that return at
+    their first instruction (the trace pointer 1 asks for that), next to the full launch."""
+    torch, lib, wl, step, _ = _setup(name)
+    if not hasattr(lib, "f2cgt_experiment_set_acc_trace"):
+        raise SystemExit("the library in tree was built without --experiments")
+    sys.path.insert(0, ROOT)
+    import bench
+
+    lib.f2cgt_experiment_set_acc_trace.argtypes = [ctypes.c_void_p]
+    lib.f2cgt_experiment_set_acc_trace.restype = None
+    _, ms = bench._time_steps(step, 40, 10)
+    print("%s launch %.1f us" % (name, ms * 1e3))
+    lib.f2cgt_experiment_set_acc_trace(ctypes.c_void_p(1))
+    _, ms = bench._time_steps(step, 40, 10)
+    lib.f2cgt_experiment_set_acc_trace(None)
+    print("the same grid, every workgroup returning at once: %.1f us" % (ms * 1e3))
 
 
 def mfma_overlap(_):
@@ -256,7 +297,7 @@ def cold_parts(name):
 
 
 if __name__ == "__main__":
-    modes = {"wave-age": wave_age, "block-phases": block_phases, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
+    modes = {"wave-age": wave_age, "block-phases": block_phases, "dispatch-cost": dispatch_cost, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
              "cold-parts": cold_parts}
     if len(sys.argv) != 3 or sys.argv[1] not in modes:
         print(__doc__)
