@@ -578,6 +578,53 @@ def test_hybrid_high_degree_and_vq_heavy():
     assert np.allclose(got, exact, rtol=1e-5, atol=1e-5 * np.abs(dec).max())
 
 
+@pytest.mark.parametrize("idx", [np.int64, np.int32])
+@pytest.mark.parametrize("vq_share", [0.05, 0.6])
+def test_hybrid_eight_row_blocks(idx, vq_share):
+    """8 to 32 edges per row on average and at most 128 columns: single-wave workgroups of eight rows, which find an
+    edge's row by compares with the block's inner row starts.  Ragged rows, runs of empty rows (equal starts), rows with
+    more than 64 edges (outside the per-row mask) and one beyond the 16-bit field capacity, a last block of three rows."""
+    rng = np.random.default_rng(int(vq_share * 100) + (idx == np.int32))
+    n_cb, K, w = 8, 256, 16
+    D = n_cb * w
+    N, n_hot, R = 20000, 4000, 8 * 150 + 3
+    row_map = np.empty(N, dtype=np.int32)
+    perm = rng.permutation(N)
+    row_map[perm[:n_hot]] = np.arange(n_hot)
+    row_map[perm[n_hot:]] = -np.arange(N - n_hot) - 1
+    sq = rng.integers(0, 256, size=(n_hot, D), dtype=np.uint8)
+    params = np.stack([rng.standard_normal(D), rng.uniform(0.01, 0.05, D)]).astype(np.float32)
+    vq = rng.integers(0, K, size=(N - n_hot, n_cb), dtype=np.uint8)
+    cb = rng.standard_normal((n_cb, K, w)).astype(np.float32)
+    deg = rng.integers(0, 33, size=R)
+    deg[rng.random(R) < 0.2] = 0          # runs of empty rows inside blocks
+    deg[16:24] = 0                        # a block without edges
+    deg[40] = 90                          # more edges than the per-row mask holds
+    deg[41] = 1
+    deg[100] = 300                        # beyond the field capacity: summed in the epilogue
+    deg[R - 1] = 17
+    indptr = np.zeros(R + 1, dtype=idx)
+    indptr[1:] = np.cumsum(deg)
+    E = int(indptr[-1])
+    assert 8.0 <= E / R <= 32.0
+    indices = rng.integers(0, N, size=E)
+    hot = rng.random(E) >= vq_share
+    indices[hot] = rng.choice(perm[:n_hot], size=int(hot.sum()))
+    indices = indices.astype(idx)
+    rc, plan = capi.dry_run("f2cgt_hybrid_decompress_spmm_csr", 0x1000, 0x1000, 0x1000, D, 0x1000, 0x1000, 0x1000, 0x1000,
+                            capi.DT_I64 if idx == np.int64 else capi.DT_I32, 0x1000, R, E, N, n_hot, N - n_hot, D, n_cb, K, w,
+                            None)
+    assert rc == 0 and plan.block == 64 and plan.rows_per_block == 8
+    got = host(capi.hybrid_decompress_spmm_csr(dev(row_map), dev(sq), dev(params), dev(vq), dev(cb), dev(indptr),
+                                               dev(indices), D))
+    dec = oc.hybrid_decompress(row_map, sq, params, vq, cb, D, np.arange(N)).astype(np.float64)
+    exact = oc.spmm_csr(dec, indptr.astype(np.int64), indices.astype(np.int64))
+    assert np.allclose(got, exact, rtol=1e-5, atol=1e-5 * np.abs(dec).max())
+    assert not got[deg == 0].any()
+    one = np.nonzero(deg == 1)[0]
+    assert np.array_equal(got[one], dec[indices[indptr[one]]].astype(np.float32))
+
+
 # ---- encode -------------------------------------------------------------------------------------
 @pytest.mark.parametrize("metric", ["l2", "cosine"])
 @pytest.mark.parametrize("m,n,k", [(1000, 256, 32), (333, 17, 5), (64, 64, 64), (129, 300, 100)])
