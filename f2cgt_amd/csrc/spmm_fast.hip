@@ -1207,6 +1207,8 @@ struct HybArgs {
   uint32_t w_magic;  // ceil(2^32 / w), 0 for w == 1: column / w as one multiply
 #ifdef F2CGT_EXPERIMENTS
   unsigned long long* trace;   // 8 words per workgroup: time stamps of its phases (100 MHz) and where it ran
+  int hot_rows;                // F2CGT_HYB_HOT: the first so many rows of the SQ table are copied to LDS by every workgroup
+  int hot_off;                 // where in the workgroup's LDS
 #endif
 };
 
@@ -1284,6 +1286,27 @@ __global__ __launch_bounds__(TB) F2CGT_SGPR_AS_SHIPPED void hybrid_acc_kernel(Hy
 #pragma unroll
     for (int p = 0; p < PRE; ++p) pre_map[p] = a.row_map[clamp_idx(pre_id[p], a.N)];
   }
+#ifdef F2CGT_EXPERIMENTS
+  // Measured variant: the hottest source rows (the first hot_rows rows of the SQ table, where the synthetic
+  // workloads keep them) are copied into the workgroup's LDS, and edges that name them are gathered from there.
+  if (VEC == 4 && a.hot_rows > 0) {
+    typedef uint32_t u32x4h __attribute__((ext_vector_type(4)));
+    const int pieces = a.hot_rows * (CH ? CH : a.feat_dim >> 2) / 4;   // 16-byte pieces, at most 8 per lane
+    const u32x4h* src = reinterpret_cast<const u32x4h*>(a.sq_codes);
+    u32x4h hv[8];
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      const int i = t + p * TB;
+      hv[p] = src[i < pieces ? i : pieces - 1];
+    }
+    u32x4h* dst = reinterpret_cast<u32x4h*>(smem + a.hot_off);
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      const int i = t + p * TB;
+      if (i < pieces) dst[i] = hv[p];
+    }
+  }
+#endif
   {   // all rows of the block's accumulator area, 16 bytes per lane (rows_per_block is a multiple of 8)
     uint4* z = reinterpret_cast<uint4*>(s_acc);
     const int n4 = (a.rows_per_block * acc_pitch) >> 2;
@@ -1397,12 +1420,25 @@ __global__ __launch_bounds__(TB) F2CGT_SGPR_AS_SHIPPED void hybrid_acc_kernel(Hy
           ee = ee < e_end ? ee : e_end - 1;
           row[u] = s_row[ee];
           er[u] = s_erow[ee];
-          const uint32_t r = (row[u] >> 30) == 0 ? row[u] : 0u;
+          uint32_t r = (row[u] >> 30) == 0 ? row[u] : 0u;
+#ifdef F2CGT_EXPERIMENTS
+          if (a.hot_rows > 0 && r < (uint32_t)a.hot_rows) r = 0u;   // comes from LDS below; the load reads row 0
+#endif
           w[u] = *reinterpret_cast<const u32x4*>(lane_codes + (uint64_t)r * (uint32_t)dwords_per_row);
         }
         // the four loads are issued together and waited for together, whatever the adds below use
 #pragma unroll
         for (int u = 0; u < U; ++u) asm volatile("" : "+v"(w[u]));
+#ifdef F2CGT_EXPERIMENTS
+        if (a.hot_rows > 0) {
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            if ((row[u] >> 30) == 0 && row[u] < (uint32_t)a.hot_rows)
+              w[u] = *reinterpret_cast<const u32x4*>(smem + a.hot_off + (size_t)row[u] * (dwords_per_row * 4) +
+                                                     (lane_on ? 16 * j : 0));
+          }
+        }
+#endif
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const int ee = e + u;
@@ -1651,11 +1687,22 @@ int launch_hybrid(HybArgs a, const void* indptr, const void* indices, int idx_dt
   }
 #endif
   a.rows_per_block = rb;
+  size_t lds = rb * acc_row + (size_t)a.chunks * 32 + (size_t)(rb + 4) * 4 + (size_t)rb * 4 + (size_t)rb * 8 +
+               (size_t)a.edge_batch * 6 + 16;
 #ifdef F2CGT_EXPERIMENTS
   a.trace = g_acc_trace;
+  a.hot_rows = 0;
+  a.hot_off = 0;
+  if (const char* v = getenv("F2CGT_HYB_HOT")) {   // hot rows in LDS: 16-byte gather, at most 8 pieces of 16 bytes per lane
+    const int want = atoi(v);
+    const bool vec4 = a.feat_dim % 16 == 0 && aligned(a.sq_codes, 16) && a.ch2 >= 4;
+    if (want > 0 && vec4 && (int64_t)want <= a.n_sq && (int64_t)want * a.feat_dim <= (int64_t)8 * TB * 16) {
+      a.hot_rows = want;
+      a.hot_off = (int)((lds + 15) & ~(size_t)15);
+      lds = (size_t)a.hot_off + (size_t)want * a.feat_dim;
+    }
+  }
 #endif
-  const size_t lds = rb * acc_row + (size_t)a.chunks * 32 + (size_t)(rb + 4) * 4 + (size_t)rb * 4 + (size_t)rb * 8 +
-                     (size_t)a.edge_batch * 6 + 16;
   const int64_t grid = ceil_div(a.R, rb);
   if (grid > 0x7fffffffll) return fail(F2CGT_E_UNSUPPORTED, "%s: too many row blocks", what);
   const bool vec4 = a.feat_dim % 16 == 0 && aligned(a.sq_codes, 16) && a.ch2 >= 4;

@@ -5,6 +5,7 @@
     python3 -m f2cgt_amd.experiments block-phases c1|c2|c4  per-workgroup phase times of sq_affine_acc_kernel / hybrid_acc_kernel
     python3 -m f2cgt_amd.experiments mfma-overlap x      fp32 MFMA and LDS-gather work on one SIMD: side by side or one after the other?
     python3 -m f2cgt_amd.experiments dispatch-cost c4    the two-table kernel's grid with workgroups that return at once
+    python3 -m f2cgt_amd.experiments hot-rows c4         the two-table kernel with the hottest source rows copied to LDS
     python3 -m f2cgt_amd.experiments lds-rate x          bytes per clock and CU that conflict-free LDS reads return
     python3 -m f2cgt_amd.experiments cold-parts c2|c3|c4|c5   launch time by what of the input is still cached (any build)
 
@@ -159,6 +160,40 @@ def dispatch_cost(name):
     print("the same grid, every workgroup returning at once: %.1f us" % (ms * 1e3))
 
 
+def hot_rows(name):
+    """The two-table kernel with the first 32 / 64 rows of the SQ table (the hottest ones of the synthetic
+    workloads) copied into every workgroup's LDS and gathered from there (F2CGT_HYB_HOT), against the shipped
+    gather through L1: launch times, and that the results are the same."""
+    torch, lib, wl, step, out = _setup(name)
+    if not hasattr(lib, "f2cgt_experiment_set_acc_trace"):
+        raise SystemExit("the library in tree was built without --experiments")
+    sys.path.insert(0, ROOT)
+    import bench
+
+    ids = wl["indices"]
+    m = wl["row_map"][ids.long()]
+    for h in (32, 64):
+        print("%s: %.3f of the edges name one of the first %d rows of the SQ table"
+              % (name, float(((m >= 0) & (m < h)).float().mean()), h))
+    os.environ.pop("F2CGT_HYB_HOT", None)
+    step()
+    torch.cuda.synchronize()
+    ref = out.clone()
+    for rnd in range(2):
+        for h in (0, 32, 64):
+            if h:
+                os.environ["F2CGT_HYB_HOT"] = str(h)
+            else:
+                os.environ.pop("F2CGT_HYB_HOT", None)
+            out.zero_()
+            step()
+            torch.cuda.synchronize()
+            same = bool(torch.equal(out, ref))
+            _, ms = bench._time_steps(step, 40, 10)
+            print("  hot rows in LDS: %2d   launch %.1f us   result identical: %s" % (h, ms * 1e3, same), flush=True)
+    os.environ.pop("F2CGT_HYB_HOT", None)
+
+
 def mfma_overlap(_):
     """Times the four arrangements of csrc/overlap_probe.hip on every CU and prints what each costs."""
     import torch
@@ -297,7 +332,7 @@ def cold_parts(name):
 
 
 if __name__ == "__main__":
-    modes = {"wave-age": wave_age, "block-phases": block_phases, "dispatch-cost": dispatch_cost, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
+    modes = {"wave-age": wave_age, "block-phases": block_phases, "dispatch-cost": dispatch_cost, "hot-rows": hot_rows, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
              "cold-parts": cold_parts}
     if len(sys.argv) != 3 or sys.argv[1] not in modes:
         print(__doc__)
