@@ -1749,11 +1749,14 @@ int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float*
   a.chunks = feat_dim / 4;
   a.ch2 = pow2_ceil(a.chunks);
   a.magic = (uint32_t)((0x100000000ull + a.chunks - 1) / a.chunks);
-  // One wave per workgroup (8 rows at 12 edges per row) for rows of up to 128 columns and 8-32 edges:
+  // One wave per workgroup (8 rows at 12 edges per row) for rows of up to 128 columns and up to 32 edges:
   // the phases of a block are dependent memory round trips, and many small blocks per CU overlap
   // them better than few large ones, without a barrier between waves (C4: 334 -> 313 us; 128
-  // threads and 16 rows: 318; twice the rows per block at either size: 332-344).  Measured slower
-  // or equal outside that range (2, 5 or 60 edges per row, 256 columns), which keeps the 256-thread form.
+  // threads and 16 rows: 318; twice the rows per block at either size: 332-344).  Against the
+  // 256-thread form on 2e7-node tables, 64 / 128 columns: 2 edges per row 145 / 228 against 148 / 243 us,
+  // 5: 192 / 298 against 196 / 309, 20: 289 / 179 against 439 / 220, 32: 247 / 163 against 697 / 325;
+  // above 32 edges per row eight rows no longer fit one batch of 256 edges (48: 752 / 585 against
+  // 663 / 311), and at 256 columns the 256-thread form is level or ahead from 5 edges per row on.
   const double avg_deg = R > 0 ? (double)E / (double)R : 0.0;
 #ifdef F2CGT_EXPERIMENTS
   if (const char* v = getenv("F2CGT_HYB_TB")) {   // workgroup size for an A/B: 64, 128 or 256
@@ -1762,7 +1765,7 @@ int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float*
     if (atoi(v) == 256) return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what);
   }
 #endif
-  if (a.ch2 <= 32 && avg_deg >= 8.0 && avg_deg <= 32.0)
+  if (a.ch2 <= 32 && avg_deg <= 32.0)
     return launch_hybrid<64>(a, indptr, indices, idx_dtype, out, st, what);
   return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what);
 }

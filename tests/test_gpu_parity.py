@@ -581,7 +581,7 @@ def test_hybrid_high_degree_and_vq_heavy():
 @pytest.mark.parametrize("idx", [np.int64, np.int32])
 @pytest.mark.parametrize("vq_share", [0.05, 0.6])
 def test_hybrid_eight_row_blocks(idx, vq_share):
-    """8 to 32 edges per row on average and at most 128 columns: single-wave workgroups of eight rows, which find an
+    """Up to 32 edges per row on average and at most 128 columns: single-wave workgroups, of eight rows here, which find an
     edge's row by compares with the block's inner row starts.  Ragged rows, runs of empty rows (equal starts), rows with
     more than 64 edges (outside the per-row mask) and one beyond the 16-bit field capacity, a last block of three rows."""
     rng = np.random.default_rng(int(vq_share * 100) + (idx == np.int32))
