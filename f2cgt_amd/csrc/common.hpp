@@ -90,7 +90,13 @@ __device__ __forceinline__ void row_range(const Idx* __restrict__ indptr, int64_
 // form takes 32.7 us per launch and the non-temporal one 27.7 us, which is also what it takes on
 // one buffer: the streamed form does not depend on the cache state.  The size rule is therefore
 // only the default (F2CGT_STORE_AUTO); f2cgt_set_store_mode overrides it either way.
-bool stream_output(int64_t out_bytes);
+// The crossover comes earlier when a launch reads more per output row or writes whole 128-byte lines:
+// at 10 edges per row plain against streamed stores take 62.9 / 56.1 us at 160 MB and 95.3 / 69.2 us at
+// 200 MB (8-bit codes, 128 columns; 76.1 / 66.2 and 110.5 / 81.0 us at 4 bit and 100 columns), at 3 edges
+// per row 37.6 / 38.4 and 48.7 / 44.2 us (128 columns) but 36.4 / 40.9 and 49.9 / 50.9 us at 100 columns,
+// whose 400-byte rows leave partial lines to merge.  Hence 140 MB for rows of whole lines or at least six
+// edges per row, and 220 MB otherwise.
+bool stream_output(int64_t out_bytes, int64_t row_bytes, double edges_per_row);
 
 // Non-temporal stores: the aggregation output is written once and never re-read by
 // the kernel, so it should not displace gathered code rows from L2 / MALL.

@@ -29,11 +29,12 @@ void plan_record(const char* kernel, int64_t grid, int block, int64_t lds_bytes,
 
 std::atomic<int> g_store_mode{F2CGT_STORE_AUTO};
 
-bool stream_output(int64_t out_bytes) {
+bool stream_output(int64_t out_bytes, int64_t row_bytes, double edges_per_row) {
   const int mode = g_store_mode.load(std::memory_order_relaxed);
   if (mode == F2CGT_STORE_STREAM) return true;
   if (mode == F2CGT_STORE_CACHED) return false;
-  return out_bytes > 220000000ll;
+  const bool early = row_bytes % 128 == 0 || edges_per_row >= 6.0;
+  return out_bytes > (early ? 140000000ll : 220000000ll);
 }
 
 int num_cus() {

@@ -58,8 +58,9 @@ int f2cgt_num_cus(void);
 
 /* How the row-block aggregation kernels (the SQ and affine-SQ fused operators) write their output
  * (no counterpart in the reference, whose kernels use plain stores, src/fusion_spmm.cu:173-236).
- *   F2CGT_STORE_AUTO    (default) outputs above 220 MB are streamed past the caches with non-temporal
- *                       stores, smaller ones are written with plain stores
+ *   F2CGT_STORE_AUTO    (default) outputs above 220 MB (above 140 MB when the output rows are whole
+ *                       128-byte lines or the graph has six or more edges per row) are streamed past
+ *                       the caches with non-temporal stores, smaller ones are written with plain stores
  *   F2CGT_STORE_STREAM  always streamed: the launch time no longer depends on what the caches hold
  *   F2CGT_STORE_CACHED  never streamed
  * Plain stores are fastest when the same output buffer is written again before the last-level cache
