@@ -6,6 +6,8 @@
     python3 -m f2cgt_amd.experiments mfma-overlap x      fp32 MFMA and LDS-gather work on one SIMD: side by side or one after the other?
     python3 -m f2cgt_amd.experiments dispatch-cost c4    the two-table kernel's grid with workgroups that return at once
     python3 -m f2cgt_amd.experiments hot-rows c4         the two-table kernel with the hottest source rows copied to LDS
+    python3 -m f2cgt_amd.experiments affine-geometry x   the affine kernel at 10-20 edges per row: block rows and workgroup size
+    python3 -m f2cgt_amd.experiments store-form x        plain against non-temporal output stores by shape (any build)
     python3 -m f2cgt_amd.experiments lds-rate x          bytes per clock and CU that conflict-free LDS reads return
     python3 -m f2cgt_amd.experiments cold-parts c2|c3|c4|c5   launch time by what of the input is still cached (any build)
 
@@ -194,6 +196,87 @@ def hot_rows(name):
     os.environ.pop("F2CGT_HYB_HOT", None)
 
 
+def _affine_case(torch, synth, gen, n_src, bits, dim, rows, fanout):
+    """Codes, parameters and a fixed-fanout CSC block with Zipf(1.1) source ids for the affine kernel."""
+    codes = torch.randint(0, 256, (n_src, dim * bits // 8), generator=gen, device="cuda", dtype=torch.uint8)
+    params = torch.stack([torch.randn(dim, device="cuda"), torch.rand(dim, device="cuda") * 0.05 + 0.01]).contiguous()
+    deg = torch.full((rows,), fanout, dtype=torch.int64, device="cuda")
+    indptr = synth.csc_from_degrees(deg, torch.int64)
+    ids = synth.zipf_ids(n_src, (rows * fanout,), 1.1, gen, "cuda", torch.int64)
+    return codes, params, indptr, ids
+
+
+def affine_geometry(_):
+    """The affine row-block kernel at 3e6 edges, 10-20 edges per row: the shipped geometry against 64-thread
+    workgroups and against eight rows per block (F2CGT_ACC_TB / F2CGT_ACC_RB, experiments build)."""
+    import torch
+
+    sys.path.insert(0, ROOT)
+    import bench
+    from f2cgt_amd import capi, synth
+
+    if not hasattr(capi.lib(), "f2cgt_experiment_set_acc_trace"):
+        raise SystemExit("the library in tree was built without --experiments")
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    cases = (("shipped", {}), ("8 rows", {"F2CGT_ACC_RB": "8"}), ("64 threads, 8 rows", {"F2CGT_ACC_TB": "64", "F2CGT_ACC_RB": "8"}),
+             ("256 threads, 16 rows", {"F2CGT_ACC_TB": "256", "F2CGT_ACC_RB": "16"}))
+    print("us per launch, 2.4e6 source rows, 3e6 edges: " + " | ".join(name for name, _ in cases))
+    for bits in (4, 8):
+        for dim in (100, 128):
+            for fanout in (10, 11, 12, 14, 16, 17, 18, 20):
+                rows = 3_000_000 // fanout
+                codes, params, indptr, ids = _affine_case(torch, synth, gen, 2_400_000, bits, dim, rows, fanout)
+                out = torch.empty((rows, dim), dtype=torch.float32, device="cuda")
+                step = lambda: capi.sq_affine_decompress_spmm_csr(codes, params, indptr, ids, bits, dim, out=out)
+                best = {}
+                for _ in range(2):
+                    for name, env in cases:
+                        for k in ("F2CGT_ACC_TB", "F2CGT_ACC_RB"):
+                            os.environ.pop(k, None)
+                        os.environ.update(env)
+                        _, ms = bench._time_steps(step, 30, 10)
+                        best[name] = min(best.get(name, 1e9), ms * 1e3)
+                for k in ("F2CGT_ACC_TB", "F2CGT_ACC_RB"):
+                    os.environ.pop(k, None)
+                print("  %d bit, %3d columns, %2d edges per row: " % (bits, dim, fanout)
+                      + " | ".join("%6.1f" % best[name] for name, _ in cases), flush=True)
+
+
+def store_form(_):
+    """Plain against non-temporal output stores of the two SQ row-block kernels by output size, row width and
+    edges per row, and what the default picks (f2cgt_set_store_mode; any build)."""
+    import torch
+
+    sys.path.insert(0, ROOT)
+    import bench
+    from f2cgt_amd import capi, synth
+
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    logcb = torch.tensor([[0.01, 3.0, -6.643856, 1.5849625, 0.4]], device="cuda")
+    print("us per launch: default | plain | non-temporal")
+    for bits, dim in ((8, 128), (4, 100)):
+        for fanout in (3, 10):
+            for out_mb in (64, 100, 128, 160, 200, 240):
+                rows = int(out_mb * 1e6 / (dim * 4))
+                codes, params, indptr, ids = _affine_case(torch, synth, gen, 2_400_000, bits, dim, rows, fanout)
+                out = torch.empty((rows, dim), dtype=torch.float32, device="cuda")
+                signed = codes.view(torch.int8) if bits == 8 else codes
+                forms = (("affine", lambda: capi.sq_affine_decompress_spmm_csr(codes, params, indptr, ids, bits, dim, out=out)),
+                         ("log", lambda: capi.sq_decompress_spmm_csr(signed, logcb, indptr, ids, bits, dim, dim, out=out)))
+                for form, step in forms:
+                    best = {}
+                    for _ in range(2):
+                        for name, mode in (("default", capi.STORE_AUTO), ("plain", capi.STORE_CACHED), ("nt", capi.STORE_STREAM)):
+                            capi.set_store_mode(mode)
+                            _, ms = bench._time_steps(step, 30, 10)
+                            best[name] = min(best.get(name, 1e9), ms * 1e3)
+                    capi.set_store_mode(capi.STORE_AUTO)
+                    print("  %-6s %d bit, %3d columns, %2d edges per row, %3d MB of output: %6.1f | %6.1f | %6.1f"
+                          % (form, bits, dim, fanout, out_mb, best["default"], best["plain"], best["nt"]), flush=True)
+
+
 def mfma_overlap(_):
     """Times the four arrangements of csrc/overlap_probe.hip on every CU and prints what each costs."""
     import torch
@@ -332,7 +415,8 @@ def cold_parts(name):
 
 
 if __name__ == "__main__":
-    modes = {"wave-age": wave_age, "block-phases": block_phases, "dispatch-cost": dispatch_cost, "hot-rows": hot_rows, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
+    modes = {"wave-age": wave_age, "block-phases": block_phases, "dispatch-cost": dispatch_cost, "hot-rows": hot_rows,
+             "affine-geometry": affine_geometry, "store-form": store_form, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
              "cold-parts": cold_parts}
     if len(sys.argv) != 3 or sys.argv[1] not in modes:
         print(__doc__)
