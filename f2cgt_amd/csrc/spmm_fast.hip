@@ -286,6 +286,8 @@ struct AccArgs {
   int rows_tail;
 #endif
   int sub_rows;        // rows that go through the accumulators at a time
+  int wide_rows;       // ... in the layout with 4 words per code dword: sub_rows, or half of it when the LDS was sized for the narrow one
+  int acc_words;       // words of the accumulator area at the start of the workgroup's LDS
   int edge_batch;
   int eff_bytes;     // leading bytes of a code row that hold output columns
   int lanes;         // 8-byte gather lanes per edge
@@ -370,7 +372,11 @@ __device__ __forceinline__ void acc_tag(const AccArgs& a, const int* ptr, int nr
 
 // Adds the code fields of the tagged edges s_edge[i0 .. i1) to the accumulators; an edge of local
 // row y goes to accumulator row y - row_base.
-template <int TB, int BITS, int NW>
+// CHUNK: a lane group takes a contiguous share of the edges instead of every gslots-th one, so that the
+// groups of one instruction work on edges (and, from a handful of edges per row on, on rows) far apart:
+// neighbouring edges of one long row add to the same accumulator words, and LDS atomics to one address
+// are served one after the other.
+template <int TB, int BITS, int NW, bool CHUNK = false>
 __device__ __forceinline__ void acc_gather(const AccArgs& a, uint32_t* s_acc, const uint2* s_edge, int i0, int i1,
                                            int row_base, int pitch) {
   constexpr uint32_t M = NW == 4 ? 0x000f000fu : (BITS == 4 ? 0x0f0f0f0fu : 0x00ff00ffu);
@@ -390,13 +396,17 @@ __device__ __forceinline__ void acc_gather(const AccArgs& a, uint32_t* s_acc, co
   constexpr int U = 4;
   if (!lane_on) return;
   uint32_t keep = 0;
-  for (int e = i0 + gslot; e < i1; e += gslots * U) {
+  const int per = CHUNK ? (i1 - i0 + gslots - 1) / gslots : 0;
+  const int first_e = CHUNK ? i0 + gslot * per : i0 + gslot;
+  const int last_e = CHUNK ? ((first_e + per) < i1 ? (first_e + per) : i1) : i1;   // one past this group's last edge
+  const int su = CHUNK ? 1 : gslots;                                               // from one load of a trip to the next
+  for (int e = first_e; e < last_e; e += su * U) {
     uint2 ed[U];
     uint64_t w[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      int ee = e + u * gslots;
-      ee = ee < i1 ? ee : i1 - 1;
+      int ee = e + u * su;
+      ee = ee < last_e ? ee : last_e - 1;
       ed[u] = s_edge[ee];
       __builtin_memcpy(&w[u], a.codes + ((uint64_t)ed[u].x * (uint32_t)a.src_dim + (uint32_t)off), 8);
     }
@@ -405,7 +415,7 @@ __device__ __forceinline__ void acc_gather(const AccArgs& a, uint32_t* s_acc, co
       // The unconditional use keeps every load up here, issued back to back; a load whose only
       // use sits in the branch below is moved into it by the compiler and waited for on its own.
       keep ^= (uint32_t)w[u];
-      if (u == 0 || e + u * gslots < i1) {
+      if (u == 0 || e + u * su < last_e) {
         const uint64_t v = w[u] >> sh;
         const uint32_t d0 = (uint32_t)v, d1 = (uint32_t)(v >> 32);
         uint32_t* acc = accj + (int)ed[u].y * pitch;
@@ -505,12 +515,12 @@ __device__ __forceinline__ void acc_finalize(const AccArgs& a, const FinParams& 
 }
 
 // All rows of the block, `sub` rows at a time through the accumulators.
-template <int TB, int BITS, int NW, typename Idx>
+template <int TB, int BITS, int NW, typename Idx, bool CHUNK = false>
 __device__ __forceinline__ void acc_block(const AccArgs& a, const FinParams& first, uint32_t* s_acc, const int* s_ptr,
                                           const float* s_rdeg, uint2* s_edge, int64_t e0, int64_t row0, int nrows,
                                           const Idx* __restrict__ indices, float* __restrict__ out) {
   const int pitch = NW == 4 ? a.pitch_w : a.pitch_n;
-  const int sub = NW == 4 ? a.sub_rows >> 1 : a.sub_rows;
+  const int sub = NW == 4 ? a.wide_rows : a.sub_rows;
   const int ne = s_ptr[nrows];
   if (ne <= a.edge_batch) {
     // common case: every edge of the block is tagged once, up front
@@ -520,7 +530,7 @@ __device__ __forceinline__ void acc_block(const AccArgs& a, const FinParams& fir
     ACC_STAMP(a, 2);
     for (int sb = 0; sb < nrows; sb += sub) {
       const int nr = (nrows - sb) < sub ? (nrows - sb) : sub;
-      acc_gather<TB, BITS, NW>(a, s_acc, s_edge, s_ptr[sb], s_ptr[sb + nr], sb, pitch);
+      acc_gather<TB, BITS, NW, CHUNK>(a, s_acc, s_edge, s_ptr[sb], s_ptr[sb + nr], sb, pitch);
       __syncthreads();
       if (sb == 0) ACC_STAMP(a, 3);
       acc_finalize<TB, BITS, NW>(a, first, s_acc, s_rdeg, row0, sb, nr, pitch, out);
@@ -541,7 +551,7 @@ __device__ __forceinline__ void acc_block(const AccArgs& a, const FinParams& fir
         if (eb != ptr[0]) __syncthreads();
         acc_tag<TB>(a, ptr, nr, eb, nb, e0, indices, s_edge);
         __syncthreads();
-        acc_gather<TB, BITS, NW>(a, s_acc, s_edge, 0, nb, 0, pitch);
+        acc_gather<TB, BITS, NW, CHUNK>(a, s_acc, s_edge, 0, nb, 0, pitch);
       }
       __syncthreads();
       acc_finalize<TB, BITS, NW>(a, first, s_acc, s_rdeg, row0, sb, nr, pitch, out);
@@ -549,15 +559,15 @@ __device__ __forceinline__ void acc_block(const AccArgs& a, const FinParams& fir
   }
 }
 
-template <int TB, int BITS, typename Idx>
+template <int TB, int BITS, typename Idx, bool CHUNK = false>
 __global__ __launch_bounds__(TB) void sq_affine_acc_kernel(AccArgs a, const Idx* __restrict__ indptr,
                                                                const Idx* __restrict__ indices,
                                                                float* __restrict__ out) {
   constexpr int CAP_N = BITS == 4 ? 17 : 257;     // edges per row: 2 accumulator words per code dword
   constexpr int CAP_W = BITS == 4 ? 4369 : 257;   // 4 words per code dword (4-bit codes only)
   extern __shared__ __align__(16) unsigned char smem[];
-  uint32_t* s_acc = reinterpret_cast<uint32_t*>(smem);                         // [sub_rows][pitch_n]
-  int* s_ptr = reinterpret_cast<int*>(s_acc + (size_t)a.sub_rows * a.pitch_n);  // [RB + 1]
+  uint32_t* s_acc = reinterpret_cast<uint32_t*>(smem);                         // [sub_rows][pitch_n] or [wide_rows][pitch_w]
+  int* s_ptr = reinterpret_cast<int*>(s_acc + a.acc_words);                    // [RB + 1]
   float* s_rdeg = reinterpret_cast<float*>(s_ptr + a.rows_per_block + 4);      // [RB]
   uint32_t* s_wflag = reinterpret_cast<uint32_t*>(s_rdeg + a.rows_per_block);  // [waves]
   uint2* s_edge = reinterpret_cast<uint2*>(s_wflag + 4);          // [edge_batch]
@@ -608,9 +618,9 @@ __global__ __launch_bounds__(TB) void sq_affine_acc_kernel(AccArgs a, const Idx*
     return;
   }
   if (BITS == 4 && (block_level & 1u))
-    acc_block<TB, BITS, 4, Idx>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
+    acc_block<TB, BITS, 4, Idx, CHUNK>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
   else
-    acc_block<TB, BITS, 2, Idx>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
+    acc_block<TB, BITS, 2, Idx, CHUNK>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
   ACC_STAMP(a, 4);
 #ifdef F2CGT_EXPERIMENTS
   if (a.trace && threadIdx.x == 0) {
@@ -645,8 +655,8 @@ __global__ __launch_bounds__(TB) void sq_affine_acc_pkernel(AccArgs a, const Idx
   constexpr int CAP_W = BITS == 4 ? 4369 : 257;
   constexpr int NID = 2;   // prefetched source ids per thread: edge_batch = NID * TB
   extern __shared__ __align__(16) unsigned char smem[];
-  uint32_t* s_acc = reinterpret_cast<uint32_t*>(smem);                         // [sub_rows][pitch_n]
-  int* s_ptr = reinterpret_cast<int*>(s_acc + (size_t)a.sub_rows * a.pitch_n);  // [RB + 1]
+  uint32_t* s_acc = reinterpret_cast<uint32_t*>(smem);                         // [sub_rows][pitch_n] or [wide_rows][pitch_w]
+  int* s_ptr = reinterpret_cast<int*>(s_acc + a.acc_words);                    // [RB + 1]
   float* s_rdeg = reinterpret_cast<float*>(s_ptr + a.rows_per_block + 4);      // [RB]
   uint32_t* s_wflag = reinterpret_cast<uint32_t*>(s_rdeg + a.rows_per_block);  // [waves]
   uint2* s_edge = reinterpret_cast<uint2*>(s_wflag + 4);                       // [edge_batch]
@@ -810,12 +820,26 @@ int launch_acc_tb(AccArgs a, size_t lds, int64_t grid, const void* indptr, const
     return launch_status(what);
   }
 #endif
-  if (idx_dtype == F2CGT_DT_I32)
-    sq_affine_acc_kernel<TB, BITS, int32_t><<<(unsigned)grid, TB, lds, st>>>(
-        a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
-  else
-    sq_affine_acc_kernel<TB, BITS, int64_t><<<(unsigned)grid, TB, lds, st>>>(
-        a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
+  // contiguous shares of the edges per lane group from six edges per row on (see acc_gather)
+  bool chunk = a.R > 0 && (double)a.E >= 6.0 * (double)a.R;
+#ifdef F2CGT_EXPERIMENTS
+  if (const char* v = getenv("F2CGT_ACC_CHUNK")) chunk = atoi(v) != 0;
+#endif
+  if (idx_dtype == F2CGT_DT_I32) {
+    if (chunk)
+      sq_affine_acc_kernel<TB, BITS, int32_t, true><<<(unsigned)grid, TB, lds, st>>>(
+          a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
+    else
+      sq_affine_acc_kernel<TB, BITS, int32_t><<<(unsigned)grid, TB, lds, st>>>(
+          a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
+  } else {
+    if (chunk)
+      sq_affine_acc_kernel<TB, BITS, int64_t, true><<<(unsigned)grid, TB, lds, st>>>(
+          a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
+    else
+      sq_affine_acc_kernel<TB, BITS, int64_t><<<(unsigned)grid, TB, lds, st>>>(
+          a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
+  }
   return launch_status(what);
 }
 
@@ -854,6 +878,8 @@ int launch_acc_sized(AccArgs a, double dg, size_t acc_row, const void* indptr, c
 #endif
   a.rows_per_block = rb;
   a.sub_rows = sub;
+  a.wide_rows = acc_row >= (size_t)a.pitch_w * 4 ? sub : sub >> 1;
+  a.acc_words = (int)(sub * acc_row / 4);
   const size_t lds = sub * acc_row + (size_t)(rb + 4) * 4 + (size_t)rb * 4 + 16 + (size_t)a.edge_batch * 8 + 16;
   int64_t grid = ceil_div(a.R, rb);
 #ifdef F2CGT_EXPERIMENTS
@@ -896,8 +922,16 @@ int launch_acc(AccArgs a, const void* indptr, const void* indices, int idx_dtype
   a.f4_per_row = a.feat_dim / 4;
   const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 1.0;
   const double dg = avg_deg > 0.5 ? avg_deg : 0.5;
-  // the wide layout runs on half the rows at a time, so it must fit twice into the narrow one
-  const size_t acc_row = (size_t)(a.pitch_n * 2 > a.pitch_w ? a.pitch_n : (a.pitch_w + 1) / 2) * 4;
+  // Sized for the narrow layout, the accumulators take the wide one (4-bit codes, a row of more than 17
+  // edges in the block) on half the rows at a time, so it must fit twice into the narrow one.  From nine
+  // edges per row on average such blocks are the rule: the accumulators are then sized for the wide layout
+  // and a block stays one pass (18 / 20 / 25 edges per row, 128 columns: 87 / 91 / 88 us in two passes).
+  bool expect_wide = BITS == 4 && dg >= 9.0;
+#ifdef F2CGT_EXPERIMENTS
+  if (const char* v = getenv("F2CGT_ACC_WIDE_FULL")) expect_wide = BITS == 4 && atoi(v) != 0;
+#endif
+  const size_t acc_row = expect_wide ? (size_t)(a.pitch_w > a.pitch_n ? a.pitch_w : a.pitch_n) * 4
+                                     : (size_t)(a.pitch_n * 2 > a.pitch_w ? a.pitch_n : (a.pitch_w + 1) / 2) * 4;
   // 128-thread workgroups: more, smaller blocks in flight per CU overlap the dependent
   // indptr -> indices -> code-row loads of one block with the output stores of others
 #ifdef F2CGT_EXPERIMENTS

@@ -6,7 +6,7 @@
     python3 -m f2cgt_amd.experiments mfma-overlap x      fp32 MFMA and LDS-gather work on one SIMD: side by side or one after the other?
     python3 -m f2cgt_amd.experiments dispatch-cost c4    the two-table kernel's grid with workgroups that return at once
     python3 -m f2cgt_amd.experiments hot-rows c4         the two-table kernel with the hottest source rows copied to LDS
-    python3 -m f2cgt_amd.experiments affine-geometry x   the affine kernel at 10-20 edges per row: block rows and workgroup size
+    python3 -m f2cgt_amd.experiments affine-geometry x   the affine kernel by edges per row: edge mapping, accumulator sizing, block rows, workgroup size
     python3 -m f2cgt_amd.experiments store-form x        plain against non-temporal output stores by shape (any build)
     python3 -m f2cgt_amd.experiments lds-rate x          bytes per clock and CU that conflict-free LDS reads return
     python3 -m f2cgt_amd.experiments cold-parts c2|c3|c4|c5   launch time by what of the input is still cached (any build)
@@ -207,8 +207,10 @@ def _affine_case(torch, synth, gen, n_src, bits, dim, rows, fanout):
 
 
 def affine_geometry(_):
-    """The affine row-block kernel at 3e6 edges, 10-20 edges per row: the shipped geometry against 64-thread
-    workgroups and against eight rows per block (F2CGT_ACC_TB / F2CGT_ACC_RB, experiments build)."""
+    """The affine row-block kernel at 3e6 edges over a range of edges per row: the shipped choices against the
+    interleaved edge-to-lane-group mapping, the accumulators sized for the narrow layout (4-bit codes: long
+    rows then take two passes), eight rows per block, and 64-thread workgroups (F2CGT_ACC_CHUNK,
+    F2CGT_ACC_WIDE_FULL, F2CGT_ACC_RB, F2CGT_ACC_TB; experiments build)."""
     import torch
 
     sys.path.insert(0, ROOT)
@@ -219,12 +221,13 @@ def affine_geometry(_):
         raise SystemExit("the library in tree was built without --experiments")
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0)
-    cases = (("shipped", {}), ("8 rows", {"F2CGT_ACC_RB": "8"}), ("64 threads, 8 rows", {"F2CGT_ACC_TB": "64", "F2CGT_ACC_RB": "8"}),
-             ("256 threads, 16 rows", {"F2CGT_ACC_TB": "256", "F2CGT_ACC_RB": "16"}))
+    knobs = ("F2CGT_ACC_TB", "F2CGT_ACC_RB", "F2CGT_ACC_CHUNK", "F2CGT_ACC_WIDE_FULL")
+    cases = (("shipped", {}), ("interleaved", {"F2CGT_ACC_CHUNK": "0"}), ("narrow-sized", {"F2CGT_ACC_WIDE_FULL": "0"}),
+             ("8 rows", {"F2CGT_ACC_RB": "8"}), ("64 threads, 8 rows", {"F2CGT_ACC_TB": "64", "F2CGT_ACC_RB": "8"}))
     print("us per launch, 2.4e6 source rows, 3e6 edges: " + " | ".join(name for name, _ in cases))
     for bits in (4, 8):
         for dim in (100, 128):
-            for fanout in (10, 11, 12, 14, 16, 17, 18, 20):
+            for fanout in (3, 5, 8, 10, 12, 14, 17, 18, 20, 25, 30, 40):
                 rows = 3_000_000 // fanout
                 codes, params, indptr, ids = _affine_case(torch, synth, gen, 2_400_000, bits, dim, rows, fanout)
                 out = torch.empty((rows, dim), dtype=torch.float32, device="cuda")
@@ -232,12 +235,12 @@ def affine_geometry(_):
                 best = {}
                 for _ in range(2):
                     for name, env in cases:
-                        for k in ("F2CGT_ACC_TB", "F2CGT_ACC_RB"):
+                        for k in knobs:
                             os.environ.pop(k, None)
                         os.environ.update(env)
                         _, ms = bench._time_steps(step, 30, 10)
                         best[name] = min(best.get(name, 1e9), ms * 1e3)
-                for k in ("F2CGT_ACC_TB", "F2CGT_ACC_RB"):
+                for k in knobs:
                     os.environ.pop(k, None)
                 print("  %d bit, %3d columns, %2d edges per row: " % (bits, dim, fanout)
                       + " | ".join("%6.1f" % best[name] for name, _ in cases), flush=True)

@@ -524,6 +524,36 @@ def test_fused_affine_high_degree_rows(bits, d, max_deg):
     assert np.allclose(got, exact, rtol=1e-5, atol=1e-5 * np.abs(dec).max())
 
 
+@pytest.mark.parametrize("idx", [np.int64, np.int32])
+@pytest.mark.parametrize("bits,d", [(4, 100), (4, 128), (8, 128), (8, 36)])
+@pytest.mark.parametrize("mean_deg", [7, 12, 24])
+def test_fused_affine_six_and_more_edges_per_row(bits, d, mean_deg, idx):
+    """From six edges per row on the lane groups of the affine kernel take contiguous shares of a block's edges, from
+    nine on the accumulators of 4-bit codes are sized for 16-bit fields (rows above 17 edges), and 11-20 edges per row
+    run sixteen rows per block.  Ragged rows around those limits, empty rows, a last block of five rows."""
+    rng = np.random.default_rng(1000 * bits + 10 * d + mean_deg + (idx == np.int32))
+    N, R = 5000, 16 * 40 + 5
+    x = (rng.standard_normal((N, d)) * 2).astype(np.float32)
+    params = oc.sq_affine_params(x, bits)
+    codes = oc.sq_affine_compress(x, params, bits)
+    store = oc.packbits(codes, bits) if bits < 8 else codes
+    deg = rng.integers(0, 2 * mean_deg + 1, size=R)
+    deg[:8] = [0, 17, 18, 1, 0, 0, 40, 16]
+    deg[R - 1] = 19
+    indptr = np.zeros(R + 1, dtype=idx)
+    indptr[1:] = np.cumsum(deg)
+    E = int(indptr[-1])
+    assert E >= 6 * R
+    indices = rng.integers(0, N, size=E).astype(idx)
+    got = host(capi.sq_affine_decompress_spmm_csr(dev(store), dev(params), dev(indptr), dev(indices), bits, d))
+    dec = oc.sq_affine_decompress(store, params, bits, d)
+    exact = oc.spmm_csr(dec.astype(np.float64), indptr.astype(np.int64), indices.astype(np.int64))
+    assert np.allclose(got, exact, rtol=1e-5, atol=1e-5 * np.abs(dec).max())
+    assert not got[deg == 0].any()
+    one = np.nonzero(deg == 1)[0]
+    assert np.array_equal(got[one], dec[indices[indptr[one]]])
+
+
 @pytest.mark.parametrize("shape", [(8, 256, 16), (16, 256, 8), (4, 64, 5), (3, 64, 100)])
 def test_hybrid_vs_oracle(shape):
     n_cb, K, w = shape
