@@ -1712,8 +1712,14 @@ int sq_affine_acc_run(const uint8_t* codes, const float* params, int64_t param_s
 
 template <int TB>
 int launch_hybrid(HybArgs a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
-                  const char* what) {
-  a.edge_batch = 4 * TB;
+                  const char* what, int edges_per_thread = 4) {
+#ifdef F2CGT_EXPERIMENTS
+  if (const char* v = getenv("F2CGT_HYB_BATCH")) {   // edges of a block that are tagged at a time, per thread
+    const int want = atoi(v);
+    if (want == 4 || want == 8 || want == 16) edges_per_thread = want;
+  }
+#endif
+  a.edge_batch = edges_per_thread * TB;
   const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 1.0;
   const int want = (int)(1.5625 * TB / (avg_deg > 0.5 ? avg_deg : 0.5));   // ~1.5 edges per thread
   int rb = 8;
@@ -1805,8 +1811,21 @@ int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float*
     if (atoi(v) == 256) return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what);
   }
 #endif
-  if (a.ch2 <= 32 && avg_deg <= 32.0)
-    return launch_hybrid<64>(a, indptr, indices, idx_dtype, out, st, what);
+  // Beyond that: the smallest workgroup whose edge batch still holds eight rows of the average length, so that
+  // a block is tagged and gathered in one go (us for 1.2e7 edges, 128 columns, 256 threads x 4 edges against the
+  // choice below: 40 edges per row 318 -> 175, 64: 310 -> 181, 80: 342 -> 264, 128: 359 -> 284, 200: 655 -> 357;
+  // 256 columns: 40: 166 -> 149, 200: 587 -> 271; 64 columns, 2.4e7 edges: 100: 608 -> 394, 200: 971 -> 510).
+  if (a.ch2 <= 32) {
+    if (avg_deg <= 32.0) return launch_hybrid<64>(a, indptr, indices, idx_dtype, out, st, what);
+    if (avg_deg <= 64.0) return launch_hybrid<128>(a, indptr, indices, idx_dtype, out, st, what);
+    if (avg_deg <= 128.0) return launch_hybrid<128>(a, indptr, indices, idx_dtype, out, st, what, 8);
+    if (a.ch2 <= 16) return launch_hybrid<128>(a, indptr, indices, idx_dtype, out, st, what, 16);
+    return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what, 8);
+  }
+  // wider rows: 128 threads below 6 edges per row (2: 676 against 756 us, 5: 360 against 382) and from 24 to 64
+  if (avg_deg <= 6.0 || (avg_deg > 24.0 && avg_deg <= 64.0))
+    return launch_hybrid<128>(a, indptr, indices, idx_dtype, out, st, what);
+  if (avg_deg > 128.0) return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what, 8);
   return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what);
 }
 

@@ -7,6 +7,7 @@
     python3 -m f2cgt_amd.experiments dispatch-cost c4    the two-table kernel's grid with workgroups that return at once
     python3 -m f2cgt_amd.experiments hot-rows c4         the two-table kernel with the hottest source rows copied to LDS
     python3 -m f2cgt_amd.experiments affine-geometry x   the affine kernel by edges per row: edge mapping, accumulator sizing, block rows, workgroup size
+    python3 -m f2cgt_amd.experiments hybrid-geometry x   the two-table kernel by edges per row: workgroup size and edge batch
     python3 -m f2cgt_amd.experiments store-form x        plain against non-temporal output stores by shape (any build)
     python3 -m f2cgt_amd.experiments lds-rate x          bytes per clock and CU that conflict-free LDS reads return
     python3 -m f2cgt_amd.experiments cold-parts c2|c3|c4|c5   launch time by what of the input is still cached (any build)
@@ -246,6 +247,46 @@ def affine_geometry(_):
                       + " | ".join("%6.1f" % best[name] for name, _ in cases), flush=True)
 
 
+def hybrid_geometry(_):
+    """The two-table kernel over edges per row and row width: the shipped choice of workgroup size and edge batch
+    against fixed ones (F2CGT_HYB_TB threads x F2CGT_HYB_BATCH edges per thread; experiments build)."""
+    import torch
+
+    sys.path.insert(0, ROOT)
+    import bench
+    from f2cgt_amd import capi, synth
+
+    if not hasattr(capi.lib(), "f2cgt_experiment_set_acc_trace"):
+        raise SystemExit("the library in tree was built without --experiments")
+    cases = (("shipped", None), ("64x4", ("64", "4")), ("128x4", ("128", "4")), ("128x8", ("128", "8")),
+             ("128x16", ("128", "16")), ("256x4", ("256", "4")), ("256x8", ("256", "8")))
+    print("us per launch, 2e7-node tables, 1.2e7 edges x 128 / columns: " + " | ".join(name for name, _ in cases))
+    for dim, n_cb in ((64, 4), (128, 8), (256, 16)):
+        for fanout in (2, 5, 12, 20, 32, 48, 64, 80, 128, 200):
+            rows = int(12_000_000 / fanout / (dim / 128))
+            wl = synth.c4_hybrid(device="cuda", idx_dtype=torch.int64, N=20_000_000, D=dim, n_cb=n_cb, w=16, R=rows,
+                                 fanout=fanout)
+            out = torch.empty((rows, dim), dtype=torch.float32, device="cuda")
+            step = bench._launcher(capi, wl, out)
+            best = {}
+            for _ in range(2):
+                for name, env in cases:
+                    os.environ.pop("F2CGT_HYB_TB", None)
+                    os.environ.pop("F2CGT_HYB_BATCH", None)
+                    if env:
+                        if env[0] == "64" and fanout * 8 > 64 * int(env[1]):
+                            continue   # several batches per block: minutes per launch at the large sizes
+                        os.environ["F2CGT_HYB_TB"], os.environ["F2CGT_HYB_BATCH"] = env
+                    _, ms = bench._time_steps(step, 15, 4)
+                    best[name] = min(best.get(name, 1e9), ms * 1e3)
+            os.environ.pop("F2CGT_HYB_TB", None)
+            os.environ.pop("F2CGT_HYB_BATCH", None)
+            print("  %3d columns, %3d edges per row: " % (dim, fanout)
+                  + " | ".join(("%6.1f" % best[name]) if name in best else "     -" for name, _ in cases), flush=True)
+            del wl, out
+            torch.cuda.empty_cache()
+
+
 def store_form(_):
     """Plain against non-temporal output stores of the two SQ row-block kernels by output size, row width and
     edges per row, and what the default picks (f2cgt_set_store_mode; any build)."""
@@ -419,7 +460,7 @@ def cold_parts(name):
 
 if __name__ == "__main__":
     modes = {"wave-age": wave_age, "block-phases": block_phases, "dispatch-cost": dispatch_cost, "hot-rows": hot_rows,
-             "affine-geometry": affine_geometry, "store-form": store_form, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
+             "affine-geometry": affine_geometry, "hybrid-geometry": hybrid_geometry, "store-form": store_form, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
              "cold-parts": cold_parts}
     if len(sys.argv) != 3 or sys.argv[1] not in modes:
         print(__doc__)

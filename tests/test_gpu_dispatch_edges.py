@@ -1,5 +1,6 @@
 """Shapes on either side of the thresholds that pick a workgroup size or a row partition: the two-table kernel runs
-one wave per workgroup up to 32 edges per row and up to 128 columns and 256 threads otherwise, the
+one wave per workgroup up to 32 edges per row and up to 128 columns, and beyond that the smallest workgroup (128 or
+256 threads, 4 to 16 edges per thread) whose edge batch holds eight rows of the average length, the
 staged-rows kernel of the log-domain SQ runs 128 threads for 1/2-bit rows and 256 for 4/8-bit
 ones.  Every side of every threshold must give the oracle's result."""
 import numpy as np
@@ -28,8 +29,8 @@ def fixed_fanout(rng, rows, n_src, fanout, ragged):
     return indptr, rng.integers(0, n_src, size=int(indptr[-1]))
 
 
-@pytest.mark.parametrize("feat_dim", [128, 112, 144])
-@pytest.mark.parametrize("fanout", [1, 2, 7, 8, 32, 33])
+@pytest.mark.parametrize("feat_dim", [128, 112, 144, 48])
+@pytest.mark.parametrize("fanout", [1, 2, 7, 8, 24, 25, 32, 33, 64, 65, 128, 129, 260])
 @pytest.mark.parametrize("ragged", [False, True])
 def test_hybrid_on_both_sides_of_the_workgroup_thresholds(feat_dim, fanout, ragged):
     rng = np.random.default_rng(1000 * feat_dim + 10 * fanout + ragged)
