@@ -1182,10 +1182,22 @@ int launch_sq_rows(RowsArgs a, const void* indptr, const void* indices, int idx_
   a.nt_out = stream_output(a.R * (int64_t)a.feat_dim * 4, (int64_t)a.feat_dim * 4,
                            a.R > 0 ? (double)a.E / (double)a.R : 0.0) ? 1 : 0;
   const size_t lut_bytes = AFFINE ? 0 : (size_t)(((a.num_codebooks << BITS) + 3) & ~3) * 4;
-  int cap = (int)((20 * 1024) / (a.pitch + 4));
-  a.edge_cap = (cap > 2 * TB ? 2 * TB : (cap < 8 ? 8 : cap)) & ~1;  // even: keeps the staging 8-byte aligned
   const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 1.0;
   const double dg = avg_deg > 0.5 ? avg_deg : 0.5;
+  int cap = (int)((20 * 1024) / (a.pitch + 4));
+  cap = cap > 2 * TB ? 2 * TB : cap;
+  {
+    // Eight rows of the average length have to fit the staging, or every block reads its code rows unstaged
+    // (3e6 edges, 128 columns: 4-bit rows 75 us at 30 edges per row and 139 us at 40; 2-bit rows 60 and 132 us).
+    // The staging grows to hold them, up to 28 KB: 40 edges per row then take 100 and 87 us.  More than that
+    // leaves too few workgroups per CU (8-bit rows at 30 edges per row: 211 us staged in 36 KB against 140 us
+    // unstaged), and such launches keep the 20 KB and read unstaged.
+    const int want = (int)(8.0 * dg * 1.1) + 8;
+    int most = (int)((28 * 1024) / (a.pitch + 4));
+    most = most > 1024 ? 1024 : most;
+    if (want > cap && want <= most) cap = want;
+  }
+  a.edge_cap = (cap < 8 ? 8 : cap) & ~1;  // even: keeps the staging 8-byte aligned
   int rb = ((int)(0.6 * a.edge_cap / dg) + 4) / 8 * 8;
   rb = rb < 8 ? 8 : (rb > 64 ? 64 : rb);
   rb = shrink_rows_per_block(rb, a.R, 16, 8, 1024);

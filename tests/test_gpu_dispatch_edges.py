@@ -64,7 +64,7 @@ def test_fused_log_sq_with_either_workgroup_size(bits, feat_dim):
     cb = np.array([[0.01, 3.0, -6.643856, 1.5849625, 0.4]], dtype=np.float32)
     per = 8 // bits
     column_slice = (feat_dim + per - 1) // per * per        # one codebook, a multiple of the codes per byte
-    for fanout, ragged in ((2, True), (12, False), (40, True)):
+    for fanout, ragged in ((2, True), (12, False), (20, False), (40, True), (60, False)):
         indptr, indices = fixed_fanout(rng, 500, n, fanout, ragged)
         stored = codes.view(np.int8) if bits == 8 else codes
         want = oc.sq_decompress_spmm_csr(stored, cb, indptr, indices, bits, column_slice, feat_dim)
