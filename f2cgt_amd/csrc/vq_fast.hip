@@ -640,17 +640,33 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
             }
           }
         } else {
+          // A mini-block with more edges than the staging holds (rows longer than the degree the launch was
+          // sized for): its edges go through the same staging 64 at a time, ids and code bytes fetched by
+          // all lanes at once for each slice (two round trips per 64 edges, not hidden, instead of two per
+          // edge and lane group), and every slot adds the edges of its row that fall into the slice.
 #pragma unroll
           for (int h = 0; h < H; ++h) acc[h][0] = acc[h][1] = acc[h][2] = acc[h][3] = 0.f;
           n = re - rb;
           const int64_t e0 = chunk_e0(par) + eb0;
-          for (int k = sub; k < n; k += SPR) {
-            const int64_t id = clamp_idx(indices[e0 + rb + k], a.N);
-            const uint32_t code = a.codes[id * a.n_cb + tile * BT + byte_idx];
+          for (int base = 0; base < ne0; base += kWEdges) {
+            const int cnt = (ne0 - base) < kWEdges ? (ne0 - base) : kWEdges;
+            const int li = lane < cnt ? lane : cnt - 1;
+            const int64_t id = clamp_idx(indices[e0 + base + li], a.N);
+            const CW c = *reinterpret_cast<const CW*>(code_base + (uint64_t)id * (uint32_t)a.n_cb);
+            __builtin_amdgcn_wave_barrier();   // the previous slice has been read
+            *reinterpret_cast<CW*>(s_codes + lane * BT) = c;
+            __builtin_amdgcn_wave_barrier();
+            const int wb = rb > base ? rb : base;
+            const int we = re < base + cnt ? re : base + cnt;
+            // edge k of the row (counted from the row's first edge) belongs to slot k % SPR
+            const int first = wb + (sub - (wb - rb) % SPR + SPR) % SPR;
+            for (int k = first; k < we; k += SPR) {
+              const uint32_t code = s_codes[(k - base) * BT + byte_idx];
 #pragma unroll
-            for (int h = 0; h < H; ++h) {
-              const float4 x = *reinterpret_cast<const float4*>(cbp + code * 128 + h * 64);
-              acc[h][0] += x.x; acc[h][1] += x.y; acc[h][2] += x.z; acc[h][3] += x.w;
+              for (int h = 0; h < H; ++h) {
+                const float4 x = *reinterpret_cast<const float4*>(cbp + code * 128 + h * 64);
+                acc[h][0] += x.x; acc[h][1] += x.y; acc[h][2] += x.z; acc[h][3] += x.w;
+              }
             }
           }
         }
@@ -1165,10 +1181,9 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     grid = (unsigned)cus;
   }
   const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 0.0;
-  // Graphs whose mini-blocks mostly fit the 64-edge staging take the wave-granular kernel: 4-row
-  // mini-blocks up to 15 edges per row, and, with whole 8-column groups in every tile (one lane
-  // per group, two float4 per edge), 2-row and 1-row mini-blocks up to 30 and 60 edges per row
-  // (larger mini-blocks for sparse rows were tried and were slower than 4-row ones).
+  // The wave-granular kernel: 4-row mini-blocks up to 16 edges per row, and, with whole 8-column
+  // groups in every tile (one lane per group, two float4 per edge), 2-row mini-blocks up to 32 and
+  // 1-row ones beyond (larger mini-blocks for sparse rows were tried and were slower than 4-row ones).
   const size_t wlds = (size_t)a.K * 128 * 4 + (size_t)(kThreads / 64) * (kWEdges * BT > 1024 ? kWEdges * BT : 1024) +
                       (size_t)(kThreads / 64) * 2 * kWPtr * 4;
   // with few edges per row the output dominates and its store pattern decides (fanout 2 at the C3
@@ -1195,10 +1210,29 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     }
   }
 #endif
+#ifdef F2CGT_EXPERIMENTS
+  if (const char* v = getenv("F2CGT_VQ_RPM")) {   // rows per mini-block whatever the degree (mini-blocks above 64 edges unstaged)
+    if (a.feat_dim % 8 == 0) {
+      if (atoi(v) == 4) return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+      if (atoi(v) == 2) return launch_wave<BT, 2, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+      if (atoi(v) == 1) return launch_wave<BT, 2, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    } else if (atoi(v) == 4) {
+      return launch_wave<BT, 1, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    }
+  }
+#endif
   if (a.feat_dim % 8 == 0) {
-    if (avg_deg <= 15.0) return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
-    if (avg_deg <= 30.0) return launch_wave<BT, 2, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
-    if (avg_deg <= 60.0) return launch_wave<BT, 2, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    // Rows per mini-block by the average degree: uniform rows of 16 / 32 / 64 edges just fit four / two / one
+    // (7.5e6 edges, 16 x 8: 16 edges per row 72 us in fours against 87 in twos, 32: 105 in twos against 167 one
+    // by one).  Mini-blocks with more edges than the staging holds go through it in slices (row_sum), so a
+    // graph whose rows are longer than its average suggests loses little (rows capped at 20 with 14.2 on
+    // average: 89 us in fours, 88 in twos; capped at 40 with 28.2: 161 in twos, 162 one by one), and rows of any
+    // length stay in this kernel: one-row mini-blocks at 64 / 200 / 2000 edges per row take 249 (2.56e7 edges) /
+    // 91 / 265 us where the block-synchronous kernel below, whose 1024-edge staging 64 such rows overflow,
+    // takes 1525 / 502 / 1624 us.
+    if (avg_deg <= 16.0) return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    if (avg_deg <= 32.0) return launch_wave<BT, 2, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    return launch_wave<BT, 2, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
   } else if (avg_deg <= 15.0) {
     return launch_wave<BT, 1, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
   }

@@ -8,6 +8,7 @@
     python3 -m f2cgt_amd.experiments hot-rows c4         the two-table kernel with the hottest source rows copied to LDS
     python3 -m f2cgt_amd.experiments affine-geometry x   the affine kernel by edges per row: edge mapping, accumulator sizing, block rows, workgroup size
     python3 -m f2cgt_amd.experiments hybrid-geometry x   the two-table kernel by edges per row: workgroup size and edge batch
+    python3 -m f2cgt_amd.experiments vq-degrees x        the fused VQ kernel on uniform and ragged rows: rows per mini-block
     python3 -m f2cgt_amd.experiments store-form x        plain against non-temporal output stores by shape (any build)
     python3 -m f2cgt_amd.experiments lds-rate x          bytes per clock and CU that conflict-free LDS reads return
     python3 -m f2cgt_amd.experiments cold-parts c2|c3|c4|c5   launch time by what of the input is still cached (any build)
@@ -287,6 +288,55 @@ def hybrid_geometry(_):
             torch.cuda.empty_cache()
 
 
+def vq_degrees(_):
+    """The fused VQ kernel (16 codebooks of 8 columns) on uniform rows and on rows capped at a fanout whose degrees
+    come from a heavy-tailed distribution: the shipped choice of rows per mini-block against four, two and one
+    (F2CGT_VQ_RPM; experiments build).  Mini-blocks above 64 edges go through the staging in slices."""
+    import torch
+
+    sys.path.insert(0, ROOT)
+    import bench
+    from f2cgt_amd import capi, synth
+
+    if not hasattr(capi.lib(), "f2cgt_experiment_set_acc_trace"):
+        raise SystemExit("the library in tree was built without --experiments")
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+    base = synth.c3_vq(device="cuda", idx_dtype=torch.int64, N=10_000_000, n_cb=16, K=256, w=8, R=1000, fanout=2)
+
+    def case(name, deg):
+        rows = deg.numel()
+        indptr = synth.csc_from_degrees(deg.to(torch.int64), torch.int64)
+        edges = int(indptr[-1])
+        wl = dict(base)
+        wl.update(indptr=indptr, indices=synth.zipf_ids(10_000_000, (edges,), 1.1, gen, "cuda", torch.int64), R=rows, E=edges)
+        out = torch.empty((rows, 128), dtype=torch.float32, device="cuda")
+        step = bench._launcher(capi, wl, out)
+        res = []
+        for rpm in ("", "4", "2", "1"):
+            os.environ.pop("F2CGT_VQ_RPM", None)
+            if rpm:
+                os.environ["F2CGT_VQ_RPM"] = rpm
+            _, ms = bench._time_steps(step, 10, 3)
+            res.append(ms * 1e3)
+        os.environ.pop("F2CGT_VQ_RPM", None)
+        print("  %-38s mean %6.2f, longest %4d, %8d edges: %7.1f | %7.1f | %7.1f | %7.1f"
+              % (name, edges / rows, int(deg.max()), edges, *res), flush=True)
+
+    print("us per launch: shipped | four | two | one row per mini-block")
+    rows = 400_000
+    for fanout in (15, 16, 20, 25, 32, 40, 64, 80, 200):
+        n = rows if fanout <= 80 else rows // 4
+        case("every row %d edges" % fanout, torch.full((n,), fanout, device="cuda"))
+        if fanout > 80:
+            continue
+        u = torch.rand((rows,), generator=gen, device="cuda")
+        for scale in (0.5, 1.0, 3.0):
+            raw = (scale * fanout * (1.0 - u).pow(-1.0 / 1.5)).floor().clamp(min=1)
+            raw = (raw * torch.rand((rows,), generator=gen, device="cuda")).ceil()
+            case("capped at %d, scale %.1f" % (fanout, scale), raw.clamp(max=fanout))
+
+
 def store_form(_):
     """Plain against non-temporal output stores of the two SQ row-block kernels by output size, row width and
     edges per row, and what the default picks (f2cgt_set_store_mode; any build)."""
@@ -460,7 +510,7 @@ def cold_parts(name):
 
 if __name__ == "__main__":
     modes = {"wave-age": wave_age, "block-phases": block_phases, "dispatch-cost": dispatch_cost, "hot-rows": hot_rows,
-             "affine-geometry": affine_geometry, "hybrid-geometry": hybrid_geometry, "store-form": store_form, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
+             "affine-geometry": affine_geometry, "hybrid-geometry": hybrid_geometry, "vq-degrees": vq_degrees, "store-form": store_form, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
              "cold-parts": cold_parts}
     if len(sys.argv) != 3 or sys.argv[1] not in modes:
         print(__doc__)

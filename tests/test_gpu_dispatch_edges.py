@@ -107,7 +107,7 @@ def test_fused_sq_on_both_sides_of_the_rows_per_block_steps(rows):
 
 @pytest.mark.parametrize("mean_deg", [22, 45])
 def test_fused_vq_chunk_dealing_with_shared_rows(mean_deg):
-    """Above 15 edges per row on average the lane groups of a pass share a row (two or one row per
+    """Above 16 edges per row on average the lane groups of a pass share a row (two or one row per
     mini-block); the same chunk dealing, sums no longer in edge order: rtol 1e-5."""
     rng = np.random.default_rng(mean_deg)
     rows, n_src, n_cb, width, feat_dim = 256 * 200 + 9, 20000, 16, 8, 128
@@ -128,6 +128,36 @@ def test_fused_vq_chunk_dealing_with_shared_rows(mean_deg):
     sub_idx = np.concatenate([indices[indptr[r]:indptr[r + 1]] for r in sample]).astype(np.int64)
     want = oc.vq_decompress_spmm_csr(codes, cbs, sub_ptr, sub_idx, feat_dim)
     assert np.allclose(got.cpu().numpy()[sample], want, rtol=RTOL, atol=RTOL * np.abs(want).max())
+
+
+@pytest.mark.parametrize("idx", [np.int64, np.int32])
+@pytest.mark.parametrize("n_cb,width", [(16, 8), (6, 32)])
+@pytest.mark.parametrize("mean_deg", [10, 16, 25, 32, 50, 100, 300])
+def test_fused_vq_rows_and_mini_blocks_longer_than_the_staging(mean_deg, n_cb, width, idx):
+    """Four-, two- and one-row mini-blocks (up to 16 / 32 / beyond edges per row on average) whose edges exceed the 64
+    a wave stages go through the staging in slices: ragged rows around the average, rows of 65, 128, 129 and 700 edges,
+    empty rows, and uniform rows at the limits (16, 32) where every mini-block is exactly full."""
+    rng = np.random.default_rng(1000 * mean_deg + n_cb + (idx == np.int32))
+    feat_dim = n_cb * width
+    rows, n_src = 16 * 12 * 9 + 7, 30000
+    codes = rng.integers(0, 256, size=(n_src, n_cb), dtype=np.uint8)
+    cbs = rng.standard_normal((n_cb, 256, width)).astype(np.float32)
+    if mean_deg in (16, 32):
+        deg = np.full(rows, mean_deg)
+    else:
+        deg = rng.integers(0, 2 * mean_deg + 1, size=rows)
+        deg[[3, 50, 51, 400]] = [65, 128, 129, 700]
+        deg[rng.integers(0, rows, size=rows // 20)] = 0
+    indptr = np.zeros(rows + 1, dtype=idx)
+    indptr[1:] = np.cumsum(deg)
+    indices = rng.integers(0, n_src, size=int(indptr[-1])).astype(idx)
+    got = capi.vq_decompress_spmm_csr(dev(codes), dev(cbs), dev(indptr), dev(indices), feat_dim)
+    torch.cuda.synchronize()
+    want = oc.vq_decompress_spmm_csr(codes, cbs, indptr.astype(np.int64), indices.astype(np.int64), feat_dim)
+    dec = oc.vq_decompress(codes, cbs, feat_dim).astype(np.float64)
+    exact = oc.spmm_csr(dec, indptr.astype(np.int64), indices.astype(np.int64))
+    assert_mean_aggregate(got.cpu().numpy(), want, exact, float(np.abs(dec).max()))
+    assert not got.cpu().numpy()[deg == 0].any()
 
 
 @pytest.mark.parametrize("idx", [np.int64, np.int32])
