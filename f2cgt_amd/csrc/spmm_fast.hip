@@ -1827,17 +1827,22 @@ int hybrid_acc_run(const int32_t* row_map, const uint8_t* sq_codes, const float*
   // a block is tagged and gathered in one go (us for 1.2e7 edges, 128 columns, 256 threads x 4 edges against the
   // choice below: 40 edges per row 318 -> 175, 64: 310 -> 181, 80: 342 -> 264, 128: 359 -> 284, 200: 655 -> 357;
   // 256 columns: 40: 166 -> 149, 200: 587 -> 271; 64 columns, 2.4e7 edges: 100: 608 -> 394, 200: 971 -> 510).
+  // The limits are exact fits for rows of one length, which an edge count that is a multiple of the row count
+  // gives away (a sampled block with a fixed fanout); ragged rows get a quarter of slack, since a block over its
+  // batch takes several rounds (rows capped at 40 with 28.2 on average: 166 us with 256-edge batches, twice the
+  // time per edge of its neighbours).
+  const double fit = (R > 0 && E % R == 0) ? 1.0 : 0.8;
   if (a.ch2 <= 32) {
-    if (avg_deg <= 32.0) return launch_hybrid<64>(a, indptr, indices, idx_dtype, out, st, what);
-    if (avg_deg <= 64.0) return launch_hybrid<128>(a, indptr, indices, idx_dtype, out, st, what);
-    if (avg_deg <= 128.0) return launch_hybrid<128>(a, indptr, indices, idx_dtype, out, st, what, 8);
+    if (avg_deg <= 32.0 * fit) return launch_hybrid<64>(a, indptr, indices, idx_dtype, out, st, what);
+    if (avg_deg <= 64.0 * fit) return launch_hybrid<128>(a, indptr, indices, idx_dtype, out, st, what);
+    if (avg_deg <= 128.0 * fit) return launch_hybrid<128>(a, indptr, indices, idx_dtype, out, st, what, 8);
     if (a.ch2 <= 16) return launch_hybrid<128>(a, indptr, indices, idx_dtype, out, st, what, 16);
     return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what, 8);
   }
   // wider rows: 128 threads below 6 edges per row (2: 676 against 756 us, 5: 360 against 382) and from 24 to 64
-  if (avg_deg <= 6.0 || (avg_deg > 24.0 && avg_deg <= 64.0))
+  if (avg_deg <= 6.0 || (avg_deg > 24.0 && avg_deg <= 64.0 * fit))
     return launch_hybrid<128>(a, indptr, indices, idx_dtype, out, st, what);
-  if (avg_deg > 128.0) return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what, 8);
+  if (avg_deg > 128.0 * fit) return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what, 8);
   return launch_hybrid<256>(a, indptr, indices, idx_dtype, out, st, what);
 }
 

@@ -1230,8 +1230,12 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     // length stay in this kernel: one-row mini-blocks at 64 / 200 / 2000 edges per row take 249 (2.56e7 edges) /
     // 91 / 265 us where the block-synchronous kernel below, whose 1024-edge staging 64 such rows overflow,
     // takes 1525 / 502 / 1624 us.
-    if (avg_deg <= 16.0) return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
-    if (avg_deg <= 32.0) return launch_wave<BT, 2, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    // An edge count that is a multiple of the row count gives rows of one length away (a sampled block with a
+    // fixed fanout): those get the exact limits, ragged rows 0.9 of them (capped at 32 with 15.2 on average: 112 us
+    // in fours, 91 in twos; capped at 64 with 30.1: 198 in twos, 171 one by one).
+    const double fit = (a.R > 0 && a.E % a.R == 0) ? 1.0 : 0.9;
+    if (avg_deg <= 16.0 * fit) return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    if (avg_deg <= 32.0 * fit) return launch_wave<BT, 2, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
     return launch_wave<BT, 2, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
   } else if (avg_deg <= 15.0) {
     return launch_wave<BT, 1, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
