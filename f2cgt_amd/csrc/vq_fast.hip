@@ -297,7 +297,11 @@ constexpr int kWPtr = 56;                     // ints per offset buffer: [0..12]
 
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
-template <int BT, int H, int RPM, typename Idx, bool DENSE = false, bool TRACE = false>
+// TAIL: code rows whose length is no multiple of BT (13 codebooks of 8 columns for 100 features: one tile of 13 code
+// bytes).  The BT bytes a lane fetches for its tile then start at any byte of the table, reach into the next row
+// (bytes the tile has no columns for) and, for the table's last row or two, past its end: those rows are fetched
+// byte by byte.
+template <int BT, int H, int RPM, typename Idx, bool DENSE = false, bool TRACE = false, bool TAIL = false>
 __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* __restrict__ indptr,
                                                            const Idx* __restrict__ indices,
                                                            float* __restrict__ out) {
@@ -375,6 +379,30 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   const float* cbp = s_cb + c4 * 4;
   const uint8_t* code_base = a.codes + tile * BT;
   const uint32_t n_last = (uint32_t)(a.N - 1);
+  // the last source row whose BT bytes for this tile lie inside the table (TAIL only)
+  const int64_t tail_room = (int64_t)a.N * a.n_cb - (int64_t)tile * BT - BT;
+  const int64_t safe_last = tail_room >= 0 ? tail_room / a.n_cb : -1;
+  auto load_codes = [&](uint32_t id) -> CW {
+    const uint8_t* src = code_base + (uint64_t)id * (uint32_t)a.n_cb;
+    CW c;
+    if constexpr (!TAIL) {
+      c = *reinterpret_cast<const CW*>(src);
+    } else {
+      if ((int64_t)id <= safe_last) {
+        __builtin_memcpy(&c, src, sizeof(CW));   // any alignment
+      } else {
+        uint32_t word[BT / 4];
+#pragma unroll
+        for (int d = 0; d < BT / 4; ++d) word[d] = 0u;
+        const int have = a.n_cb - tile * BT;     // code bytes of this tile in a row (< BT here)
+#pragma unroll
+        for (int b = 0; b < BT; ++b)
+          if (b < have) word[b >> 2] |= (uint32_t)src[b] << (8 * (b & 3));
+        __builtin_memcpy(&c, word, sizeof(CW));
+      }
+    }
+    return c;
+  };
 
   // loads the row offsets of the chunk that starts at row0, and parks them in offset buffer `which`
   int64_t Preg = 0;
@@ -467,7 +495,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     {
       const uint64_t raw = (uint64_t)Ireg;
       const uint32_t id = (raw >> 32) ? n_last : ((uint32_t)raw < n_last ? (uint32_t)raw : n_last);
-      Creg = *reinterpret_cast<const CW*>(code_base + (uint64_t)(on ? id : 0u) * (uint32_t)a.n_cb);   // C(0)
+      Creg = load_codes(on ? id : 0u);   // C(0)
     }
     {
       const bool v = has_rows && 1 < n_mini;
@@ -517,7 +545,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     {  // C(g+1): the id fetched one step ago is clamped only now (ids outside [0, N) read row N - 1)
       const uint64_t raw = (uint64_t)Ireg;
       const uint32_t id = (raw >> 32) ? n_last : ((uint32_t)raw < n_last ? (uint32_t)raw : n_last);
-      Creg = *reinterpret_cast<const CW*>(code_base + (uint64_t)id * (uint32_t)a.n_cb);
+      Creg = load_codes(id);
     }
     eb2 = 0; ne2 = 0;
     {  // I(g+2)
@@ -652,7 +680,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
             const int cnt = (ne0 - base) < kWEdges ? (ne0 - base) : kWEdges;
             const int li = lane < cnt ? lane : cnt - 1;
             const int64_t id = clamp_idx(indices[e0 + base + li], a.N);
-            const CW c = *reinterpret_cast<const CW*>(code_base + (uint64_t)id * (uint32_t)a.n_cb);
+            const CW c = load_codes((uint32_t)id);
             __builtin_amdgcn_wave_barrier();   // the previous slice has been read
             *reinterpret_cast<CW*>(s_codes + lane * BT) = c;
             __builtin_amdgcn_wave_barrier();
@@ -1146,9 +1174,14 @@ int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int id
 #endif
   // the sparse-row form (results turned round in LDS before they are stored) is its own instantiation
   constexpr bool CAN_DENSE = H == 2 && RPM == 4;
-  const bool dense = CAN_DENSE && a.dense_store == 1;
+  const bool tail = a.n_cb % BT != 0 || !aligned(a.codes, BT);
+  const bool dense = CAN_DENSE && a.dense_store == 1 && !tail;
   const void* kern;
-  if (idx_dtype == F2CGT_DT_I32)
+  if (tail)
+    kern = idx_dtype == F2CGT_DT_I32
+               ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false, false, true>)
+               : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t, false, false, true>);
+  else if (idx_dtype == F2CGT_DT_I32)
     kern = dense ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, CAN_DENSE>)
                  : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false>);
   else
@@ -1197,7 +1230,7 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     const char* v = getenv("F2CGT_VQ_STRIP");
     const int mode = v ? atoi(v) : 0;     // 0 off; tens: 0 plain, 1 non-temporal, 2 no stores; units: 2 = KE by degree, 6 = KE 16
     if (mode == 20) a.dense_store = 2;
-    if (mode % 10 > 0 && avg_deg <= 24.0) {
+    if (mode % 10 > 0 && avg_deg <= 24.0 && a.n_cb % BT == 0 && aligned(a.codes, BT)) {
       VqArgs b = a;
       b.dense_store = (mode / 10) % 10;
       if (mode >= 100) b.N = 1;   // experiment: every source id reads row 0
@@ -1237,7 +1270,8 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     if (avg_deg <= 16.0 * fit) return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
     if (avg_deg <= 32.0 * fit) return launch_wave<BT, 2, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
     return launch_wave<BT, 2, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
-  } else if (avg_deg <= 15.0) {
+  } else if (avg_deg <= 15.0 || a.n_cb % BT != 0 || !aligned(a.codes, BT)) {
+    // (the block-synchronous kernel below reads whole aligned code words; longer rows go through the staging in slices)
     return launch_wave<BT, 1, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
   }
   if (plan_only()) {
@@ -1268,8 +1302,6 @@ bool vq_pipe_eligible(const void* codes, const float* codebooks, const float* ou
   if (E < 1 || N < 1 || codes == nullptr) return false;  // idle lanes read row 0 / indptr[0]
   if (K < 1 || K > 256) return false;
   if (w != 8 && w != 16 && w != 32) return false;
-  const int bt = 128 / w;
-  if (n_cb % bt != 0 || !aligned(codes, bt)) return false;
   if (feat_dim < 16 || feat_dim % 4 != 0 || feat_dim > n_cb * w) return false;
   if (!aligned(out, 16) || !aligned(codebooks, 4)) return false;
   if (N >= (1ll << 32)) return false;

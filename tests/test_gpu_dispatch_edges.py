@@ -131,6 +131,33 @@ def test_fused_vq_chunk_dealing_with_shared_rows(mean_deg):
 
 
 @pytest.mark.parametrize("idx", [np.int64, np.int32])
+@pytest.mark.parametrize("feat_dim,n_cb,width", [(100, 13, 8), (64, 8, 8), (96, 12, 8), (192, 24, 8), (160, 5, 32),
+                                                 (96, 3, 32), (48, 3, 16), (200, 13, 16), (100, 4, 32), (600, 19, 32),
+                                                 (120, 16, 8)])
+@pytest.mark.parametrize("mean_deg", [3, 12, 40])
+def test_fused_vq_code_rows_that_are_no_multiple_of_a_tile(feat_dim, n_cb, width, mean_deg, idx):
+    """Code rows of 13, 8, 12, 24 ... bytes where a 128-column tile takes 16 (8, 4) of them: the pipelined kernel
+    fetches its code words at any alignment and reads the table's last rows byte by byte.  Many edges name the last two
+    source rows; feat_dim may be less than n_cb * width (the reference's truncation)."""
+    rng = np.random.default_rng(feat_dim * 100 + mean_deg + (idx == np.int32))
+    n_src, rows = 777, 3000
+    codes = rng.integers(0, 256, size=(n_src, n_cb), dtype=np.uint8)
+    cbs = rng.standard_normal((n_cb, 256, width)).astype(np.float32)
+    deg = rng.integers(0, 2 * mean_deg + 1, size=rows)
+    indptr = np.zeros(rows + 1, dtype=idx)
+    indptr[1:] = np.cumsum(deg)
+    indices = rng.integers(0, n_src, size=int(indptr[-1])).astype(idx)
+    indices[::7] = n_src - 1
+    indices[1::11] = n_src - 2
+    got = capi.vq_decompress_spmm_csr(dev(codes), dev(cbs), dev(indptr), dev(indices), feat_dim)
+    torch.cuda.synchronize()
+    want = oc.vq_decompress_spmm_csr(codes, cbs, indptr.astype(np.int64), indices.astype(np.int64), feat_dim)
+    dec = oc.vq_decompress(codes, cbs, feat_dim).astype(np.float64)
+    exact = oc.spmm_csr(dec, indptr.astype(np.int64), indices.astype(np.int64))
+    assert_mean_aggregate(got.cpu().numpy(), want, exact, float(np.abs(dec).max()))
+
+
+@pytest.mark.parametrize("idx", [np.int64, np.int32])
 @pytest.mark.parametrize("n_cb,width", [(16, 8), (6, 32)])
 @pytest.mark.parametrize("mean_deg", [10, 16, 25, 32, 50, 100, 300])
 def test_fused_vq_rows_and_mini_blocks_longer_than_the_staging(mean_deg, n_cb, width, idx):

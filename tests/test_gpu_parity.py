@@ -924,7 +924,10 @@ def test_module_surface_end_to_end():
     ipv, ixv = random_graph(rng, 400, 3000, 15)
     o1 = lib.spmm_csr(lib.vq_decompress(codes8, cbk, 16), dev(ipv), dev(ixv))
     o2 = lib.vq_decompress_spmm_csr(codes8, cbk, dev(ipv), dev(ixv), 16)
-    assert torch.equal(o1, o2)
+    # 400 rows take the pipelined kernel, whose mean is the sum times a refined reciprocal: within 2 ulp of the
+    # division that spmm_csr performs (the reference's own 3-row case stays on the bit-exact per-row form)
+    dec64 = host(lib.vq_decompress(codes8, cbk, 16)).astype(np.float64)
+    assert_mean_aggregate(host(o2), host(o1), oc.spmm_csr(dec64, ipv, ixv), float(np.abs(dec64).max()))
     with pytest.raises(RuntimeError, match="column_slice"):
         lib.sq_decompress_spmm_csr(exp, dev(cb), ip, ix, 4, 0, 100)
     with pytest.raises(RuntimeError):
