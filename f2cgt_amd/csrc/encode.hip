@@ -1236,6 +1236,151 @@ __global__ __launch_bounds__(256) void pairwise_kernel(const float* __restrict__
   }
 }
 
+// ---- any dimension, any number of centres: vector-ALU tiles with a running arg-min ----------------
+// The assignment for shapes the matrix-core kernels do not take (more than 64 dimensions, or centres that do
+// not fit their LDS layout).  A 256-thread workgroup owns 128 rows of x and walks the centres in tiles of 128
+// with the 8 x 8 register tiles of pairwise_kernel (unexpanded sum of squared differences, or the cosine
+// distance); instead of writing the distances a thread keeps, for each of its 8 rows, the smallest and the
+// second smallest score and the centre of the smallest (first minimum: strict compares in rising centre order),
+// and the 16 threads of a row combine theirs at the end.  fp32 sums of k terms are good to about k ulp, so a
+// row whose two best scores are closer than that is decided again by exact_argmin_row (float64, one wave per
+// such row), as is a row without a finite score.
+__global__ __launch_bounds__(256) void predict_tiled_kernel(const float* __restrict__ x,
+                                                            const float* __restrict__ centers,
+                                                            int64_t* __restrict__ lab64,
+                                                            uint8_t* __restrict__ lab8, int64_t m, int n, int k,
+                                                            int metric) {
+  __shared__ __align__(16) float xs[kChunk][kTile + 4];
+  __shared__ __align__(16) float ys[kChunk][kTile + 4];
+  __shared__ int s_again[kTile];
+  __shared__ int s_count;
+  const int tx = threadIdx.x & 15;  // 8 centres of a tile each
+  const int ty = threadIdx.x >> 4;  // 8 rows each
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const bool cosine = metric == F2CGT_METRIC_COSINE;
+  const float tol = (float)(k + 8) * 2.4e-7f;
+  const int64_t row_tiles = (m + kTile - 1) / kTile;
+  for (int64_t rt = blockIdx.x; rt < row_tiles; rt += gridDim.x) {
+    const int64_t i0 = rt * kTile;
+    float best[8], second[8];
+    int arg[8];
+#pragma unroll
+    for (int a = 0; a < 8; ++a) {
+      best[a] = INFINITY;
+      second[a] = INFINITY;
+      arg[a] = 0;
+    }
+    if (threadIdx.x == 0) s_count = 0;
+    for (int j0 = 0; j0 < n; j0 += kTile) {
+      float acc[8][8], xn[8], yn[8];
+#pragma unroll
+      for (int a = 0; a < 8; ++a) {
+        xn[a] = 0.f;
+        yn[a] = 0.f;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) acc[a][b] = 0.f;
+      }
+      for (int k0 = 0; k0 < k; k0 += kChunk) {
+        __syncthreads();
+        for (int t = threadIdx.x; t < kTile * kChunk; t += 256) {
+          const int r = t / kChunk, c = t % kChunk;
+          const bool kin = k0 + c < k;
+          xs[c][r] = (kin && i0 + r < m) ? x[(i0 + r) * k + k0 + c] : 0.f;
+          ys[c][r] = (kin && j0 + r < n) ? centers[(int64_t)(j0 + r) * k + k0 + c] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int c = 0; c < kChunk; ++c) {
+          float xv[8], yv[8];
+          const float4 xa = *reinterpret_cast<const float4*>(&xs[c][ty * 8]);
+          const float4 xb = *reinterpret_cast<const float4*>(&xs[c][ty * 8 + 4]);
+          const float4 ya = *reinterpret_cast<const float4*>(&ys[c][tx * 4]);
+          const float4 yb = *reinterpret_cast<const float4*>(&ys[c][64 + tx * 4]);
+          xv[0] = xa.x; xv[1] = xa.y; xv[2] = xa.z; xv[3] = xa.w; xv[4] = xb.x; xv[5] = xb.y; xv[6] = xb.z; xv[7] = xb.w;
+          yv[0] = ya.x; yv[1] = ya.y; yv[2] = ya.z; yv[3] = ya.w; yv[4] = yb.x; yv[5] = yb.y; yv[6] = yb.z; yv[7] = yb.w;
+          if (cosine) {
+#pragma unroll
+            for (int a = 0; a < 8; ++a) {
+              xn[a] = __fmaf_rn(xv[a], xv[a], xn[a]);
+              yn[a] = __fmaf_rn(yv[a], yv[a], yn[a]);
+#pragma unroll
+              for (int b = 0; b < 8; ++b) acc[a][b] = __fmaf_rn(xv[a], yv[b], acc[a][b]);
+            }
+          } else {
+#pragma unroll
+            for (int a = 0; a < 8; ++a)
+#pragma unroll
+              for (int b = 0; b < 8; ++b) {
+                const float d = xv[a] - yv[b];
+                acc[a][b] = __fmaf_rn(d, d, acc[a][b]);
+              }
+          }
+        }
+      }
+      // the tile's scores into the running (best, second, centre) of the thread's rows, centres in rising order
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const int col = j0 + tx * 4 + (b & 3) + (b >> 2) * 64;
+#pragma unroll
+        for (int a = 0; a < 8; ++a) {
+          float v = acc[a][b];
+          if (cosine) {
+            float den = sqrtf(xn[a]) * sqrtf(yn[b]);
+            den = den > 1e-8f ? den : 1e-8f;
+            v = 1.f - v / den;
+          }
+          if (col >= n) v = INFINITY;
+          const bool lt = v < best[a];
+          second[a] = __builtin_amdgcn_fmed3f(best[a], second[a], v);
+          arg[a] = lt ? col : arg[a];
+          best[a] = lt ? v : best[a];
+        }
+      }
+    }
+    // the 16 threads of a row (consecutive lanes) combine: smallest score, lowest centre among equals
+#pragma unroll
+    for (int a = 0; a < 8; ++a) {
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1) {
+        const float ob = __shfl_xor(best[a], off), os = __shfl_xor(second[a], off);
+        const int oa = __shfl_xor(arg[a], off);
+        const bool take = ob < best[a] || (ob == best[a] && oa < arg[a]);
+        const float hi = take ? best[a] : ob;          // the larger of the two smallest
+        second[a] = fminf(fminf(second[a], os), hi);
+        arg[a] = take ? oa : arg[a];
+        best[a] = take ? ob : best[a];
+      }
+    }
+    __syncthreads();   // s_count cleared, staging no longer read
+    if (tx == 0) {
+#pragma unroll
+      for (int a = 0; a < 8; ++a) {
+        const int64_t i = i0 + ty * 8 + a;
+        if (i >= m) continue;
+        // NaN compares false everywhere: a row of NaN keeps best = inf and is decided by the exact form
+        const bool close = !(second[a] - best[a] > tol * (cosine ? 1.f : (fabsf(best[a]) + fabsf(second[a]))));
+        if (close || !(best[a] < INFINITY)) {
+          s_again[atomicAdd(&s_count, 1)] = ty * 8 + a;
+        } else {
+          if (lab64) lab64[i] = arg[a];
+          if (lab8) lab8[i] = (uint8_t)arg[a];
+        }
+      }
+    }
+    __syncthreads();
+    const int again = s_count;
+    for (int f = wave; f < again; f += 4) {
+      const int64_t i = i0 + s_again[f];
+      const int lab = exact_argmin_row(x + i * k, centers, n, k, metric, lane);
+      if (lane == 0) {
+        if (lab64) lab64[i] = lab;
+        if (lab8) lab8[i] = (uint8_t)lab;
+      }
+    }
+    __syncthreads();   // s_again read before the next row tile clears the count
+  }
+}
+
 template <int KH>
 int launch_mfma(const float* x, const float* centers, int64_t* l64, uint8_t* l8, int64_t m, int n,
                 int k, int metric, int n_pad, size_t lds, hipStream_t st) {
@@ -1379,6 +1524,13 @@ extern "C" int f2cgt_kmeans_predict(const float* x, const float* centers, int64_
       case 16: return launch_mfma<16>(x, centers, labels_i64, labels_u8, m, (int)n, (int)k, metric, n_pad, lds, st);
       default: return launch_mfma<32>(x, centers, labels_i64, labels_u8, m, (int)n, (int)k, metric, n_pad, lds, st);
     }
+  }
+  if (m >= 64) {   // tiles of 128 rows (a handful of rows: one wave per row, exact, below)
+    const int64_t tiles = ceil_div(m, (int64_t)kTile);
+    const int64_t cap = (int64_t)num_cus() * 4;
+    predict_tiled_kernel<<<(int)(tiles < cap ? tiles : cap), 256, 0, st>>>(x, centers, labels_i64, labels_u8, m,
+                                                                         (int)n, (int)k, metric);
+    return launch_status("kmeans_predict");
   }
   int64_t need = ceil_div(m, 4);
   int64_t cap = (int64_t)num_cus() * 8;

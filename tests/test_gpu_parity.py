@@ -720,7 +720,11 @@ def test_pairwise_cosine_with_vectors_without_a_direction():
 
 @pytest.mark.parametrize("metric", ["l2", "cosine"])
 @pytest.mark.parametrize("m,n,k", [(20000, 256, 32), (5000, 256, 8), (3001, 100, 16), (777, 37, 5),
-                                   (4000, 256, 64), (500, 1000, 24), (300, 50, 200)])
+                                   (4000, 256, 64), (500, 1000, 24), (300, 50, 200),
+                                   # beyond the matrix-core kernels (more than 64 dimensions, many centres): tiles on the
+                                   # vector ALUs with a running arg-min; 63 rows and fewer: one wave per row
+                                   (5000, 256, 65), (3000, 300, 128), (700, 4096, 8), (129, 17, 200), (64, 3, 70),
+                                   (63, 5, 100), (4000, 256, 96), (1000, 512, 64)])
 def test_kmeans_predict_vs_oracle(metric, m, n, k):
     rng = np.random.default_rng(m + n + k)
     x = rng.standard_normal((m, k)).astype(np.float32)
@@ -735,7 +739,7 @@ def test_kmeans_predict_vs_oracle(metric, m, n, k):
 
 
 @pytest.mark.parametrize("metric", ["l2", "cosine"])
-@pytest.mark.parametrize("m,n,k", [(2000, 8, 8), (3000, 256, 32), (500, 1000, 24), (300, 50, 200)])
+@pytest.mark.parametrize("m,n,k", [(2000, 8, 8), (3000, 256, 32), (500, 1000, 24), (300, 50, 200), (3000, 256, 96)])
 def test_kmeans_predict_rows_that_are_not_numbers(metric, m, n, k):
     """Rows with NaN or infinite entries have no nearest centre.  Their labels must still be valid
     indices (centre 0: the callers' trainer turns NaN distances into 1 before its arg-min,
@@ -760,10 +764,11 @@ def test_kmeans_predict_rows_that_are_not_numbers(metric, m, n, k):
         assert np.array_equal(got8.astype(np.int64), got)
 
 
-def test_kmeans_predict_exact_ties_pick_first():
+@pytest.mark.parametrize("k", [32, 96])
+def test_kmeans_predict_exact_ties_pick_first(k):
     rng = np.random.default_rng(11)
-    x = rng.standard_normal((4000, 32)).astype(np.float32)
-    c = rng.standard_normal((256, 32)).astype(np.float32)
+    x = rng.standard_normal((4000, k)).astype(np.float32)
+    c = rng.standard_normal((256, k)).astype(np.float32)
     c[200] = c[7]
     c[255] = c[100]
     got = host(capi.kmeans_predict(dev(x), dev(c), "l2"))
