@@ -112,6 +112,22 @@ __device__ __forceinline__ void store_nt4(float* p, float a, float b, float c, f
   __builtin_nontemporal_store(v, reinterpret_cast<f4*>(p));
 }
 
+// The same 16 bytes at an address that is only a multiple of 8 (rows of 4 k + 2 columns): global memory takes a
+// four-dword store at any dword, so this is still one instruction.
+__device__ __forceinline__ void store_nt4_align8(float* p, float a, float b, float c, float d) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  typedef f4 f4a8 __attribute__((aligned(8)));
+  f4 v = {a, b, c, d};
+  __builtin_nontemporal_store(v, reinterpret_cast<f4a8*>(p));
+}
+
+__device__ __forceinline__ void store4_align8(float* p, float a, float b, float c, float d) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  typedef f4 f4a8 __attribute__((aligned(8)));
+  f4 v = {a, b, c, d};
+  *reinterpret_cast<f4a8*>(p) = v;
+}
+
 // Stages the 128-column tile `tile` of VQ codebooks [n_cb][K][w] (w a multiple of 4) into LDS as
 // [code][128 columns], columns from tile_cols on zero.  A thread issues UNROLL loads back to back
 // before it waits for the first, so the 128 KB of a 256-code tile cost a few load latencies

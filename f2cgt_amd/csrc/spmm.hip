@@ -125,6 +125,9 @@ struct PlainDec {
     if constexpr (NOUT_ == 4 && std::is_same<T, float>::value) {
       const float4 q = *reinterpret_cast<const float4*>(p);
       r.v[0] = q.x; r.v[1] = q.y; r.v[2] = q.z; r.v[3] = q.w;
+    } else if constexpr (NOUT_ == 2 && std::is_same<T, float>::value) {
+      const float2 q = *reinterpret_cast<const float2*>(p);
+      r.v[0] = q.x; r.v[1] = q.y;
     } else {
 #pragma unroll
       for (int i = 0; i < NOUT_; ++i) r.v[i] = p[i];
@@ -620,6 +623,11 @@ extern "C" int f2cgt_spmm_csr(const void* feat, int feat_dtype, void* out, const
         PlainDec<float, 4> d{static_cast<const float*>(feat), feat_dim};
         return run(d, indptr, indices, idx_dtype, static_cast<float*>(out), num_rows, num_edges,
                    num_src_rows, D, plan(num_rows, D, 1, 4, 0), 0, true, st, what);
+      }
+      if (D % 2 == 0 && aligned(feat, 8) && aligned(out, 8)) {   // rows of 8-byte pairs (602 columns: 961 us against 1703 with single floats)
+        PlainDec<float, 2> d{static_cast<const float*>(feat), feat_dim};
+        return run(d, indptr, indices, idx_dtype, static_cast<float*>(out), num_rows, num_edges,
+                   num_src_rows, D, plan(num_rows, D, 1, 2, 0), 0, true, st, what);
       }
       PlainDec<float, 1> d{static_cast<const float*>(feat), feat_dim};
       return run(d, indptr, indices, idx_dtype, static_cast<float*>(out), num_rows, num_edges,

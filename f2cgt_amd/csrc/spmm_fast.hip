@@ -438,21 +438,36 @@ struct FinParams {
   float mn[4], sc[4];
 };
 
+// HALF != 0: rows of 4 k + 2 columns.  They start at multiples of 8 bytes only and end with a group of two columns:
+// that group's parameters are fetched column by column (nothing is read past the row's last column), the 16-byte
+// stores go to any dword, and the last group stores its two columns alone.  HALF is 1 for cached and 2 for streamed
+// stores, fixed when the kernel is chosen: with both forms of the under-aligned store behind one run-time test the
+// compiler folds them into one and the streamed form is lost.
+template <int HALF = 0>
 __device__ __forceinline__ FinParams acc_fin_params(const AccArgs& a) {
   FinParams p;
   const int t = threadIdx.x;
   const int g = (int)(((uint32_t)t * a.fin_magic) >> 16);
   const int l = t - g * a.fin_group;
   const int c4 = (g < a.fin_slots && l < a.f4_per_row) ? l : 0;
+  if (HALF == 0 || c4 * 4 + 4 <= a.feat_dim) {   // four consecutive parameters: one load each for min and scale
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    p.mn[i] = a.params[c4 * 4 + i];
-    p.sc[i] = a.params[a.param_stride + c4 * 4 + i];
+    for (int i = 0; i < 4; ++i) {
+      p.mn[i] = a.params[c4 * 4 + i];
+      p.sc[i] = a.params[a.param_stride + c4 * 4 + i];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int col = c4 * 4 + i >= a.feat_dim ? a.feat_dim - 1 : c4 * 4 + i;
+      p.mn[i] = a.params[col];
+      p.sc[i] = a.params[a.param_stride + col];
+    }
   }
   return p;
 }
 
-template <int TB, int BITS, int NW>
+template <int TB, int BITS, int NW, int HALF = 0>
 __device__ __forceinline__ void acc_finalize(const AccArgs& a, const FinParams& first, const uint32_t* s_acc,
                                              const float* s_rdeg, int64_t row0, int rb, int nr, int pitch,
                                              float* __restrict__ out) {
@@ -469,12 +484,22 @@ __device__ __forceinline__ void acc_finalize(const AccArgs& a, const FinParams& 
       sc[i] = first.sc[i];
     }
     if (c4 != l) {
+      if (HALF == 0 || c4 * 4 + 4 <= a.feat_dim) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        mn[i] = a.params[c4 * 4 + i];
-        sc[i] = a.params[a.param_stride + c4 * 4 + i];
+        for (int i = 0; i < 4; ++i) {
+          mn[i] = a.params[c4 * 4 + i];
+          sc[i] = a.params[a.param_stride + c4 * 4 + i];
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int col = c4 * 4 + i >= a.feat_dim ? a.feat_dim - 1 : c4 * 4 + i;
+          mn[i] = a.params[col];
+          sc[i] = a.params[a.param_stride + col];
+        }
       }
     }
+    const bool half_group = HALF != 0 && c4 * 4 + 2 == a.feat_dim;
     const int d = BITS == 4 ? (c4 >> 1) : c4;     // code dword that holds these 4 columns
     const int fsh = BITS == 4 ? (c4 & 1) * 16 : 0;
     const uint32_t* accd = s_acc + ((d & 1) * NW) * lanes + (d >> 1);
@@ -508,14 +533,25 @@ __device__ __forceinline__ void acc_finalize(const AccArgs& a, const FinParams& 
       if (rdeg == 0.f) v0 = v1 = v2 = v3 = 0.f;
       // plain stores: rows are not cache-line multiples in general, and the L2 merges the partial
       // lines that neighbouring waves write before they go to HBM
-      if (a.nt_out) store_nt4(o + (int64_t)r * a.feat_dim, v0, v1, v2, v3);
-      else *reinterpret_cast<float4*>(o + (int64_t)r * a.feat_dim) = make_float4(v0, v1, v2, v3);
+      if constexpr (HALF != 0) {
+        float* dst = o + (int64_t)r * a.feat_dim;
+        if (half_group) {
+          if constexpr (HALF == 2) store_nt2(dst, v0, v1);
+          else *reinterpret_cast<float2*>(dst) = make_float2(v0, v1);
+        } else {
+          if constexpr (HALF == 2) store_nt4_align8(dst, v0, v1, v2, v3);
+          else store4_align8(dst, v0, v1, v2, v3);
+        }
+      } else {
+        if (a.nt_out) store_nt4(o + (int64_t)r * a.feat_dim, v0, v1, v2, v3);
+        else *reinterpret_cast<float4*>(o + (int64_t)r * a.feat_dim) = make_float4(v0, v1, v2, v3);
+      }
     }
   }
 }
 
 // All rows of the block, `sub` rows at a time through the accumulators.
-template <int TB, int BITS, int NW, typename Idx, bool CHUNK = false>
+template <int TB, int BITS, int NW, typename Idx, bool CHUNK = false, int HALF = 0>
 __device__ __forceinline__ void acc_block(const AccArgs& a, const FinParams& first, uint32_t* s_acc, const int* s_ptr,
                                           const float* s_rdeg, uint2* s_edge, int64_t e0, int64_t row0, int nrows,
                                           const Idx* __restrict__ indices, float* __restrict__ out) {
@@ -533,7 +569,7 @@ __device__ __forceinline__ void acc_block(const AccArgs& a, const FinParams& fir
       acc_gather<TB, BITS, NW, CHUNK>(a, s_acc, s_edge, s_ptr[sb], s_ptr[sb + nr], sb, pitch);
       __syncthreads();
       if (sb == 0) ACC_STAMP(a, 3);
-      acc_finalize<TB, BITS, NW>(a, first, s_acc, s_rdeg, row0, sb, nr, pitch, out);
+      acc_finalize<TB, BITS, NW, HALF>(a, first, s_acc, s_rdeg, row0, sb, nr, pitch, out);
       if (sb + sub < nrows) {
         __syncthreads();
         acc_zero<TB>(s_acc, sub * pitch);
@@ -554,12 +590,12 @@ __device__ __forceinline__ void acc_block(const AccArgs& a, const FinParams& fir
         acc_gather<TB, BITS, NW, CHUNK>(a, s_acc, s_edge, 0, nb, 0, pitch);
       }
       __syncthreads();
-      acc_finalize<TB, BITS, NW>(a, first, s_acc, s_rdeg, row0, sb, nr, pitch, out);
+      acc_finalize<TB, BITS, NW, HALF>(a, first, s_acc, s_rdeg, row0, sb, nr, pitch, out);
     }
   }
 }
 
-template <int TB, int BITS, typename Idx, bool CHUNK = false>
+template <int TB, int BITS, typename Idx, bool CHUNK = false, int HALF = 0>
 __global__ __launch_bounds__(TB) void sq_affine_acc_kernel(AccArgs a, const Idx* __restrict__ indptr,
                                                                const Idx* __restrict__ indices,
                                                                float* __restrict__ out) {
@@ -584,7 +620,7 @@ __global__ __launch_bounds__(TB) void sq_affine_acc_kernel(AccArgs a, const Idx*
   const int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block;
 #endif
   const int nrows = (int)((a.R - row0) < row_cap ? (a.R - row0) : row_cap);
-  const FinParams first = acc_fin_params(a);
+  const FinParams first = acc_fin_params<HALF>(a);
   int64_t e0 = (int64_t)indptr[row0];
   e0 = e0 < 0 ? 0 : (e0 > a.E ? a.E : e0);
   uint32_t level = 0;
@@ -618,9 +654,9 @@ __global__ __launch_bounds__(TB) void sq_affine_acc_kernel(AccArgs a, const Idx*
     return;
   }
   if (BITS == 4 && (block_level & 1u))
-    acc_block<TB, BITS, 4, Idx, CHUNK>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
+    acc_block<TB, BITS, 4, Idx, CHUNK, HALF>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
   else
-    acc_block<TB, BITS, 2, Idx, CHUNK>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
+    acc_block<TB, BITS, 2, Idx, CHUNK, HALF>(a, first, s_acc, s_ptr, s_rdeg, s_edge, e0, row0, nrows, indices, out);
   ACC_STAMP(a, 4);
 #ifdef F2CGT_EXPERIMENTS
   if (a.trace && threadIdx.x == 0) {
@@ -805,7 +841,7 @@ int launch_acc_tb(AccArgs a, size_t lds, int64_t grid, const void* indptr, const
     return 0;
   }
 #ifdef F2CGT_EXPERIMENTS
-  if (a.rows_per_block + 1 <= TB && a.edge_batch == 2 * TB && acc_persistent_enabled()) {
+  if (a.rows_per_block + 1 <= TB && a.edge_batch == 2 * TB && a.feat_dim % 4 == 0 && acc_persistent_enabled()) {
     // as many workgroups as the device holds at once (LDS bound), each walking blocks grid apart
     int64_t per_cu = lds > 0 ? (int64_t)(160 * 1024) / (int64_t)lds : 16;
     per_cu = per_cu > 2048 / TB ? 2048 / TB : (per_cu < 1 ? 1 : per_cu);
@@ -825,21 +861,26 @@ int launch_acc_tb(AccArgs a, size_t lds, int64_t grid, const void* indptr, const
 #ifdef F2CGT_EXPERIMENTS
   if (const char* v = getenv("F2CGT_ACC_CHUNK")) chunk = atoi(v) != 0;
 #endif
-  if (idx_dtype == F2CGT_DT_I32) {
-    if (chunk)
-      sq_affine_acc_kernel<TB, BITS, int32_t, true><<<(unsigned)grid, TB, lds, st>>>(
-          a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
-    else
-      sq_affine_acc_kernel<TB, BITS, int32_t><<<(unsigned)grid, TB, lds, st>>>(
-          a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
-  } else {
-    if (chunk)
-      sq_affine_acc_kernel<TB, BITS, int64_t, true><<<(unsigned)grid, TB, lds, st>>>(
-          a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
-    else
-      sq_affine_acc_kernel<TB, BITS, int64_t><<<(unsigned)grid, TB, lds, st>>>(
-          a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
-  }
+  const int half = a.feat_dim % 4 == 0 ? 0 : (a.nt_out ? 2 : 1);   // 4 k + 2 columns: cached or streamed stores
+#define F2CGT_ACC_GO(I, C, H)                                                   \
+  sq_affine_acc_kernel<TB, BITS, I, C, H><<<(unsigned)grid, TB, lds, st>>>(     \
+      a, static_cast<const I*>(indptr), static_cast<const I*>(indices), out)
+#define F2CGT_ACC_HALF(I, C)                                                    \
+  do {                                                                          \
+    if (half == 0) F2CGT_ACC_GO(I, C, 0);                                       \
+    else if (half == 1) F2CGT_ACC_GO(I, C, 1);                                  \
+    else F2CGT_ACC_GO(I, C, 2);                                                 \
+  } while (0)
+#define F2CGT_ACC_IDX(I)                                                        \
+  do {                                                                          \
+    if (chunk) F2CGT_ACC_HALF(I, true);                                         \
+    else F2CGT_ACC_HALF(I, false);                                              \
+  } while (0)
+  if (idx_dtype == F2CGT_DT_I32) F2CGT_ACC_IDX(int32_t);
+  else F2CGT_ACC_IDX(int64_t);
+#undef F2CGT_ACC_IDX
+#undef F2CGT_ACC_HALF
+#undef F2CGT_ACC_GO
   return launch_status(what);
 }
 
@@ -919,7 +960,7 @@ int launch_acc(AccArgs a, const void* indptr, const void* indices, int idx_dtype
     a.pitch_w = 8 * a.lanes + ((8 * a.lanes) % 16 == 0 ? 4 : 0);
   }
 #endif
-  a.f4_per_row = a.feat_dim / 4;
+  a.f4_per_row = (a.feat_dim + 3) / 4;
   const double avg_deg = a.R > 0 ? (double)a.E / (double)a.R : 1.0;
   const double dg = avg_deg > 0.5 ? avg_deg : 0.5;
   // Sized for the narrow layout, the accumulators take the wide one (4-bit codes, a row of more than 17
@@ -972,7 +1013,12 @@ __device__ __forceinline__ float mean_of(float sum, float d, float r) {
   return __fmaf_rn(__fmaf_rn(-q, d, sum), r, q);
 }
 
-template <int BITS, bool AFFINE, typename Idx, int TB>
+// HALF: 0, or 1 / 2 for output rows at any multiple of 8 bytes, possibly with a last group of two columns (rows of
+// 4 k + 2 columns), written with cached / streamed stores (see acc_fin_params).  4- and 8-bit rows always take 1 or 2:
+// with the store form fixed at compile time the row loop came out 3-5 % faster at 100-256 columns and 17-19 % at 600
+// (3e6 edges, 10 per row, 4 bit: 97.8 -> 93.7 us at 128 columns, 592 -> 489 us at 600); 1- and 2-bit rows measured
+// level to 2 % slower and keep the run-time test.
+template <int BITS, bool AFFINE, typename Idx, int TB, int HALF = 0>
 __global__ __launch_bounds__(TB) void sq_rows_kernel(RowsArgs a, const Idx* __restrict__ indptr,
                                                              const Idx* __restrict__ indices,
                                                              float* __restrict__ out) {
@@ -1084,7 +1130,8 @@ __global__ __launch_bounds__(TB) void sq_rows_kernel(RowsArgs a, const Idx* __re
     int lb[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int col = c4 * 4 + i;
+      // a last group of two columns takes the last column's parameters for the two it has not
+      const int col = HALF != 0 && c4 * 4 + i >= a.feat_dim ? a.feat_dim - 1 : c4 * 4 + i;
       if (AFFINE) {
         mn[i] = a.table[col];
         sc[i] = a.table[a.param_stride + col];
@@ -1102,6 +1149,9 @@ __global__ __launch_bounds__(TB) void sq_rows_kernel(RowsArgs a, const Idx* __re
     const unsigned char* sp = s_codes + boff;
     const uint8_t* gp = a.codes + boff;
     float* o = out + (row0 * (int64_t)a.feat_dim + c4 * 4);
+    // Rows of 4 k + 2 columns start at multiples of 8 bytes only and end with a group of two columns: the 16-byte
+    // stores go to any dword, the last group stores its two columns alone and, unstaged, reads only their bytes.
+    const bool half_group = HALF != 0 && c4 * 4 + 2 == a.feat_dim;
     for (int ri = g; ri < nrows; ri += a.fin_slots) {
       const int r = s_order[ri];
       const int b = s_ptr[r], e = s_ptr[r + 1];
@@ -1127,7 +1177,11 @@ __global__ __launch_bounds__(TB) void sq_rows_kernel(RowsArgs a, const Idx* __re
         } else {
           const uint8_t* src = gp + (uint64_t)clamp_idx(indices[e0 + k], a.N) * (uint32_t)a.src_dim;
           const uint8_t* sr1 = gp + (uint64_t)clamp_idx(indices[e0 + k1], a.N) * (uint32_t)a.src_dim;
-          if (BITS == 8) { __builtin_memcpy(&w, src, 4); __builtin_memcpy(&x, sr1, 4); }
+          if (BITS >= 4 && half_group) {
+            if (BITS == 8) { uint16_t h0, h1; __builtin_memcpy(&h0, src, 2); __builtin_memcpy(&h1, sr1, 2); w = h0; x = h1; }
+            else { w = *src; x = *sr1; }
+          }
+          else if (BITS == 8) { __builtin_memcpy(&w, src, 4); __builtin_memcpy(&x, sr1, 4); }
           else if (BITS == 4) { uint16_t h0, h1; __builtin_memcpy(&h0, src, 2); __builtin_memcpy(&h1, sr1, 2); w = h0; x = h1; }
           else { w = *src; x = *sr1; }
         }
@@ -1155,8 +1209,19 @@ __global__ __launch_bounds__(TB) void sq_rows_kernel(RowsArgs a, const Idx* __re
         rc = __fmaf_rn(__fmaf_rn(-d, rc, 1.f), rc, rc);
         s0 = mean_of(s0, d, rc); s1 = mean_of(s1, d, rc); s2 = mean_of(s2, d, rc); s3 = mean_of(s3, d, rc);
       }
-      if (a.nt_out) store_nt4(o + (int64_t)r * a.feat_dim, s0, s1, s2, s3);
-      else *reinterpret_cast<float4*>(o + (int64_t)r * a.feat_dim) = make_float4(s0, s1, s2, s3);
+      if constexpr (HALF != 0) {
+        float* dst = o + (int64_t)r * a.feat_dim;
+        if (half_group) {
+          if constexpr (HALF == 2) store_nt2(dst, s0, s1);
+          else *reinterpret_cast<float2*>(dst) = make_float2(s0, s1);
+        } else {
+          if constexpr (HALF == 2) store_nt4_align8(dst, s0, s1, s2, s3);
+          else store4_align8(dst, s0, s1, s2, s3);
+        }
+      } else {
+        if (a.nt_out) store_nt4(o + (int64_t)r * a.feat_dim, s0, s1, s2, s3);
+        else *reinterpret_cast<float4*>(o + (int64_t)r * a.feat_dim) = make_float4(s0, s1, s2, s3);
+      }
     }
   }
 }
@@ -1175,7 +1240,7 @@ int launch_sq_rows(RowsArgs a, const void* indptr, const void* indices, int idx_
   const int lanes2 = pow2_ceil(a.lanes);
   a.lane_shift = 0;
   while ((1 << a.lane_shift) < lanes2) ++a.lane_shift;
-  a.f4_per_row = a.feat_dim / 4;
+  a.f4_per_row = (a.feat_dim + 3) / 4;
   a.fin_group = a.f4_per_row < TB ? a.f4_per_row : TB;
   a.fin_slots = TB / a.fin_group;
   a.fin_magic = (uint32_t)((65536 + a.fin_group - 1) / a.fin_group);
@@ -1227,12 +1292,22 @@ int launch_sq_rows(RowsArgs a, const void* indptr, const void* indices, int idx_
                 a.edge_cap);
     return 0;
   }
-  if (idx_dtype == F2CGT_DT_I32)
-    sq_rows_kernel<BITS, AFFINE, int32_t, TB><<<(unsigned)grid, TB, lds, st>>>(
-        a, static_cast<const int32_t*>(indptr), static_cast<const int32_t*>(indices), out);
-  else
-    sq_rows_kernel<BITS, AFFINE, int64_t, TB><<<(unsigned)grid, TB, lds, st>>>(
-        a, static_cast<const int64_t*>(indptr), static_cast<const int64_t*>(indices), out);
+  const int half = (a.feat_dim % 4 == 0 && BITS < 4) ? 0 : (a.nt_out ? 2 : 1);
+#define F2CGT_ROWS_GO(I, H)                                                      \
+  sq_rows_kernel<BITS, AFFINE, I, TB, H><<<(unsigned)grid, TB, lds, st>>>(       \
+      a, static_cast<const I*>(indptr), static_cast<const I*>(indices), out)
+#define F2CGT_ROWS_IDX(I)                                                        \
+  do {                                                                           \
+    if constexpr (BITS < 4) {                                                    \
+      if (half == 0) F2CGT_ROWS_GO(I, 0);                                        \
+    }                                                                            \
+    if (half == 1) F2CGT_ROWS_GO(I, 1);                                          \
+    else if (half == 2) F2CGT_ROWS_GO(I, 2);                                     \
+  } while (0)
+  if (idx_dtype == F2CGT_DT_I32) F2CGT_ROWS_IDX(int32_t);
+  else F2CGT_ROWS_IDX(int64_t);
+#undef F2CGT_ROWS_IDX
+#undef F2CGT_ROWS_GO
   return launch_status(what);
 }
 
@@ -1628,7 +1703,7 @@ static bool sq_rows_pitch_ok(int feat_dim, int target_bits) {
 
 bool sq_block_eligible(const void* codes, const float* out, int64_t N, int64_t src_dim, int feat_dim,
                        int target_bits, int64_t lut_entries) {
-  if ((target_bits == 1 || target_bits == 2 || target_bits == 4 || target_bits == 8) && feat_dim % 4 == 0 &&
+  if ((target_bits == 1 || target_bits == 2 || target_bits == 4 || target_bits == 8) && feat_dim % 2 == 0 &&
       (int64_t)feat_dim * target_bits >= 64 &&
       src_dim >= 8 && feat_dim <= 4096 && sq_rows_pitch_ok(feat_dim, target_bits) && aligned(out, 16) &&
       N < (1ll << 32) && src_dim < (1ll << 24) && src_dim * (8 / target_bits) >= feat_dim &&
@@ -1657,7 +1732,7 @@ int sq_block_run(bool affine, const uint8_t* codes, const float* table, int64_t 
                  int target_bits, hipStream_t st, const char* what) {
   // the 128-thread staged-rows kernel (degree-ordered rows) covers every shape with float4 column
   // groups; the 256-thread block kernel below stays for the remaining ones
-  if (feat_dim % 4 == 0 && (int64_t)feat_dim * target_bits >= 64 && src_dim >= 8 && feat_dim <= 4096 &&
+  if (feat_dim % 2 == 0 && (int64_t)feat_dim * target_bits >= 64 && src_dim >= 8 && feat_dim <= 4096 &&
       sq_rows_pitch_ok(feat_dim, target_bits)) {
     RowsArgs r{};
     r.codes = codes; r.table = table; r.param_stride = param_stride; r.column_slice = column_slice;
@@ -1698,7 +1773,7 @@ bool sq_affine_acc_eligible(const void* codes, const float* out, int64_t N, int6
                             int target_bits) {
   if (target_bits != 4 && target_bits != 8) return false;
   if (codes == nullptr || !aligned(out, 16)) return false;
-  if (feat_dim % 4 != 0 || feat_dim > 4096) return false;
+  if (feat_dim % 2 != 0 || feat_dim > 4096) return false;
   if (feat_dim * target_bits < 64) return false;  // a gather lane loads 8 bytes of the row
   if (src_dim < 8 || src_dim >= (1ll << 20) || src_dim * (8 / target_bits) < feat_dim) return false;
   if (N < 1 || N >= (1ll << 32)) return false;

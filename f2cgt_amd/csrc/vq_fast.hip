@@ -301,7 +301,16 @@ __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlan
 // bytes).  The BT bytes a lane fetches for its tile then start at any byte of the table, reach into the next row
 // (bytes the tile has no columns for) and, for the table's last row or two, past its end: those rows are fetched
 // byte by byte.
-template <int BT, int H, int RPM, typename Idx, bool DENSE = false, bool TRACE = false, bool TAIL = false>
+// EVEN2 (H == 1): feat_dim is even but no multiple of 4 (602 columns).  Output rows then start at multiples of 8
+// bytes only and the last column group of the last tile has two columns.  A lane still stores its four values with
+// one 16-byte store (global memory takes it at any dword); the lane of the two-column group fetches the previous
+// group's last two sums from that group's lane and stores the 16 bytes that end with its own two, so that every lane
+// issues the same single store (1191 us with one column per lane, 507 us with two 8-byte stores per lane; 602
+// columns, 3e6 edges, 10 per row).  A tile of two columns in all (130 = 128 + 2) stores those alone.  The codebooks
+// hold the columns up to the next multiple of 4, since n_cb * w >= feat_dim is a multiple of 8, so the sums are
+// formed as for a full group.
+template <int BT, int H, int RPM, typename Idx, bool DENSE = false, bool TRACE = false, bool TAIL = false,
+          bool EVEN2 = false>
 __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* __restrict__ indptr,
                                                            const Idx* __restrict__ indices,
                                                            float* __restrict__ out) {
@@ -329,7 +338,8 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
     tile = blockIdx.x % a.n_tiles;
     stripe = blockIdx.x / a.n_tiles;
   }
-  const int tile_cols = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
+  const int tile_cols_out = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
+  const int tile_cols = EVEN2 ? (tile_cols_out + 3) & ~3 : tile_cols_out;   // columns staged and summed
 
   // A workgroup owns one contiguous range of rows, cut into chunks of 12 rows.  The waves deal the
   // chunks among themselves through a counter in LDS: wave w starts with chunk w and takes the next
@@ -377,6 +387,7 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   const int col0 = c4 * 4 * H;                 // first column of the lane inside the tile
   const int byte_idx = col0 / a.w;
   const float* cbp = s_cb + c4 * 4;
+  const int prev_group_lane = (lane & ~(kLanesPerRow - 1)) + (c4 > 0 ? c4 - 1 : 0);   // EVEN2
   const uint8_t* code_base = a.codes + tile * BT;
   const uint32_t n_last = (uint32_t)(a.N - 1);
   // the last source row whose BT bytes for this tile lie inside the table (TAIL only)
@@ -772,8 +783,21 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
           // so that they are issued back to back (see above)
           const uint32_t off_b = (uint32_t)row * ((uint32_t)a.feat_dim * 4u) + 4u * (uint32_t)col0;
           float* dst = reinterpret_cast<float*>(obase + off_b);
+          if constexpr (EVEN2) {
+            if (tile_cols_out < 4) {          // a tile of two columns: nothing to pair them with
+              store_nt2(dst, acc[0][0], acc[0][1]);
+            } else if (tile_cols_out & 2) {   // the tile ends with a group of two columns
+              const bool half_group = col0 + 2 >= tile_cols_out;
+              const float p2 = __shfl(acc[0][2], prev_group_lane), p3 = __shfl(acc[0][3], prev_group_lane);
+              store_nt4_align8(half_group ? dst - 2 : dst, half_group ? p2 : acc[0][0], half_group ? p3 : acc[0][1],
+                               half_group ? acc[0][0] : acc[0][2], half_group ? acc[0][1] : acc[0][3]);
+            } else {
+              store_nt4_align8(dst, acc[0][0], acc[0][1], acc[0][2], acc[0][3]);
+            }
+          } else {
 #pragma unroll
-          for (int h = 0; h < H; ++h) store_nt4(dst + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+            for (int h = 0; h < H; ++h) store_nt4(dst + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+          }
         }
       }
     }
@@ -1177,6 +1201,22 @@ int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int id
   const bool tail = a.n_cb % BT != 0 || !aligned(a.codes, BT);
   const bool dense = CAN_DENSE && a.dense_store == 1 && !tail;
   const void* kern;
+  if constexpr (H == 1 && RPM == 4) {
+    if (a.feat_dim % 4 != 0) {   // even widths that are no multiple of 4
+      kern = tail ? (idx_dtype == F2CGT_DT_I32
+                         ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false, false, true, true>)
+                         : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t, false, false, true, true>))
+                  : (idx_dtype == F2CGT_DT_I32
+                         ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false, false, false, true>)
+                         : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t, false, false, false, true>));
+      const hipError_t e2 = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
+      if (e2 != hipSuccess) return fail((int)e2, "%s: cannot reserve %zu B of LDS", what, wlds);
+      void* params2[] = {const_cast<VqArgs*>(&a), &indptr, &indices, &out};
+      const hipError_t le2 = hipLaunchKernel(kern, dim3(grid), dim3(kThreads), params2, wlds, st);
+      if (le2 != hipSuccess) return fail((int)le2, "%s: launch failed: %s", what, hipGetErrorString(le2));
+      return launch_status(what);
+    }
+  }
   if (tail)
     kern = idx_dtype == F2CGT_DT_I32
                ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false, false, true>)
@@ -1230,7 +1270,7 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     const char* v = getenv("F2CGT_VQ_STRIP");
     const int mode = v ? atoi(v) : 0;     // 0 off; tens: 0 plain, 1 non-temporal, 2 no stores; units: 2 = KE by degree, 6 = KE 16
     if (mode == 20) a.dense_store = 2;
-    if (mode % 10 > 0 && avg_deg <= 24.0 && a.n_cb % BT == 0 && aligned(a.codes, BT)) {
+    if (mode % 10 > 0 && avg_deg <= 24.0 && a.n_cb % BT == 0 && aligned(a.codes, BT) && a.feat_dim % 4 == 0) {
       VqArgs b = a;
       b.dense_store = (mode / 10) % 10;
       if (mode >= 100) b.N = 1;   // experiment: every source id reads row 0
@@ -1270,7 +1310,7 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     if (avg_deg <= 16.0 * fit) return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
     if (avg_deg <= 32.0 * fit) return launch_wave<BT, 2, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
     return launch_wave<BT, 2, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
-  } else if (avg_deg <= 15.0 || a.n_cb % BT != 0 || !aligned(a.codes, BT)) {
+  } else if (avg_deg <= 15.0 || a.n_cb % BT != 0 || !aligned(a.codes, BT) || a.feat_dim % 4 != 0) {
     // (the block-synchronous kernel below reads whole aligned code words; longer rows go through the staging in slices)
     return launch_wave<BT, 1, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
   }
@@ -1302,7 +1342,7 @@ bool vq_pipe_eligible(const void* codes, const float* codebooks, const float* ou
   if (E < 1 || N < 1 || codes == nullptr) return false;  // idle lanes read row 0 / indptr[0]
   if (K < 1 || K > 256) return false;
   if (w != 8 && w != 16 && w != 32) return false;
-  if (feat_dim < 16 || feat_dim % 4 != 0 || feat_dim > n_cb * w) return false;
+  if (feat_dim < 16 || feat_dim % 2 != 0 || feat_dim > n_cb * w) return false;
   if (!aligned(out, 16) || !aligned(codebooks, 4)) return false;
   if (N >= (1ll << 32)) return false;
   if (R < 4 * kRows) return false;  // tiny problems: the per-row skeleton has less start-up cost

@@ -73,6 +73,45 @@ def test_fused_log_sq_with_either_workgroup_size(bits, feat_dim):
         assert np.allclose(got.cpu().numpy(), want, rtol=RTOL, atol=RTOL * 3.0)
 
 
+@pytest.mark.parametrize("idx", [np.int64, np.int32])
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("feat_dim", [602, 102, 66, 18])
+def test_fused_sq_rows_of_an_even_number_of_columns_that_is_no_multiple_of_four(feat_dim, bits, idx):
+    """602, 102 ... columns: output rows start at multiples of 8 bytes only and end with a group of two columns, code
+    rows may end inside a byte group.  Affine and log-domain forms, staged and unstaged blocks (rows of 2, 12, 40 and
+    300 edges on average), plain and streamed stores; many edges name the table's last row."""
+    rng = np.random.default_rng(13 * feat_dim + bits + (idx == np.int32))
+    n = 3000
+    per = 8 // bits
+    src_dim = (feat_dim + per - 1) // per
+    codes = rng.integers(0, 256, size=(n, src_dim), dtype=np.uint8)
+    if feat_dim % per:                                   # bits of a row's last byte beyond its columns stay 0
+        codes[:, -1] &= (1 << (bits * (feat_dim % per))) - 1
+    params = np.stack([rng.standard_normal(feat_dim) - 3, 0.01 + 0.02 * rng.random(feat_dim)]).astype(np.float32)
+    cb = np.array([[0.01, 3.0, -6.643856, 1.5849625, 0.4]], dtype=np.float32)
+    column_slice = src_dim * per
+    stored = codes.view(np.int8) if bits == 8 else codes
+    for fanout, ragged in ((2, True), (12, False), (40, True), (300, True)):
+        indptr, indices = fixed_fanout(rng, 400, n, fanout, ragged)
+        indices[::5] = n - 1
+        ip, ix = dev(indptr.astype(idx)), dev(indices.astype(idx))
+        dec_a = oc.sq_affine_decompress(codes, params, bits, feat_dim).astype(np.float64)
+        exact_a = oc.spmm_csr(dec_a, indptr, indices)
+        want_a = oc.sq_affine_decompress_spmm_csr(codes, params, indptr, indices, bits, feat_dim)
+        want_l = oc.sq_decompress_spmm_csr(stored, cb, indptr, indices, bits, column_slice, feat_dim)
+        for mode in (capi.STORE_CACHED, capi.STORE_STREAM):
+            was = capi.set_store_mode(mode)
+            try:
+                got_a = capi.sq_affine_decompress_spmm_csr(dev(codes), dev(params), ip, ix, bits, feat_dim)
+                got_l = capi.sq_decompress_spmm_csr(dev(stored), dev(cb), ip, ix, bits, column_slice, feat_dim)
+                torch.cuda.synchronize()
+            finally:
+                capi.set_store_mode(was)
+            assert_mean_aggregate(got_a.cpu().numpy(), want_a, exact_a, float(np.abs(dec_a).max()))
+            err = np.abs(got_l.cpu().numpy() - want_l).max()
+            assert err <= RTOL * 3.0, (fanout, mode, float(err))
+
+
 @pytest.mark.parametrize("rows", [16383, 16384, 32767, 32768, 65535, 65536, 114687, 114688])
 def test_fused_sq_on_both_sides_of_the_rows_per_block_steps(rows):
     # launches below ~2000 workgroups shrink their row blocks in steps of 8 rows: the integer-accumulating
@@ -133,12 +172,15 @@ def test_fused_vq_chunk_dealing_with_shared_rows(mean_deg):
 @pytest.mark.parametrize("idx", [np.int64, np.int32])
 @pytest.mark.parametrize("feat_dim,n_cb,width", [(100, 13, 8), (64, 8, 8), (96, 12, 8), (192, 24, 8), (160, 5, 32),
                                                  (96, 3, 32), (48, 3, 16), (200, 13, 16), (100, 4, 32), (600, 19, 32),
-                                                 (120, 16, 8)])
+                                                 (120, 16, 8), (602, 19, 32), (102, 13, 8), (50, 7, 8), (90, 3, 32),
+                                                 (30, 4, 8), (130, 17, 8), (258, 17, 16)])
 @pytest.mark.parametrize("mean_deg", [3, 12, 40])
 def test_fused_vq_code_rows_that_are_no_multiple_of_a_tile(feat_dim, n_cb, width, mean_deg, idx):
     """Code rows of 13, 8, 12, 24 ... bytes where a 128-column tile takes 16 (8, 4) of them: the pipelined kernel
     fetches its code words at any alignment and reads the table's last rows byte by byte.  Many edges name the last two
-    source rows; feat_dim may be less than n_cb * width (the reference's truncation)."""
+    source rows; feat_dim may be less than n_cb * width (the reference's truncation).  Output rows of an even number
+    of columns that is no multiple of four (602, 102, 50 ...) are only 8-byte aligned: they are written in 8-byte
+    pairs, the last pair of a row possibly alone in its group of four."""
     rng = np.random.default_rng(feat_dim * 100 + mean_deg + (idx == np.int32))
     n_src, rows = 777, 3000
     codes = rng.integers(0, 256, size=(n_src, n_cb), dtype=np.uint8)

@@ -287,7 +287,7 @@ def test_sq_affine_decompress_padded_storage(bits):
 
 # ---- plain CSC mean ---------------------------------------------------------------------------
 @pytest.mark.parametrize("idx", [np.int32, np.int64])
-@pytest.mark.parametrize("d", [1, 7, 100, 128, 300])
+@pytest.mark.parametrize("d", [1, 7, 100, 128, 300, 2, 6, 102, 602])
 def test_spmm_csr_f32(idx, d):
     rng = np.random.default_rng(d)
     feat = rng.standard_normal((1000, d)).astype(np.float32)
@@ -295,6 +295,11 @@ def test_spmm_csr_f32(idx, d):
     got = host(capi.spmm_csr(dev(feat), dev(indptr), dev(indices)))
     want = oc.spmm_csr(feat, indptr, indices)
     assert np.array_equal(got, want)  # sequential edge order is kept
+    # a feature matrix that starts 4 bytes off an 8-byte boundary takes the one-column-per-lane form
+    flat = torch.zeros(feat.size + 1, dtype=torch.float32, device="cuda")
+    flat[1:] = dev(feat).reshape(-1)
+    got = host(capi.spmm_csr(flat[1:].view(1000, d), dev(indptr), dev(indices)))
+    assert np.array_equal(got, want)
 
 
 def test_spmm_csr_f16_f64_and_empty():
