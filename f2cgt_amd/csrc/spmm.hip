@@ -31,9 +31,19 @@ template <> struct packed_word<2> { using type = uint16_t; };
 template <> struct packed_word<4> { using type = uint32_t; };
 
 // ---- output store ----------------------------------------------------------------
-template <int NOUT, typename Acc, typename Out>
+// A decoder that declares kAlign8 writes rows that start at multiples of 8 bytes only (4 k + 2 columns).
+template <class Dec, class = void> struct dec_align8 : std::false_type {};
+template <class Dec> struct dec_align8<Dec, std::void_t<decltype(Dec::kAlign8)>> : std::bool_constant<Dec::kAlign8> {};
+
+template <int NOUT, typename Acc, typename Out, bool A8 = false>
 __device__ __forceinline__ void store_mean(Out* __restrict__ o, const Acc (&acc)[NOUT], Acc deg,
                                            int nvalid, bool vec_ok) {
+  if constexpr (A8) {
+    static_assert(NOUT == 4 && std::is_same<Out, float>::value, "four fp32 columns per lane");
+    if (nvalid >= 4) store_nt4_align8(o, acc[0] / deg, acc[1] / deg, acc[2] / deg, acc[3] / deg);
+    else store_nt2(o, acc[0] / deg, acc[1] / deg);   // the row's last two columns
+    return;
+  }
   if constexpr (std::is_same<Out, float>::value) {
     if (vec_ok && nvalid >= NOUT) {
       if constexpr (NOUT == 2) {
@@ -99,13 +109,48 @@ __global__ __launch_bounds__(kMaxBlock) void agg_kernel(Dec dec, const Idx* __re
         for (int u = 0; u < kUnroll; ++u)
           if (s[u] >= 0) dec.accum(ctx, raw[u], acc);
       }
-      store_mean<NOUT, Acc, typename Dec::Out>(out + r * (int64_t)feat_dim + col0, acc, deg, nvalid,
-                                               vec_ok);
+      store_mean<NOUT, Acc, typename Dec::Out, dec_align8<Dec>::value>(out + r * (int64_t)feat_dim + col0, acc, deg,
+                                                                       nvalid, vec_ok);
     }
   }
 }
 
 // ---- decoders ---------------------------------------------------------------------
+
+// Uncompressed fp32 features of 4 k + 2 columns (602): rows start at multiples of 8 bytes only.  A lane still owns
+// four columns and moves them with one 16-byte access, which global memory takes at any dword; the lane of the row's
+// last two columns moves those alone (2e6 edges at 10 per row, 602 columns: 1703 us with one column per lane, 961 us
+// with two, 679 us so; 620 us at 600 columns).
+struct PlainPairsDec {
+  static constexpr int NOUT = 4;
+  static constexpr bool kAlign8 = true;
+  using Acc = float;
+  using Out = float;
+  struct Ctx { int col0; bool whole; };
+  struct Raw { float v[4]; };
+  const float* __restrict__ feat;
+  int64_t D;
+  __device__ void block_setup(unsigned char*, int, int) {}
+  __device__ Ctx column_setup(int col0) const { return Ctx{col0, col0 + 4 <= D}; }
+  __device__ Raw load(const Ctx& c, int64_t s) const {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    typedef f4 f4a8 __attribute__((aligned(8)));
+    Raw r;
+    const float* p = feat + s * D + c.col0;
+    if (c.whole) {
+      const f4 q = *reinterpret_cast<const f4a8*>(p);
+      r.v[0] = q.x; r.v[1] = q.y; r.v[2] = q.z; r.v[3] = q.w;
+    } else {
+      const float2 q = *reinterpret_cast<const float2*>(p);
+      r.v[0] = q.x; r.v[1] = q.y; r.v[2] = 0.f; r.v[3] = 0.f;
+    }
+    return r;
+  }
+  __device__ void accum(const Ctx&, const Raw& r, float (&acc)[4]) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] += r.v[i];
+  }
+};
 
 // Uncompressed features (spmm_csr).
 template <typename T, int NOUT_>
@@ -624,7 +669,12 @@ extern "C" int f2cgt_spmm_csr(const void* feat, int feat_dtype, void* out, const
         return run(d, indptr, indices, idx_dtype, static_cast<float*>(out), num_rows, num_edges,
                    num_src_rows, D, plan(num_rows, D, 1, 4, 0), 0, true, st, what);
       }
-      if (D % 2 == 0 && aligned(feat, 8) && aligned(out, 8)) {   // rows of 8-byte pairs (602 columns: 961 us against 1703 with single floats)
+      if (D % 2 == 0 && D >= 6 && aligned(feat, 8) && aligned(out, 8)) {   // rows of 4 k + 2 columns
+        PlainPairsDec d{static_cast<const float*>(feat), feat_dim};
+        return run(d, indptr, indices, idx_dtype, static_cast<float*>(out), num_rows, num_edges,
+                   num_src_rows, D, plan(num_rows, D, 1, 4, 0), 0, true, st, what);
+      }
+      if (D % 2 == 0 && aligned(feat, 8) && aligned(out, 8)) {   // two columns
         PlainDec<float, 2> d{static_cast<const float*>(feat), feat_dim};
         return run(d, indptr, indices, idx_dtype, static_cast<float*>(out), num_rows, num_edges,
                    num_src_rows, D, plan(num_rows, D, 1, 2, 0), 0, true, st, what);

@@ -223,9 +223,13 @@ struct F4Args {
   int64_t total_f4;
   uint32_t f4_per_row;
   uint32_t magic;         // ceil(2^32 / f4_per_row)
+  int feat_dim;           // HALF decoders: columns of a row, 4 * f4_per_row - 2
 };
 
-template <int BITS, bool AFFINE>
+// HALF: rows of 4 k + 2 columns.  A lane still owns a group of four columns of a row; output rows start at multiples
+// of 8 bytes only, which a 16-byte store takes at any dword, and the row's last group holds two columns: it loads only
+// their code bytes and stores them alone (the tables in LDS repeat the last column for the two it has not).
+template <int BITS, bool AFFINE, bool HALF = false>
 __global__ __launch_bounds__(kBlock) void sq_decode_f4_kernel(F4Args a) {
   constexpr int NCODE = 1 << BITS;
   constexpr uint32_t MASK = NCODE - 1;
@@ -235,14 +239,15 @@ __global__ __launch_bounds__(kBlock) void sq_decode_f4_kernel(F4Args a) {
   int* s_cbi = reinterpret_cast<int*>(s_tab + ((a.n_cb * NCODE + 3) & ~3));
   if (AFFINE) {
     for (int i = threadIdx.x; i < feat_dim; i += kBlock) {
-      s_tab[(i >> 2) * 8 + (i & 3)] = a.table[i];
-      s_tab[(i >> 2) * 8 + 4 + (i & 3)] = a.table[a.param_stride + i];
+      const int col = HALF && i >= a.feat_dim ? a.feat_dim - 1 : i;
+      s_tab[(i >> 2) * 8 + (i & 3)] = a.table[col];
+      s_tab[(i >> 2) * 8 + 4 + (i & 3)] = a.table[a.param_stride + col];
     }
   } else {
     for (int i = threadIdx.x; i < a.n_cb * NCODE; i += kBlock)
       s_tab[i] = sq_log_value<BITS>((uint32_t)(i & MASK), a.table + (int64_t)(i >> BITS) * 5);
     for (int i = threadIdx.x; i < feat_dim; i += kBlock) {
-      int64_t cb = i / a.column_slice;
+      int64_t cb = (HALF && i >= a.feat_dim ? a.feat_dim - 1 : i) / a.column_slice;
       cb = cb < a.n_cb ? cb : a.n_cb - 1;
       s_cbi[i] = (int)cb * NCODE;
     }
@@ -256,7 +261,7 @@ __global__ __launch_bounds__(kBlock) void sq_decode_f4_kernel(F4Args a) {
   if ((rb + 1) * (int64_t)a.f4_per_row <= base) ++rb;
   const uint32_t cb0 = (uint32_t)(base - rb * a.f4_per_row);
 
-  uint32_t word[kF4Items], c4s[kF4Items];
+  uint32_t word[kF4Items], c4s[kF4Items], rls[kF4Items];
 #pragma unroll
   for (int k = 0; k < kF4Items; ++k) {
     const uint32_t li = cb0 + threadIdx.x + k * kBlock;
@@ -265,7 +270,11 @@ __global__ __launch_bounds__(kBlock) void sq_decode_f4_kernel(F4Args a) {
     const bool on = base + threadIdx.x + k * kBlock < a.total_f4;
     const uint8_t* src = a.codes + (on ? (rb + rl) * a.src_dim : 0);
     c4s[k] = c4;
-    if (BITS == 8) {
+    rls[k] = rl;
+    if (HALF && BITS >= 4 && on && c4 + 1 == a.f4_per_row) {   // the row's last two columns
+      if (BITS == 8) { uint16_t w; __builtin_memcpy(&w, src + 4 * c4, 2); word[k] = w; }
+      else word[k] = src[2 * c4];
+    } else if (BITS == 8) {
       uint32_t w; __builtin_memcpy(&w, src + (on ? 4 * c4 : 0), 4); word[k] = w;
     } else if (BITS == 4) {
       uint16_t w; __builtin_memcpy(&w, src + (on ? 2 * c4 : 0), 2); word[k] = w;
@@ -295,7 +304,13 @@ __global__ __launch_bounds__(kBlock) void sq_decode_f4_kernel(F4Args a) {
       v[2] = s_tab[cbi.z + ((word[k] >> (2 * BITS)) & MASK)];
       v[3] = s_tab[cbi.w + ((word[k] >> (3 * BITS)) & MASK)];
     }
-    store_nt4(a.out + i * 4, v[0], v[1], v[2], v[3]);
+    if constexpr (HALF) {
+      float* dst = a.out + ((rb + rls[k]) * (int64_t)a.feat_dim + 4 * c4);
+      if (c4 + 1 == a.f4_per_row) store_nt2(dst, v[0], v[1]);
+      else store_nt4_align8(dst, v[0], v[1], v[2], v[3]);
+    } else {
+      store_nt4(a.out + i * 4, v[0], v[1], v[2], v[3]);
+    }
   }
 }
 
@@ -305,20 +320,23 @@ int decode_f4_launch(const uint8_t* codes, float* out, const float* table, int64
                      int64_t column_slice, int n_cb, int64_t rows, int64_t src_dim, int64_t feat_dim,
                      hipStream_t st, const char* what) {
   // (one float4 per row would need the reciprocal 2^32, which does not fit the 32-bit multiplier)
-  if (feat_dim % 4 != 0 || feat_dim < 8 || feat_dim > 8192 || !aligned(out, 16)) return -1;
-  const size_t lds = AFFINE ? (size_t)feat_dim * 8
-                            : ((((size_t)n_cb << BITS) + 3) / 4 * 4 + (size_t)feat_dim) * 4;
+  if (feat_dim % 2 != 0 || feat_dim < 8 || feat_dim > 8192 || !aligned(out, 16)) return -1;
+  const int64_t padded = (feat_dim + 3) / 4 * 4;   // rows of 4 k + 2 columns: tables for the group of two as for four
+  const size_t lds = AFFINE ? (size_t)padded * 8
+                            : ((((size_t)n_cb << BITS) + 3) / 4 * 4 + (size_t)padded) * 4;
   if (lds > (size_t)kMaxLutBytes) return -1;
   F4Args a{};
   a.codes = codes; a.out = out; a.table = table;
   a.param_stride = param_stride; a.column_slice = column_slice; a.n_cb = AFFINE ? 0 : n_cb;
   a.src_dim = src_dim;
-  a.f4_per_row = (uint32_t)(feat_dim / 4);
-  a.total_f4 = rows * (feat_dim / 4);
+  a.feat_dim = (int)feat_dim;
+  a.f4_per_row = (uint32_t)(padded / 4);
+  a.total_f4 = rows * (padded / 4);
   a.magic = (uint32_t)((0x100000000ull + a.f4_per_row - 1) / a.f4_per_row);
   const int64_t grid = ceil_div(a.total_f4, kF4Items * kBlock);
   if (grid > 0x7fffffffll) return -1;
-  sq_decode_f4_kernel<BITS, AFFINE><<<(unsigned)grid, kBlock, lds, st>>>(a);
+  if (feat_dim % 4 == 0) sq_decode_f4_kernel<BITS, AFFINE><<<(unsigned)grid, kBlock, lds, st>>>(a);
+  else sq_decode_f4_kernel<BITS, AFFINE, true><<<(unsigned)grid, kBlock, lds, st>>>(a);
   return launch_status(what);
 }
 

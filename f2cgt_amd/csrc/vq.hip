@@ -68,11 +68,16 @@ struct VqTileArgs {
   int n_tiles, n_stripes;
 };
 
+// HALF: rows of 4 k + 2 columns.  Output rows start at multiples of 8 bytes only, which a 16-byte store takes at any
+// dword; the row's last column group holds two columns and stores them alone (the tile is staged up to the next
+// multiple of four: the codebooks hold those columns, n_cb * w being a multiple of four that is at least feat_dim).
+template <bool HALF>
 __global__ __launch_bounds__(kTileThreads) void vq_decompress_tile_kernel(VqTileArgs a) {
   extern __shared__ __align__(16) float s_cb[];
   const int tile = blockIdx.x % a.n_tiles;
   const int stripe = blockIdx.x / a.n_tiles;
-  const int tile_cols = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
+  const int tile_cols_out = (a.feat_dim - tile * 128) >= 128 ? 128 : (a.feat_dim - tile * 128);
+  const int tile_cols = HALF ? (tile_cols_out + 3) & ~3 : tile_cols_out;
   stage_codebook_tile<kTileThreads, false>(s_cb, a.codebooks, a.K, a.w, tile, tile_cols);
   __syncthreads();
   const int c4 = threadIdx.x & 31;
@@ -82,6 +87,15 @@ __global__ __launch_bounds__(kTileThreads) void vq_decompress_tile_kernel(VqTile
   const uint8_t* cp = a.codes + col0 / a.w;
   const float* cbp = s_cb + c4 * 4;
   float* op = a.out + col0;
+  const bool pair = HALF && c4 * 4 + 2 == tile_cols_out;   // the row's last two columns
+  auto store = [&](float* dst, const float4& x) {
+    if constexpr (HALF) {
+      if (pair) store_nt2(dst, x.x, x.y);
+      else store_nt4_align8(dst, x.x, x.y, x.z, x.w);
+    } else {
+      store_nt4(dst, x.x, x.y, x.z, x.w);
+    }
+  };
   const int64_t steps = a.rows / kTileRows;   // full steps
   const uint32_t kmax = (uint32_t)a.K - 1u;
 
@@ -104,7 +118,7 @@ __global__ __launch_bounds__(kTileThreads) void vq_decompress_tile_kernel(VqTile
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u)
-      store_nt4(op + (s * kTileRows + rs + 32 * u) * (int64_t)a.feat_dim, x[u].x, x[u].y, x[u].z, x[u].w);
+      store(op + (s * kTileRows + rs + 32 * u) * (int64_t)a.feat_dim, x[u]);
 #pragma unroll
     for (int u = 0; u < 8; ++u) code[u] = next[u];
   }
@@ -114,7 +128,7 @@ __global__ __launch_bounds__(kTileThreads) void vq_decompress_tile_kernel(VqTile
       uint32_t c = cp[r * a.n_cb];
       c = c < kmax ? c : kmax;
       const float4 x = *reinterpret_cast<const float4*>(cbp + c * 128);
-      store_nt4(op + r * (int64_t)a.feat_dim, x.x, x.y, x.z, x.w);
+      store(op + r * (int64_t)a.feat_dim, x);
     }
   }
 }
@@ -122,7 +136,7 @@ __global__ __launch_bounds__(kTileThreads) void vq_decompress_tile_kernel(VqTile
 // Returns -1 when the shape is not covered.
 int launch_tile(const uint8_t* codes, const float* codebooks, float* out, int64_t rows, int64_t feat_dim,
                 int n_cb, int K, int w, hipStream_t st) {
-  if (K > 256 || w < 4 || 128 % w != 0 || feat_dim % 4 != 0 || feat_dim < 64) return -1;
+  if (K > 256 || w < 4 || 128 % w != 0 || feat_dim % 2 != 0 || feat_dim < 64) return -1;
   if (!aligned(out, 16) || rows < 4 * kTileRows) return -1;
   VqTileArgs a{codes, codebooks, out, rows, (int)feat_dim, n_cb, K, w, 0, 0};
   a.n_tiles = (int)ceil_div(feat_dim, 128);
@@ -130,10 +144,13 @@ int launch_tile(const uint8_t* codes, const float* codebooks, float* out, int64_
   if (a.n_tiles > cus) return -1;
   a.n_stripes = cus / a.n_tiles;
   const size_t lds = (size_t)K * 128 * 4;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(vq_decompress_tile_kernel),
+  const bool half = feat_dim % 4 != 0;
+  hipError_t e = hipFuncSetAttribute(half ? reinterpret_cast<const void*>(vq_decompress_tile_kernel<true>)
+                                          : reinterpret_cast<const void*>(vq_decompress_tile_kernel<false>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return fail((int)e, "vq_decompress: cannot reserve %zu B of LDS", lds);
-  vq_decompress_tile_kernel<<<(unsigned)(a.n_stripes * a.n_tiles), kTileThreads, lds, st>>>(a);
+  if (half) vq_decompress_tile_kernel<true><<<(unsigned)(a.n_stripes * a.n_tiles), kTileThreads, lds, st>>>(a);
+  else vq_decompress_tile_kernel<false><<<(unsigned)(a.n_stripes * a.n_tiles), kTileThreads, lds, st>>>(a);
   return launch_status("vq_decompress");
 }
 

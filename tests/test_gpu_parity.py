@@ -197,6 +197,20 @@ def test_sq_decompress_every_code(bits):
     assert np.array_equal(want[0, :n], oc.sq_lut(cbs, bits)[0])
 
 
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("d,cs", [(602, 304), (102, 102), (66, 40)])
+def test_sq_decompress_rows_of_4k_plus_2_columns(bits, d, cs):
+    """Even widths that are no multiple of four: output rows start at multiples of 8 bytes only and end with a group of
+    two columns; the last source row's code bytes end with the table."""
+    rng = np.random.default_rng(bits * 1000 + d)
+    x = (rng.standard_normal((3001, d)) * rng.uniform(0.5, 2, size=d)).astype(np.float32)
+    n_cb = (d + cs - 1) // cs
+    cbs = np.stack([oc.sq_codebook(x[:, i * cs:(i + 1) * cs]) for i in range(n_cb)])
+    store = oc.sq_codes_to_storage(oc.sq_compress(x, cbs, bits, cs), bits)
+    got = host(capi.sq_decompress(dev(store), dev(cbs), bits, cs, d))
+    assert np.array_equal(got, oc.sq_decompress(store, cbs, bits, cs, d))
+
+
 def test_sq_decompress_accepts_int8_storage():
     rng = np.random.default_rng(9)
     x = rng.uniform(-1, 1, size=(100, 64)).astype(np.float32)
@@ -208,7 +222,7 @@ def test_sq_decompress_accepts_int8_storage():
 
 
 @pytest.mark.parametrize("bits", [1, 2, 4, 8])
-@pytest.mark.parametrize("d", [10, 100, 128])
+@pytest.mark.parametrize("d", [10, 100, 128, 102, 602, 66])
 def test_sq_affine_decompress_bit_exact(bits, d):
     rng = np.random.default_rng(bits * 10 + d)
     x = (rng.standard_normal((2000, d)) * rng.uniform(0.5, 2, size=d)).astype(np.float32)
@@ -257,7 +271,9 @@ def test_vq_decompress_codebook_larger_than_lds():
 
 
 @pytest.mark.parametrize("shape", [(16, 256, 8, 128, 5077), (8, 64, 16, 100, 3001), (25, 256, 4, 100, 1024),
-                                   (24, 200, 32, 768, 2049), (2, 256, 64, 128, 4096), (16, 256, 8, 64, 1500)])
+                                   (24, 200, 32, 768, 2049), (2, 256, 64, 128, 4096), (16, 256, 8, 64, 1500),
+                                   (19, 256, 32, 602, 2049), (13, 256, 8, 102, 3001), (17, 64, 8, 130, 1100),
+                                   (9, 256, 8, 66, 1500)])
 def test_vq_decompress_tile_path(shape):
     # uint8 codes + fp32 codebooks of a width dividing 128: the persistent LDS-tile kernel, with
     # row counts that leave a remainder after the last full 256-row step
