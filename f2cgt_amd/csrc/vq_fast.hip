@@ -309,8 +309,10 @@ __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlan
 // columns, 3e6 edges, 10 per row).  A tile of two columns in all (130 = 128 + 2) stores those alone.  The codebooks
 // hold the columns up to the next multiple of 4, since n_cb * w >= feat_dim is a multiple of 8, so the sums are
 // formed as for a full group.
+// QUAD (H == 2): the two 16-byte halves of a lane's result are exchanged inside lane quads before they are stored,
+// so that a store instruction writes whole 64-byte pieces (see the store at the end of a step).
 template <int BT, int H, int RPM, typename Idx, bool DENSE = false, bool TRACE = false, bool TAIL = false,
-          bool EVEN2 = false>
+          bool EVEN2 = false, bool QUAD = false>
 __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* __restrict__ indptr,
                                                            const Idx* __restrict__ indices,
                                                            float* __restrict__ out) {
@@ -794,6 +796,39 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
             } else {
               store_nt4_align8(dst, acc[0][0], acc[0][1], acc[0][2], acc[0][3]);
             }
+          } else if constexpr (QUAD) {
+            // A lane's eight columns are 32 contiguous bytes; stored as they are, each of the two store
+            // instructions writes 16 of every 32 bytes.  Here the four lanes of a quad exchange their halves
+            // (lane permutes inside the quad, no LDS), so that one instruction writes the first 64 contiguous
+            // bytes of the quad's 128 and the other the last 64: lane k stores half (k & 1) of lane (k >> 1),
+            // then of lane 2 + (k >> 1).
+            const int lr = lane & (kLanesPerRow - 1), k = lr & 3;
+            const bool odd = (k & 1) != 0;
+            float va[4], vb[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+              const int lo_a = __builtin_amdgcn_update_dpp(0, __float_as_int(acc[0][t]), 0x50, 0xf, 0xf, false);
+              const int hi_a = __builtin_amdgcn_update_dpp(0, __float_as_int(acc[1][t]), 0x50, 0xf, 0xf, false);
+              const int lo_b = __builtin_amdgcn_update_dpp(0, __float_as_int(acc[0][t]), 0xfa, 0xf, 0xf, false);
+              const int hi_b = __builtin_amdgcn_update_dpp(0, __float_as_int(acc[1][t]), 0xfa, 0xf, 0xf, false);
+              va[t] = __int_as_float(odd ? hi_a : lo_a);
+              vb[t] = __int_as_float(odd ? hi_b : lo_b);
+            }
+            // Columns of this lane's two pieces inside the tile.  A first piece beyond the tile's columns belongs to
+            // a lane beyond them as well, which holds a copy of the last column group: it stores that group's second
+            // half, the tile's last 16 bytes.  A second piece beyond the columns repeats the lane's first store.
+            const int col_a = (lr >> 2) * 32 + 4 * k, col_b = col_a + 16;
+            const int last = tile_cols - 4;
+            const bool in_a = col_a <= last, in_b = col_b <= last;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+              va[t] = in_a ? va[t] : acc[1][t];
+              vb[t] = in_b ? vb[t] : va[t];
+            }
+            const int pa = in_a ? col_a : last, pb = in_b ? col_b : pa;
+            const uint32_t row_b = (uint32_t)row * ((uint32_t)a.feat_dim * 4u);
+            store_nt4(reinterpret_cast<float*>(obase + (row_b + 4u * (uint32_t)pa)), va[0], va[1], va[2], va[3]);
+            store_nt4(reinterpret_cast<float*>(obase + (row_b + 4u * (uint32_t)pb)), vb[0], vb[1], vb[2], vb[3]);
           } else {
 #pragma unroll
             for (int h = 0; h < H; ++h) store_nt4(dst + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
@@ -1217,7 +1252,17 @@ int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int id
       return launch_status(what);
     }
   }
-  if (tail)
+  constexpr bool CAN_QUAD = H == 2 && RPM == 4;
+  const bool quad = CAN_QUAD && a.dense_store == 4;
+  if (quad && tail)
+    kern = idx_dtype == F2CGT_DT_I32
+               ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false, false, true, false, CAN_QUAD>)
+               : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t, false, false, true, false, CAN_QUAD>);
+  else if (quad)
+    kern = idx_dtype == F2CGT_DT_I32
+               ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false, false, false, false, CAN_QUAD>)
+               : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t, false, false, false, false, CAN_QUAD>);
+  else if (tail)
     kern = idx_dtype == F2CGT_DT_I32
                ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false, false, true>)
                : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t, false, false, true>);
@@ -1262,6 +1307,18 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
   // with few edges per row the output dominates and its store pattern decides (fanout 2 at the C3
   // shape: 845 -> 405 us); from about 8 edges per row the detour through LDS costs more than it saves
   a.dense_store = avg_deg <= 8.0;
+  // Above that, with the code table small enough to stay cached (the launch is then bound by its output) and
+  // either rows of up to 11 edges or an output that the 256 MB last-level cache cannot hold while the two halves
+  // of a 32-byte piece arrive, the halves are exchanged inside lane quads so that every store instruction writes
+  // whole 64-byte pieces (dense_store 4; 1e6 source rows, 3e6 edges at 10 per row: 16 x 16 121 -> 87 us,
+  // 32 x 16 166 -> 90, 8 x 32 126 -> 90, 64 x 8 150 -> 93, 16 x 8 49 -> 42; 7.5e6 edges at 15 per row from a 160 MB
+  // table, 16 x 8: 80.7 -> 78.0 us).  Where the gather dominates the exchange only costs its 24 vector
+  // instructions per row pass (a 5.8 GB table, 24 x 32 at 10 edges per row: 418 -> 454 us), and 64-column tiles
+  // (half the lanes of a row idle) and six-tile rows measured 3-12 % slower with it: those keep the plain stores.
+  if (!a.dense_store && a.feat_dim % 8 == 0 && a.feat_dim >= 128 && a.n_tiles <= 4 &&
+      avg_deg <= 16.0 * ((a.R > 0 && a.E % a.R == 0) ? 1.0 : 0.9) && a.N * (int64_t)a.n_cb <= (192ll << 20) &&
+      (avg_deg <= 11.0 || a.R * (int64_t)a.feat_dim * 4 >= (200ll << 20)))
+    a.dense_store = 4;
 #ifdef F2CGT_EXPERIMENTS
   {
     if (const char* d = getenv("F2CGT_VQ_DEFER")) a.store_late = atoi(d);
