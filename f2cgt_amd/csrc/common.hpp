@@ -132,11 +132,22 @@ __device__ __forceinline__ void store4_align8(float* p, float a, float b, float 
 // [code][128 columns], columns from tile_cols on zero.  A thread issues UNROLL loads back to back
 // before it waits for the first, so the 128 KB of a 256-code tile cost a few load latencies
 // instead of one per element.  PAIR places column 8 j + 4 h + t at h * 64 + 4 j + t (the layout
-// of the kernels that give one lane a whole 8-column code).  With 16-byte aligned codebooks and
-// tile_cols a multiple of 4 the loads are float4.
+// of the kernels that give one lane a whole 8-column code); with lg > 0 the lanes own their columns
+// in groups of g = 2^lg (pair_pos).  With 16-byte aligned codebooks and tile_cols a multiple of 4 the
+// loads are float4.
+//
+// pair_pos: where the PAIR layout keeps tile column c (a multiple of 4).  Lane j = g c' + k of a row owns the
+// columns 8 g c' + 4 g h + 4 k + t (h = 0, 1; t < 4) and reads them at h * 64 + 4 j + t: g = 1 is a lane's own
+// eight columns; with g = 4 (codebooks of 32 columns and more: the four lanes share their code) the h-th store
+// instruction of a wave writes the 64 contiguous bytes 4 k + t of every group instead of 16 of every 32.
+__device__ __forceinline__ int pair_pos(int c, int lg) {
+  const int g1 = (1 << lg) - 1;
+  const int j = ((c >> (3 + lg)) << lg) + ((c >> 2) & g1);
+  return ((c >> (2 + lg)) & 1) * 64 + 4 * j;
+}
 template <int THREADS, bool PAIR>
 __device__ __forceinline__ void stage_codebook_tile(float* __restrict__ s_cb, const float* __restrict__ codebooks,
-                                                    int K, int w, int tile, int tile_cols) {
+                                                    int K, int w, int tile, int tile_cols, int lg = 0) {
   constexpr int UNROLL = 8;
   const bool vec = (reinterpret_cast<uintptr_t>(codebooks) & 15) == 0 && (tile_cols & 3) == 0 && (w & 3) == 0;
   if (vec) {
@@ -158,7 +169,7 @@ __device__ __forceinline__ void stage_codebook_tile(float* __restrict__ s_cb, co
       for (int u = 0; u < UNROLL; ++u) {
         const int i = i0 + u * THREADS;
         const int code = i >> 5, c = (i & 31) * 4;
-        const int pos = PAIR ? ((c >> 2) & 1) * 64 + (c >> 3) * 4 : c;
+        const int pos = PAIR ? pair_pos(c, lg) : c;
         if (i < n4) *reinterpret_cast<float4*>(s_cb + (code << 7) + pos) = v[u];
       }
     }
@@ -181,7 +192,7 @@ __device__ __forceinline__ void stage_codebook_tile(float* __restrict__ s_cb, co
     for (int u = 0; u < UNROLL; ++u) {
       const int i = i0 + u * THREADS;
       const int code = i >> 7, c = i & 127;
-      const int pos = PAIR ? ((c >> 2) & 1) * 64 + (c >> 3) * 4 + (c & 3) : c;
+      const int pos = PAIR ? pair_pos(c & ~3, lg) + (c & 3) : c;
       if (i < n) s_cb[(code << 7) + pos] = v[u];
     }
   }
@@ -211,13 +222,13 @@ __device__ __forceinline__ void stage_codebook_load(float4 (&v)[8], const float*
   }
 }
 template <int THREADS, bool PAIR>
-__device__ __forceinline__ void stage_codebook_store(float* __restrict__ s_cb, const float4 (&v)[8], int K) {
+__device__ __forceinline__ void stage_codebook_store(float* __restrict__ s_cb, const float4 (&v)[8], int K, int lg = 0) {
   const int n4 = K * 32;
 #pragma unroll
   for (int u = 0; u < 8; ++u) {
     const int i = threadIdx.x + u * THREADS;
     const int code = i >> 5, c = (i & 31) * 4;
-    const int pos = PAIR ? ((c >> 2) & 1) * 64 + (c >> 3) * 4 : c;
+    const int pos = PAIR ? pair_pos(c, lg) : c;
     if (i < n4) *reinterpret_cast<float4*>(s_cb + (code << 7) + pos) = v[u];
   }
 }

@@ -39,6 +39,7 @@ struct VqArgs {
   int n_tiles, n_stripes;
   int stripes_per_xcd;  // > 0: the column tiles of a stripe share one XCD (see the kernel)
   int dense_store;      // sparse rows: results go through LDS so that every store instruction is dense
+  int own_lg;           // 2: the launch takes the form whose lanes own their columns in groups of four (pair_pos)
   int store_late;       // experiments build only: 9 = the time-stamped form of the wave kernel
   unsigned long long* trace;   // experiments build only: per wave {start, first step, end} in 100 MHz ticks
 };
@@ -311,8 +312,9 @@ __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlan
 // formed as for a full group.
 // QUAD (H == 2): the two 16-byte halves of a lane's result are exchanged inside lane quads before they are stored,
 // so that a store instruction writes whole 64-byte pieces (see the store at the end of a step).
+// OWN (H == 2): the binary logarithm of the number of lanes that own the columns of a code together (pair_pos).
 template <int BT, int H, int RPM, typename Idx, bool DENSE = false, bool TRACE = false, bool TAIL = false,
-          bool EVEN2 = false, bool QUAD = false>
+          bool EVEN2 = false, bool QUAD = false, int OWN = 0>
 __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* __restrict__ indptr,
                                                            const Idx* __restrict__ indices,
                                                            float* __restrict__ out) {
@@ -386,7 +388,9 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
   const int groups = tile_cols / (4 * H);      // column groups of this tile (tile_cols % (4 H) == 0)
   const int c4 = (lane & (kLanesPerRow - 1)) < groups ? (lane & (kLanesPerRow - 1)) : groups - 1;
   const int half = lane / kLanesPerRow;
-  const int col0 = c4 * 4 * H;                 // first column of the lane inside the tile
+  // first column of the lane inside the tile; with H == 2 its second float4 lies 4 << own_lg columns on (pair_pos)
+  constexpr int own_lg = H == 2 ? OWN : 0;
+  const int col0 = H == 2 ? ((c4 >> own_lg) << (3 + own_lg)) + 4 * (c4 & ((1 << own_lg) - 1)) : c4 * 4;
   const int byte_idx = col0 / a.w;
   const float* cbp = s_cb + c4 * 4;
   const int prev_group_lane = (lane & ~(kLanesPerRow - 1)) + (c4 > 0 ? c4 - 1 : 0);   // EVEN2
@@ -517,12 +521,12 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
       const Idx* src = on ? indices + e0 + eb1 + lane : indptr;
       Ireg = (int64_t)*src;                                // I(1)
     }
-    stage_codebook_store<kThreads, H == 2>(s_cb, cbv, a.K);
+    stage_codebook_store<kThreads, H == 2>(s_cb, cbv, a.K, own_lg);
     __syncthreads();
     if (!has_rows) return;
     g_first = 0;
   } else {
-    stage_codebook_tile<kThreads, H == 2>(s_cb, a.codebooks, a.K, a.w, tile, tile_cols);
+    stage_codebook_tile<kThreads, H == 2>(s_cb, a.codebooks, a.K, a.w, tile, tile_cols, own_lg);
     if (threadIdx.x == 0) *s_next = kWaves;
     __syncthreads();
     if (!has_rows) return;
@@ -830,8 +834,13 @@ __global__ __launch_bounds__(kThreads) void vq_wave_kernel(VqArgs a, const Idx* 
             store_nt4(reinterpret_cast<float*>(obase + (row_b + 4u * (uint32_t)pa)), va[0], va[1], va[2], va[3]);
             store_nt4(reinterpret_cast<float*>(obase + (row_b + 4u * (uint32_t)pb)), vb[0], vb[1], vb[2], vb[3]);
           } else {
+            // H == 2: the second float4 lies 16 bytes on, or 64 with columns owned in groups of four lanes (pair_pos).
+            // The distance is a literal so that it folds into the second store: with it in a register the two are no
+            // longer issued back to back, the halves of a 32-byte piece reach the L2 apart and leave it as partial
+            // writes (24 x 32 from a 5.8 GB table: 433 -> 958 us).
 #pragma unroll
-            for (int h = 0; h < H; ++h) store_nt4(dst + 4 * h, acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+            for (int h = 0; h < H; ++h)
+              store_nt4(dst + ((4 * h) << own_lg), acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
           }
         }
       }
@@ -1223,7 +1232,8 @@ template <int BT, int H, int RPM>
 int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int idx_dtype, float* out, hipStream_t st,
                 const char* what, unsigned grid, size_t wlds) {
   if (plan_only()) {
-    plan_record("vq_wave_kernel", grid, kThreads, (int64_t)wlds, 0, H, RPM, a.dense_store);
+    plan_record("vq_wave_kernel", grid, kThreads, (int64_t)wlds, 0, H, RPM, a.dense_store,
+                (H == 2 && RPM == 4 && BT == 4 && a.dense_store == 0) ? a.own_lg : 0);
     return 0;
   }
 #ifdef F2CGT_EXPERIMENTS
@@ -1254,6 +1264,22 @@ int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int id
   }
   constexpr bool CAN_QUAD = H == 2 && RPM == 4;
   const bool quad = CAN_QUAD && a.dense_store == 4;
+  if constexpr (H == 2 && RPM == 4 && BT == 4) {   // codebooks of 32 columns
+    if (a.own_lg == 2 && a.dense_store == 0) {
+      kern = tail ? (idx_dtype == F2CGT_DT_I32
+                         ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false, false, true, false, false, 2>)
+                         : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t, false, false, true, false, false, 2>))
+                  : (idx_dtype == F2CGT_DT_I32
+                         ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false, false, false, false, false, 2>)
+                         : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t, false, false, false, false, false, 2>));
+      const hipError_t e3 = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
+      if (e3 != hipSuccess) return fail((int)e3, "%s: cannot reserve %zu B of LDS", what, wlds);
+      void* params3[] = {const_cast<VqArgs*>(&a), &indptr, &indices, &out};
+      const hipError_t le3 = hipLaunchKernel(kern, dim3(grid), dim3(kThreads), params3, wlds, st);
+      if (le3 != hipSuccess) return fail((int)le3, "%s: launch failed: %s", what, hipGetErrorString(le3));
+      return launch_status(what);
+    }
+  }
   if (quad && tail)
     kern = idx_dtype == F2CGT_DT_I32
                ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false, false, true, false, CAN_QUAD>)
@@ -1340,6 +1366,13 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     }
   }
 #endif
+  // Codebooks of 32 columns: the four lanes that share a code can own its columns as a group, so that a store
+  // instruction writes 64 contiguous bytes per group at no cost in instructions (pair_pos; its own instantiation,
+  // OWN = 2).  Taken where the exchange inside quads is not and the code table stays cached.
+  a.own_lg = 0;
+  if (a.dense_store == 0 && a.w == 32 && a.feat_dim % 32 == 0 && a.feat_dim >= 128 &&
+      avg_deg <= 16.0 * ((a.R > 0 && a.E % a.R == 0) ? 1.0 : 0.9) && a.N * (int64_t)a.n_cb <= (192ll << 20))
+    a.own_lg = 2;
 #ifdef F2CGT_EXPERIMENTS
   if (const char* v = getenv("F2CGT_VQ_RPM")) {   // rows per mini-block whatever the degree (mini-blocks above 64 edges unstaged)
     if (a.feat_dim % 8 == 0) {

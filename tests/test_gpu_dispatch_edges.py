@@ -201,13 +201,16 @@ def test_fused_vq_code_rows_that_are_no_multiple_of_a_tile(feat_dim, n_cb, width
 
 @pytest.mark.parametrize("idx", [np.int64, np.int32])
 @pytest.mark.parametrize("feat_dim,n_cb,width", [(128, 16, 8), (136, 17, 8), (200, 25, 8), (200, 13, 16), (264, 33, 8),
-                                                 (512, 16, 32), (160, 5, 32), (328, 41, 8)])
-@pytest.mark.parametrize("fanout,ragged", [(9, False), (10, True), (11, False), (14, True)])
+                                                 (512, 16, 32), (160, 5, 32), (328, 41, 8), (256, 16, 16), (96, 6, 16),
+                                                 (96, 3, 32), (224, 7, 32)])
+@pytest.mark.parametrize("fanout,ragged", [(9, False), (10, True), (11, False), (14, True), (20, False), (40, True)])
 def test_fused_vq_halves_exchanged_inside_lane_quads(feat_dim, n_cb, width, fanout, ragged, idx):
     """Nine to eleven edges per row from a small code table: the two 16-byte halves of a lane's eight columns are
     exchanged inside lane quads so that a store instruction writes whole 64-byte pieces.  Last tiles of 8, 72 and 32
     columns leave quads with one, two or three lanes beyond the columns, whose pieces must not be stored; 13 x 16 and
-    5 x 32 are code rows that are no multiple of a tile; the last tile of 328 columns is 72 columns wide."""
+    5 x 32 are code rows that are no multiple of a tile; the last tile of 328 columns is 72 columns wide.  With
+    codebooks of 32 (16) columns and rows of whole such groups the four (two) lanes that share a code own its columns
+    together instead, at every row length (four-, two- and one-row mini-blocks)."""
     rng = np.random.default_rng(feat_dim * 31 + fanout + (idx == np.int32))
     n_src, rows = 5000, 2500
     codes = rng.integers(0, 256, size=(n_src, n_cb), dtype=np.uint8)
