@@ -1244,7 +1244,7 @@ int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int id
   // the sparse-row form (results turned round in LDS before they are stored) is its own instantiation
   constexpr bool CAN_DENSE = H == 2 && RPM == 4;
   const bool tail = a.n_cb % BT != 0 || !aligned(a.codes, BT);
-  const bool dense = CAN_DENSE && a.dense_store == 1 && !tail;
+  const bool dense = CAN_DENSE && a.dense_store == 1;
   const void* kern;
   if constexpr (H == 1 && RPM == 4) {
     if (a.feat_dim % 4 != 0) {   // even widths that are no multiple of 4
@@ -1288,6 +1288,10 @@ int launch_wave(const VqArgs& a, const void* indptr, const void* indices, int id
     kern = idx_dtype == F2CGT_DT_I32
                ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false, false, false, false, CAN_QUAD>)
                : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t, false, false, false, false, CAN_QUAD>);
+  else if (tail && dense)
+    kern = idx_dtype == F2CGT_DT_I32
+               ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, CAN_DENSE, false, true>)
+               : reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int64_t, CAN_DENSE, false, true>);
   else if (tail)
     kern = idx_dtype == F2CGT_DT_I32
                ? reinterpret_cast<const void*>(vq_wave_kernel<BT, H, RPM, int32_t, false, false, true>)
@@ -1397,6 +1401,16 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     // fixed fanout): those get the exact limits, ragged rows 0.9 of them (capped at 32 with 15.2 on average: 112 us
     // in fours, 91 in twos; capped at 64 with 30.1: 198 in twos, 171 one by one).
     const double fit = (a.R > 0 && a.E % a.R == 0) ? 1.0 : 0.9;
+    // Sparse rows that are no whole 128-byte lines (feat_dim no multiple of 32): one float4 per lane, 32 lanes per
+    // row, is ahead of the eight-column form whose results are turned round in LDS (3e6 edges at 3 / 6 per row:
+    // 25 x 8 326 / 165 -> 299 / 146 us, 21 x 8 299 / 150 -> 257 / 123, 15 x 8 186 / 102 -> 152 / 76, 19 x 32 at 600
+    // columns 603 / 313 -> 551 / 279; rows of whole lines the other way round: 24 x 8 172 / 101 against 191 / 100,
+    // 7 x 32 180 / 96 against 192 / 103).
+    if (avg_deg <= 8.0 && a.feat_dim % 32 != 0) {
+      a.dense_store = 0;
+      a.own_lg = 0;
+      return launch_wave<BT, 1, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    }
     if (avg_deg <= 16.0 * fit) return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
     if (avg_deg <= 32.0 * fit) return launch_wave<BT, 2, 2>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
     return launch_wave<BT, 2, 1>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);

@@ -160,3 +160,11 @@ def test_fused_vq_store_form_by_shape():
     assert form(300_000, 20, 128, 4, 32, 1_000_000) == (0, 0)
     assert form(300_000, 10, 600, 19, 32, 1_000_000) == (0, 0)      # 600 columns: the last tile ends inside a group of 32
     assert form(300_000, 10, 100, 13, 8, 1_000_000)[1] == 0         # four columns per lane: dense as they are
+    # aux[0]: float4 per lane and edge (2 = a lane owns eight columns); sparse rows that are no whole 128-byte lines
+    # take one, code rows that are no multiple of a tile (24 x 8, 7 x 32) can take the turn through LDS
+    lanes = lambda rows, fanout, d, n_cb, w: capi.dry_run(
+        "f2cgt_vq_decompress_spmm_csr", A16, capi.DT_U8, A16, A16, A16, capi.DT_I64, A16, rows, rows * fanout,
+        1_000_000, d, n_cb, 256, w, None)[1].aux[0]
+    assert lanes(1_000_000, 3, 200, 25, 8) == 1 and lanes(300_000, 10, 200, 25, 8) == 2
+    assert lanes(1_000_000, 3, 192, 24, 8) == 2 and form(1_000_000, 3, 192, 24, 8, 1_000_000) == (1, 0)
+    assert lanes(1_000_000, 3, 224, 7, 32) == 2 and lanes(1_000_000, 3, 600, 19, 32) == 1
