@@ -223,13 +223,10 @@ struct F4Args {
   int64_t total_f4;
   uint32_t f4_per_row;
   uint32_t magic;         // ceil(2^32 / f4_per_row)
-  int feat_dim;           // HALF decoders: columns of a row, 4 * f4_per_row - 2
+  int feat_dim;           // sq_decode_pairs_kernel: columns of a row
 };
 
-// HALF: rows of 4 k + 2 columns.  A lane still owns a group of four columns of a row; output rows start at multiples
-// of 8 bytes only, which a 16-byte store takes at any dword, and the row's last group holds two columns: it loads only
-// their code bytes and stores them alone (the tables in LDS repeat the last column for the two it has not).
-template <int BITS, bool AFFINE, bool HALF = false>
+template <int BITS, bool AFFINE>
 __global__ __launch_bounds__(kBlock) void sq_decode_f4_kernel(F4Args a) {
   constexpr int NCODE = 1 << BITS;
   constexpr uint32_t MASK = NCODE - 1;
@@ -239,15 +236,14 @@ __global__ __launch_bounds__(kBlock) void sq_decode_f4_kernel(F4Args a) {
   int* s_cbi = reinterpret_cast<int*>(s_tab + ((a.n_cb * NCODE + 3) & ~3));
   if (AFFINE) {
     for (int i = threadIdx.x; i < feat_dim; i += kBlock) {
-      const int col = HALF && i >= a.feat_dim ? a.feat_dim - 1 : i;
-      s_tab[(i >> 2) * 8 + (i & 3)] = a.table[col];
-      s_tab[(i >> 2) * 8 + 4 + (i & 3)] = a.table[a.param_stride + col];
+      s_tab[(i >> 2) * 8 + (i & 3)] = a.table[i];
+      s_tab[(i >> 2) * 8 + 4 + (i & 3)] = a.table[a.param_stride + i];
     }
   } else {
     for (int i = threadIdx.x; i < a.n_cb * NCODE; i += kBlock)
       s_tab[i] = sq_log_value<BITS>((uint32_t)(i & MASK), a.table + (int64_t)(i >> BITS) * 5);
     for (int i = threadIdx.x; i < feat_dim; i += kBlock) {
-      int64_t cb = (HALF && i >= a.feat_dim ? a.feat_dim - 1 : i) / a.column_slice;
+      int64_t cb = i / a.column_slice;
       cb = cb < a.n_cb ? cb : a.n_cb - 1;
       s_cbi[i] = (int)cb * NCODE;
     }
@@ -261,7 +257,7 @@ __global__ __launch_bounds__(kBlock) void sq_decode_f4_kernel(F4Args a) {
   if ((rb + 1) * (int64_t)a.f4_per_row <= base) ++rb;
   const uint32_t cb0 = (uint32_t)(base - rb * a.f4_per_row);
 
-  uint32_t word[kF4Items], c4s[kF4Items], rls[kF4Items];
+  uint32_t word[kF4Items], c4s[kF4Items];
 #pragma unroll
   for (int k = 0; k < kF4Items; ++k) {
     const uint32_t li = cb0 + threadIdx.x + k * kBlock;
@@ -270,11 +266,7 @@ __global__ __launch_bounds__(kBlock) void sq_decode_f4_kernel(F4Args a) {
     const bool on = base + threadIdx.x + k * kBlock < a.total_f4;
     const uint8_t* src = a.codes + (on ? (rb + rl) * a.src_dim : 0);
     c4s[k] = c4;
-    rls[k] = rl;
-    if (HALF && BITS >= 4 && on && c4 + 1 == a.f4_per_row) {   // the row's last two columns
-      if (BITS == 8) { uint16_t w; __builtin_memcpy(&w, src + 4 * c4, 2); word[k] = w; }
-      else word[k] = src[2 * c4];
-    } else if (BITS == 8) {
+    if (BITS == 8) {
       uint32_t w; __builtin_memcpy(&w, src + (on ? 4 * c4 : 0), 4); word[k] = w;
     } else if (BITS == 4) {
       uint16_t w; __builtin_memcpy(&w, src + (on ? 2 * c4 : 0), 2); word[k] = w;
@@ -304,12 +296,91 @@ __global__ __launch_bounds__(kBlock) void sq_decode_f4_kernel(F4Args a) {
       v[2] = s_tab[cbi.z + ((word[k] >> (2 * BITS)) & MASK)];
       v[3] = s_tab[cbi.w + ((word[k] >> (3 * BITS)) & MASK)];
     }
-    if constexpr (HALF) {
-      float* dst = a.out + ((rb + rls[k]) * (int64_t)a.feat_dim + 4 * c4);
-      if (c4 + 1 == a.f4_per_row) store_nt2(dst, v[0], v[1]);
-      else store_nt4_align8(dst, v[0], v[1], v[2], v[3]);
+    store_nt4(a.out + i * 4, v[0], v[1], v[2], v[3]);
+  }
+}
+
+// Rows of 4 k + 2 columns, decoded through a flat view of the output: the matrix as a whole is still a run of
+// 16-byte pieces (rows * feat_dim is a multiple of 4 when the row count is even; an odd count leaves one pair),
+// and a piece is two column pairs, of one row or of the end of a row and the start of the next.  A lane owns
+// a piece: two (row, pair) positions from one multiply-high each, the code bits of the two pairs (2 / 1 bytes,
+// a nibble, two bits), the per-column tables from LDS, and one aligned 16-byte store, so that the stores of a
+// workgroup are as dense as for rows of whole float4 groups (4e5 rows of 602 columns, 4 bit: 253 us with a group of
+// four columns per lane and stores that start 8 bytes off, 176 us at 600 columns).
+template <int BITS, bool AFFINE>
+__global__ __launch_bounds__(kBlock) void sq_decode_pairs_kernel(F4Args a) {
+  constexpr int NCODE = 1 << BITS;
+  constexpr uint32_t MASK = NCODE - 1;
+  extern __shared__ __align__(16) float s_tab[];
+  // affine: [column][min, scale]; log domain: LUT [n_cb][NCODE], then the LUT base of each column
+  int* s_cbi = reinterpret_cast<int*>(s_tab + ((a.n_cb * NCODE + 3) & ~3));
+  if (AFFINE) {
+    for (int i = threadIdx.x; i < a.feat_dim; i += kBlock) {
+      s_tab[2 * i] = a.table[i];
+      s_tab[2 * i + 1] = a.table[a.param_stride + i];
+    }
+  } else {
+    for (int i = threadIdx.x; i < a.n_cb * NCODE; i += kBlock)
+      s_tab[i] = sq_log_value<BITS>((uint32_t)(i & MASK), a.table + (int64_t)(i >> BITS) * 5);
+    for (int i = threadIdx.x; i < a.feat_dim; i += kBlock) {
+      int64_t cb = i / a.column_slice;
+      cb = cb < a.n_cb ? cb : a.n_cb - 1;
+      s_cbi[i] = (int)cb * NCODE;
+    }
+  }
+  __syncthreads();
+  const uint32_t ppr = a.f4_per_row;             // pairs per row (feat_dim / 2)
+  const int64_t total_pairs = a.total_f4;        // rows * pairs per row
+  const int64_t base = (int64_t)blockIdx.x * (kF4Items * kBlock);
+  // first row of the workgroup's span of pairs: floor(2 base / ppr), from the fp64 quotient and a fix-up; the pairs
+  // of the span are then counted from that row's first, small enough for the 32-bit multiply-high to be exact
+  int64_t rb = (int64_t)((double)(2 * base) / (double)ppr);
+  if (rb * ppr > 2 * base) --rb;
+  if ((rb + 1) * (int64_t)ppr <= 2 * base) ++rb;
+  const uint32_t l0 = (uint32_t)(2 * base - rb * ppr);
+  auto pair = [&](int64_t p, float& v0, float& v1) {
+    const uint32_t li = l0 + (uint32_t)(p - 2 * base);
+    const uint32_t rl = __umulhi(li, a.magic);
+    const uint32_t cp = li - rl * ppr;
+    const uint8_t* src = a.codes + (rb + rl) * a.src_dim;
+    uint32_t c0, c1;
+    if (BITS == 8) {
+      uint16_t w; __builtin_memcpy(&w, src + 2 * cp, 2);
+      c0 = w & 0xffu; c1 = w >> 8;
+    } else if (BITS == 4) {
+      const uint32_t w = src[cp];
+      c0 = w & 0xfu; c1 = w >> 4;
+    } else if (BITS == 2) {
+      const uint32_t w = src[cp >> 1] >> ((cp & 1) * 4);
+      c0 = w & 3u; c1 = (w >> 2) & 3u;
     } else {
-      store_nt4(a.out + i * 4, v[0], v[1], v[2], v[3]);
+      const uint32_t w = src[cp >> 2] >> ((cp & 3) * 2);
+      c0 = w & 1u; c1 = (w >> 1) & 1u;
+    }
+    const uint32_t col = 2 * cp;
+    if (AFFINE) {
+      const float4 t = *reinterpret_cast<const float4*>(s_tab + 2 * col);   // min, scale of the two columns
+      v0 = __fadd_rn(t.x, __fmul_rn((float)c0, t.y));
+      v1 = __fadd_rn(t.z, __fmul_rn((float)c1, t.w));
+    } else {
+      const int2 cbi = *reinterpret_cast<const int2*>(s_cbi + col);
+      v0 = s_tab[cbi.x + c0];
+      v1 = s_tab[cbi.y + c1];
+    }
+  };
+  const int64_t n4 = total_pairs >> 1;
+#pragma unroll
+  for (int k = 0; k < kF4Items; ++k) {
+    const int64_t i = base + threadIdx.x + k * kBlock;
+    if (i < n4) {
+      float v[4];
+      pair(2 * i, v[0], v[1]);
+      pair(2 * i + 1, v[2], v[3]);
+      store_nt4(a.out + 4 * i, v[0], v[1], v[2], v[3]);
+    } else if (i == n4 && (total_pairs & 1)) {   // an odd number of rows: the matrix ends with one pair
+      float v0, v1;
+      pair(2 * i, v0, v1);
+      store_nt2(a.out + 4 * i, v0, v1);
     }
   }
 }
@@ -321,22 +392,25 @@ int decode_f4_launch(const uint8_t* codes, float* out, const float* table, int64
                      hipStream_t st, const char* what) {
   // (one float4 per row would need the reciprocal 2^32, which does not fit the 32-bit multiplier)
   if (feat_dim % 2 != 0 || feat_dim < 8 || feat_dim > 8192 || !aligned(out, 16)) return -1;
-  const int64_t padded = (feat_dim + 3) / 4 * 4;   // rows of 4 k + 2 columns: tables for the group of two as for four
-  const size_t lds = AFFINE ? (size_t)padded * 8
-                            : ((((size_t)n_cb << BITS) + 3) / 4 * 4 + (size_t)padded) * 4;
+  const size_t lds = AFFINE ? (size_t)feat_dim * 8
+                            : ((((size_t)n_cb << BITS) + 3) / 4 * 4 + (size_t)feat_dim) * 4;
   if (lds > (size_t)kMaxLutBytes) return -1;
   F4Args a{};
   a.codes = codes; a.out = out; a.table = table;
   a.param_stride = param_stride; a.column_slice = column_slice; a.n_cb = AFFINE ? 0 : n_cb;
   a.src_dim = src_dim;
   a.feat_dim = (int)feat_dim;
-  a.f4_per_row = (uint32_t)(padded / 4);
-  a.total_f4 = rows * (padded / 4);
+  // items per row: float4 groups, or column pairs for rows of 4 k + 2 columns (the flat view: two pairs per lane,
+  // plus one lane for the last pair of an odd number of rows)
+  const bool pairs = feat_dim % 4 != 0;
+  a.f4_per_row = (uint32_t)(pairs ? feat_dim / 2 : feat_dim / 4);
+  a.total_f4 = rows * a.f4_per_row;
   a.magic = (uint32_t)((0x100000000ull + a.f4_per_row - 1) / a.f4_per_row);
-  const int64_t grid = ceil_div(a.total_f4, kF4Items * kBlock);
+  const int64_t lanes = pairs ? a.total_f4 / 2 + 1 : a.total_f4;
+  const int64_t grid = ceil_div(lanes, kF4Items * kBlock);
   if (grid > 0x7fffffffll) return -1;
-  if (feat_dim % 4 == 0) sq_decode_f4_kernel<BITS, AFFINE><<<(unsigned)grid, kBlock, lds, st>>>(a);
-  else sq_decode_f4_kernel<BITS, AFFINE, true><<<(unsigned)grid, kBlock, lds, st>>>(a);
+  if (pairs) sq_decode_pairs_kernel<BITS, AFFINE><<<(unsigned)grid, kBlock, lds, st>>>(a);
+  else sq_decode_f4_kernel<BITS, AFFINE><<<(unsigned)grid, kBlock, lds, st>>>(a);
   return launch_status(what);
 }
 
