@@ -51,7 +51,8 @@ WIDE = [2040, 2044, 2048, 2052, 3000, 4080, 4088, 4092, 4096]
 @pytest.mark.parametrize("bits", [1, 2, 4, 8])
 def test_fused_sq_geometry_over_feature_widths(bits):
     per = 8 // bits
-    dims = sorted(set([4, 8, 12, 16, 24, 36, 64, 100, 128, 256, 300, 512, 768, 1000, 1024, 2000] + WIDE))
+    dims = sorted(set([4, 8, 12, 16, 24, 36, 64, 100, 128, 256, 300, 512, 768, 1000, 1024, 2000] + WIDE +
+                      [6, 10, 18, 30, 66, 102, 130, 602, 1022, 2042, 2046, 4090, 4094]))   # 4 k + 2 columns
     seen = set()
     for d in dims:
         for fanout in (1, 10, 60):
@@ -63,6 +64,21 @@ def test_fused_sq_geometry_over_feature_widths(bits):
             assert rc == 0 and plan is not None, (bits, d, capi.lib().f2cgt_last_error())
             seen.add(check_geometry(plan))
     assert "sq_rows_kernel" in seen and (bits < 4 or "agg_kernel" in seen)
+
+
+def test_even_widths_that_are_no_multiple_of_four_take_the_row_block_kernels():
+    for d in (18, 66, 102, 602):
+        for bits in (4, 8):
+            assert plan_affine(bits, d)[1].kernel.decode() == "sq_affine_acc_kernel", (bits, d)
+            assert plan_log_sq(bits, d)[1].kernel.decode() == "sq_rows_kernel", (bits, d)
+    for bits in (1, 2):
+        assert plan_log_sq(bits, 602)[1].kernel.decode() == "sq_rows_kernel"
+        assert plan_affine(bits, 602)[1].kernel.decode() == "sq_rows_kernel"
+    for d in (17, 101, 601):   # odd widths: one column per lane
+        assert plan_affine(4, d)[1].kernel.decode() == "agg_kernel"
+    vq = capi.dry_run("f2cgt_vq_decompress_spmm_csr", A16, capi.DT_U8, A16, A16, A16, capi.DT_I64, A16, 200_000,
+                      2_000_000, 1_000_000, 602, 19, 256, 32, None)
+    assert vq[0] == 0 and vq[1].kernel.decode() == "vq_wave_kernel" and vq[1].aux[0] == 1
 
 
 def test_wide_rows_leave_the_row_block_kernels():

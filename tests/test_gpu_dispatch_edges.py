@@ -75,7 +75,7 @@ def test_fused_log_sq_with_either_workgroup_size(bits, feat_dim):
 
 @pytest.mark.parametrize("idx", [np.int64, np.int32])
 @pytest.mark.parametrize("bits", [1, 2, 4, 8])
-@pytest.mark.parametrize("feat_dim", [602, 102, 66, 18])
+@pytest.mark.parametrize("feat_dim", [602, 102, 66, 18, 14, 10])
 def test_fused_sq_rows_of_an_even_number_of_columns_that_is_no_multiple_of_four(feat_dim, bits, idx):
     """602, 102 ... columns: output rows start at multiples of 8 bytes only and end with a group of two columns, code
     rows may end inside a byte group.  Affine and log-domain forms, staged and unstaged blocks (rows of 2, 12, 40 and
