@@ -12,7 +12,8 @@ box's host cores on a bounded sample of the same workload.
 
 Every benchmark configuration is in that one line: next to the headline workload's `roofline`,
 `configs` holds the other fused workloads (C1, C3, C3 with scattered ids, C4, C5) and the C5 encode
-step, each with its own launch count, `launch_us` (and, for C3 / C4 / C5, `cold_launch_us` / `frac_cold`
+step, each with its own launch count, `launch_us` (and, for C3 / C4 / C5, `cold_launch_us` / `frac_cold`,
+for C3 / C5 also `cold_streaming_launch_us` / `frac_cold_streaming` in the streaming store mode
 with three blocks and outputs in rotation), `edges_per_s`, `algorithmic_bytes`,
 `compulsory_bytes`, measured HBM `traffic` and four fractions of the 8 TB/s peak:
 `frac_algorithmic` (every edge charged its source row), `frac_traffic` (the bytes the counters saw
@@ -203,6 +204,17 @@ def _configs(idx):
                 entry["cold_launch_us"] = cold_ms * 1e3
                 # the warm fraction scaled by the launch times (the blocks in rotation are the same size)
                 entry["frac_cold"] = entry["frac"] * ms_launch / cold_ms
+                if name in ("c3", "c5"):
+                    # the same rotation in the streaming store mode, which for the fused VQ operator selects the
+                    # form whose store instructions write whole lines at every row length up to 16 edges
+                    was = capi.set_store_mode(capi.STORE_STREAM)
+                    try:
+                        s_ms, _, _ = _cold_launch_ms(name, idx, wl, blocks=3, rounds=max(4, steps // 6),
+                                                     warm_rounds=max(2, warmup // 6))
+                    finally:
+                        capi.set_store_mode(was)
+                    entry["cold_streaming_launch_us"] = s_ms * 1e3
+                    entry["frac_cold_streaming"] = entry["frac"] * ms_launch / s_ms
                 out = None
             res[key] = entry
             del wl, out

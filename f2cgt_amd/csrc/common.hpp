@@ -97,6 +97,7 @@ __device__ __forceinline__ void row_range(const Idx* __restrict__ indptr, int64_
 // whose 400-byte rows leave partial lines to merge.  Hence 140 MB for rows of whole lines or at least six
 // edges per row, and 220 MB otherwise.
 bool stream_output(int64_t out_bytes, int64_t row_bytes, double edges_per_row);
+int store_mode();   // F2CGT_STORE_AUTO / _STREAM / _CACHED as last set by f2cgt_set_store_mode
 
 // Non-temporal stores: the aggregation output is written once and never re-read by
 // the kernel, so it should not displace gathered code rows from L2 / MALL.

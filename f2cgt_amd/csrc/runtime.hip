@@ -37,6 +37,8 @@ bool stream_output(int64_t out_bytes, int64_t row_bytes, double edges_per_row) {
   return out_bytes > (early ? 140000000ll : 220000000ll);
 }
 
+int store_mode() { return g_store_mode.load(std::memory_order_relaxed); }
+
 int num_cus() {
   if (t_plan_only) return 256;   // a dry run must not depend on (or wake) a device
   static std::atomic<int> cached[64];   // 0 = not asked yet; callers may come from several threads

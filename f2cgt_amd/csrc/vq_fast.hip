@@ -19,6 +19,7 @@
 #include "spmm_fast.hpp"
 
 #include <cstdlib>
+#include <cstring>
 #include <type_traits>
 
 namespace f2cgt {
@@ -1337,18 +1338,30 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
   // with few edges per row the output dominates and its store pattern decides (fanout 2 at the C3
   // shape: 845 -> 405 us); from about 8 edges per row the detour through LDS costs more than it saves
   a.dense_store = avg_deg <= 8.0;
-  // Above that, with the code table small enough to stay cached (the launch is then bound by its output) and
-  // either rows of up to 11 edges or an output that the 256 MB last-level cache cannot hold while the two halves
-  // of a 32-byte piece arrive, the halves are exchanged inside lane quads so that every store instruction writes
-  // whole 64-byte pieces (dense_store 4; 1e6 source rows, 3e6 edges at 10 per row: 16 x 16 121 -> 87 us,
-  // 32 x 16 166 -> 90, 8 x 32 126 -> 90, 64 x 8 150 -> 93, 16 x 8 49 -> 42; 7.5e6 edges at 15 per row from a 160 MB
-  // table, 16 x 8: 80.7 -> 78.0 us).  Where the gather dominates the exchange only costs its 24 vector
-  // instructions per row pass (a 5.8 GB table, 24 x 32 at 10 edges per row: 418 -> 454 us), and 64-column tiles
-  // (half the lanes of a row idle) and six-tile rows measured 3-12 % slower with it: those keep the plain stores.
-  if (!a.dense_store && a.feat_dim % 8 == 0 && a.feat_dim >= 128 && a.n_tiles <= 4 &&
-      avg_deg <= 16.0 * ((a.R > 0 && a.E % a.R == 0) ? 1.0 : 0.9) && a.N * (int64_t)a.n_cb <= (192ll << 20) &&
-      (avg_deg <= 11.0 || a.R * (int64_t)a.feat_dim * 4 >= (200ll << 20)))
-    a.dense_store = 4;
+  // Above that (up to 16 edges per row, four-row mini-blocks) the form is chosen by what binds the launch:
+  //  * the code table beyond the caches (over 192 MB) or rows of more than four column tiles: the gather binds, the
+  //    results are stored as they are (24 x 32 from a 5.8 GB table: 423 us; 446 through LDS, 454 with the exchange);
+  //  * an output of 200 MB and more from a cached table: through LDS as for sparse rows, the form whose store
+  //    instructions write whole lines.  Warm it is level with the exchange (7.5e6 edges at 15 per row from a 160 MB
+  //    table, 16 x 8: 79.1 against 79.4 us; plain 80.7), with graphs and outputs in rotation, where the output's
+  //    lines are not in the last-level cache when they are written, well ahead (108.7 against 125.8 us, plain 120);
+  //  * a smaller output at up to 11 edges per row: the halves of a lane's eight columns are exchanged inside lane
+  //    quads so that every store instruction writes whole 64-byte pieces (dense_store 4; 1e6 source rows, 3e6 edges
+  //    at 10 per row, plain -> exchange: 16 x 16 121 -> 87 us, 32 x 16 166 -> 90, 8 x 32 126 -> 90, 64 x 8 150 -> 93,
+  //    16 x 8 49 -> 42; the plain form's time at these shapes varies by a factor of two between builds and boxes,
+  //    the exchange's does not).  64-column tiles (half the lanes of a row idle) measured 6-13 % slower with it.
+  // F2CGT_STORE_STREAM (the caller's outputs are written once and read later) takes the LDS form throughout: with
+  // buffers in rotation the 5.8 GB case runs in 588 us against 681.
+  const bool rpm4 = avg_deg <= 16.0 * ((a.R > 0 && a.E % a.R == 0) ? 1.0 : 0.9);
+  if (!a.dense_store && a.feat_dim % 8 == 0 && rpm4) {
+    const bool cached_table = a.N * (int64_t)a.n_cb <= (192ll << 20);
+    if (store_mode() == F2CGT_STORE_STREAM) {
+      a.dense_store = 1;
+    } else if (cached_table && a.feat_dim >= 128 && a.n_tiles <= 4) {
+      if (a.R * (int64_t)a.feat_dim * 4 >= (200ll << 20)) a.dense_store = 1;
+      else if (avg_deg <= 11.0) a.dense_store = 4;
+    }
+  }
 #ifdef F2CGT_EXPERIMENTS
   {
     if (const char* d = getenv("F2CGT_VQ_DEFER")) a.store_late = atoi(d);
@@ -1378,6 +1391,18 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
       avg_deg <= 16.0 * ((a.R > 0 && a.E % a.R == 0) ? 1.0 : 0.9) && a.N * (int64_t)a.n_cb <= (192ll << 20))
     a.own_lg = 2;
 #ifdef F2CGT_EXPERIMENTS
+  if (const char* v = getenv("F2CGT_VQ_STORE")) {   // the store form whatever the shape: plain | lds | quad | own | h1
+    const bool rpm4 = avg_deg <= 16.0 * ((a.R > 0 && a.E % a.R == 0) ? 1.0 : 0.9);
+    if (a.feat_dim % 8 == 0 && rpm4) {
+      if (!strcmp(v, "h1")) {
+        a.dense_store = 0; a.own_lg = 0;
+        return launch_wave<BT, 1, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+      }
+      a.own_lg = (!strcmp(v, "own") && a.w == 32 && a.feat_dim % 32 == 0) ? 2 : 0;
+      a.dense_store = !strcmp(v, "lds") ? 1 : (!strcmp(v, "quad") ? 4 : 0);
+      return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);
+    }
+  }
   if (const char* v = getenv("F2CGT_VQ_RPM")) {   // rows per mini-block whatever the degree (mini-blocks above 64 edges unstaged)
     if (a.feat_dim % 8 == 0) {
       if (atoi(v) == 4) return launch_wave<BT, 2, 4>(a, indptr, indices, idx_dtype, out, st, what, grid, wlds);

@@ -9,6 +9,7 @@
     python3 -m f2cgt_amd.experiments affine-geometry x   the affine kernel by edges per row: edge mapping, accumulator sizing, block rows, workgroup size
     python3 -m f2cgt_amd.experiments hybrid-geometry x   the two-table kernel by edges per row: workgroup size and edge batch
     python3 -m f2cgt_amd.experiments vq-degrees x        the fused VQ kernel on uniform and ragged rows: rows per mini-block
+    python3 -m f2cgt_amd.experiments vq-store-forms warm|rotate   the fused VQ kernel's store forms by shape
     python3 -m f2cgt_amd.experiments store-form x        plain against non-temporal output stores by shape (any build)
     python3 -m f2cgt_amd.experiments lds-rate x          bytes per clock and CU that conflict-free LDS reads return
     python3 -m f2cgt_amd.experiments cold-parts c2|c3|c4|c5   launch time by what of the input is still cached (any build)
@@ -337,6 +338,71 @@ def vq_degrees(_):
             case("capped at %d, scale %.1f" % (fanout, scale), raw.clamp(max=fanout))
 
 
+def vq_store_forms(how):
+    """The fused VQ kernel's ways of storing a lane's eight columns (F2CGT_VQ_STORE; experiments build): as they are
+    (two 16-byte stores that each write 16 of every 32 bytes), turned round in LDS (256 contiguous bytes per row and
+    instruction), halves exchanged inside lane quads (64 contiguous bytes), columns owned by groups of four lanes
+    (codebooks of 32 columns: 64 contiguous bytes at no cost in instructions), and one float4 per lane (32 lanes per
+    row).  `warm`: one graph and one output; `rotate`: five graphs and outputs in turn, so that neither the source ids
+    nor the output lines of a launch are cached when it starts."""
+    import torch
+
+    sys.path.insert(0, ROOT)
+    from f2cgt_amd import capi, synth
+
+    if not hasattr(capi.lib(), "f2cgt_experiment_set_acc_trace"):
+        raise SystemExit("the library in tree was built without --experiments")
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    copies = 5 if how == "rotate" else 1
+
+    def timed(fns, steps=30, warm=10):
+        for i in range(warm):
+            fns[i % len(fns)]()
+        torch.cuda.synchronize()
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for i in range(steps):
+            fns[i % len(fns)]()
+        t1.record()
+        torch.cuda.synchronize()
+        return t0.elapsed_time(t1) / steps * 1e3
+
+    forms = ("", "plain", "lds", "quad", "own", "h1")
+    print("us per launch (%s): shipped | plain | through LDS | quad exchange | groups of four lanes | one float4 per lane"
+          % how)
+    shapes = [(1_000_000, d, w, f, 3_000_000 if d <= 256 else 2_000_000)
+              for w, d in ((8, 128), (8, 256), (8, 512), (8, 768), (16, 128), (16, 256), (16, 512), (32, 128), (32, 256),
+                           (32, 768), (8, 64), (8, 200), (32, 600))
+              for f in (5, 8, 10, 12, 14, 16)]
+    shapes += [(10_000_000, 128, 8, 15, 7_500_000), (10_000_000, 128, 8, 10, 5_000_000), (10_000_000, 256, 16, 10, 3_000_000),
+               (240_000_000, 768, 32, 10, 6_000_000)]
+    for n_src, dim, w, fanout, edges in shapes:
+        rows = edges // fanout
+        n_cb = (dim + w - 1) // w
+        codes = torch.randint(0, 256, (n_src, n_cb), generator=gen, device="cuda", dtype=torch.uint8)
+        cbs = torch.randn((n_cb, 256, w), device="cuda")
+        indptr = synth.csc_from_degrees(torch.full((rows,), fanout, dtype=torch.int64, device="cuda"), torch.int64)
+        ids = [synth.zipf_ids(n_src, (rows * fanout,), 1.1, gen, "cuda", torch.int64) for _ in range(copies)]
+        outs = [torch.empty((rows, dim), dtype=torch.float32, device="cuda") for _ in range(copies)]
+        fns = [(lambda i=i: capi.vq_decompress_spmm_csr(codes, cbs, indptr, ids[i], dim, out=outs[i])) for i in range(copies)]
+        res = []
+        for form in forms:
+            os.environ.pop("F2CGT_VQ_STORE", None)
+            if form == "own" and not (w == 32 and dim % 32 == 0):
+                res.append(float("nan"))
+                continue
+            if form:
+                os.environ["F2CGT_VQ_STORE"] = form
+            res.append(timed(fns))
+        os.environ.pop("F2CGT_VQ_STORE", None)
+        print("  %9d source rows, %3d columns as %2d x %-2d, %2d edges per row, %4d MB out: " % (
+            n_src, dim, n_cb, w, fanout, rows * dim * 4 // 1_000_000)
+            + " | ".join("     -" if r != r else "%6.1f" % r for r in res), flush=True)
+        del codes, ids, outs, fns
+        torch.cuda.empty_cache()
+
+
 def store_form(_):
     """Plain against non-temporal output stores of the two SQ row-block kernels by output size, row width and
     edges per row, and what the default picks (f2cgt_set_store_mode; any build)."""
@@ -510,7 +576,7 @@ def cold_parts(name):
 
 if __name__ == "__main__":
     modes = {"wave-age": wave_age, "block-phases": block_phases, "dispatch-cost": dispatch_cost, "hot-rows": hot_rows,
-             "affine-geometry": affine_geometry, "hybrid-geometry": hybrid_geometry, "vq-degrees": vq_degrees, "store-form": store_form, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
+             "affine-geometry": affine_geometry, "hybrid-geometry": hybrid_geometry, "vq-degrees": vq_degrees, "vq-store-forms": vq_store_forms, "store-form": store_form, "mfma-overlap": mfma_overlap, "lds-rate": lds_rate,
              "cold-parts": cold_parts}
     if len(sys.argv) != 3 or sys.argv[1] not in modes:
         print(__doc__)

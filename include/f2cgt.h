@@ -66,7 +66,10 @@ int f2cgt_num_cus(void);
  * Plain stores are fastest when the same output buffer is written again before the last-level cache
  * (256 MB) has been turned over, as in a loop over one buffer; a caller whose outputs are written
  * once and consumed later (a training step with other large kernels in between) is better off
- * streaming.  Results are identical in every mode.  Process-wide; returns the previous mode, or
+ * streaming.  The fused VQ operator stores through the same path in every mode; in F2CGT_STORE_STREAM it
+ * takes, at up to 16 edges per row, the form whose store instructions write whole lines (a few per cent
+ * slower into a buffer that is still cached, 14 % faster into one that is not).
+ * Results are identical in every mode.  Process-wide; returns the previous mode, or
  * F2CGT_E_INVALID for a value that is none of the three (the mode is then unchanged). */
 #define F2CGT_STORE_AUTO 0
 #define F2CGT_STORE_STREAM 1

@@ -149,10 +149,11 @@ def test_rows_per_block_follow_the_launch_size():
 
 
 def test_fused_vq_store_form_by_shape():
-    """aux[2] of a vq_wave_kernel plan is the store form: 1 = results turned round in LDS (up to 8 edges per row),
-    4 = halves exchanged inside lane quads (a cached code table and either up to 11 edges per row or an output beyond
-    the last-level cache), 0 = stored as they are; aux[3] is the binary logarithm of the number of lanes that own the
-    columns of a code together (2 for codebooks of 32 columns from a cached table where the exchange is not taken)."""
+    """aux[2] of a vq_wave_kernel plan is the store form: 1 = results turned round in LDS (up to 8 edges per row, and up
+    to 16 for an output of 200 MB and more from a cached code table, or throughout in the streaming store mode), 4 =
+    halves exchanged inside lane quads (a cached table, a smaller output, up to 11 edges per row), 0 = stored as they
+    are; aux[3] is the binary logarithm of the number of lanes that own the columns of a code together (2 for
+    codebooks of 32 columns from a cached table where neither of the other forms is taken)."""
     def form(rows, fanout, d, n_cb, w, n_src):
         rc, plan = capi.dry_run("f2cgt_vq_decompress_spmm_csr", A16, capi.DT_U8, A16, A16, A16, capi.DT_I64, A16, rows,
                                 rows * fanout, n_src, d, n_cb, 256, w, None)
@@ -161,13 +162,14 @@ def test_fused_vq_store_form_by_shape():
     assert form(300_000, 5, 128, 16, 8, 1_000_000) == (1, 0)
     assert form(300_000, 5, 128, 4, 32, 1_000_000) == (1, 0)
     assert form(300_000, 10, 128, 16, 8, 1_000_000) == (4, 0)
-    assert form(300_000, 10, 256, 16, 16, 1_000_000) == (4, 0)
-    assert form(300_000, 14, 256, 16, 16, 1_000_000) == (4, 0)      # 307 MB of output
+    assert form(150_000, 10, 256, 16, 16, 1_000_000) == (4, 0)
+    assert form(300_000, 10, 256, 16, 16, 1_000_000) == (1, 0)      # 307 MB of output
+    assert form(300_000, 14, 256, 16, 16, 1_000_000) == (1, 0)
     assert form(100_000, 14, 256, 16, 16, 1_000_000) == (0, 0)
-    assert form(300_000, 10, 512, 16, 32, 1_000_000) == (4, 0)
+    assert form(300_000, 10, 512, 16, 32, 1_000_000) == (1, 0)
     assert form(100_000, 14, 512, 16, 32, 1_000_000) == (0, 2)
-    assert form(200_000, 10, 768, 24, 32, 1_000_000) == (0, 2)       # six column tiles: no exchange
-    assert form(500_000, 15, 128, 16, 8, 10_000_000) == (4, 0)      # 256 MB of output from a 160 MB table
+    assert form(200_000, 10, 768, 24, 32, 1_000_000) == (0, 2)       # six column tiles
+    assert form(500_000, 15, 128, 16, 8, 10_000_000) == (1, 0)      # 256 MB of output from a 160 MB table
     assert form(100_000, 15, 128, 16, 8, 10_000_000) == (0, 0)      # 51 MB of output: the halves meet in the cache
     assert form(600_000, 10, 768, 24, 32, 240_000_000) == (0, 0)    # a 5.8 GB table: the gather dominates
     assert form(200_000, 10, 768, 96, 8, 1_000_000) == (0, 0)       # six column tiles
@@ -176,6 +178,13 @@ def test_fused_vq_store_form_by_shape():
     assert form(300_000, 20, 128, 4, 32, 1_000_000) == (0, 0)
     assert form(300_000, 10, 600, 19, 32, 1_000_000) == (0, 0)      # 600 columns: the last tile ends inside a group of 32
     assert form(300_000, 10, 100, 13, 8, 1_000_000)[1] == 0         # four columns per lane: dense as they are
+    was = capi.set_store_mode(capi.STORE_STREAM)
+    try:
+        assert form(600_000, 10, 768, 24, 32, 240_000_000) == (1, 0)
+        assert form(300_000, 10, 128, 16, 8, 1_000_000) == (1, 0)
+        assert form(300_000, 20, 128, 16, 8, 1_000_000) == (0, 0)
+    finally:
+        capi.set_store_mode(was)
     # aux[0]: float4 per lane and edge (2 = a lane owns eight columns); sparse rows that are no whole 128-byte lines
     # take one, code rows that are no multiple of a tile (24 x 8, 7 x 32) can take the turn through LDS
     lanes = lambda rows, fanout, d, n_cb, w: capi.dry_run(

@@ -223,6 +223,15 @@ def test_fused_vq_halves_exchanged_inside_lane_quads(feat_dim, n_cb, width, fano
     dec = oc.vq_decompress(codes, cbs, feat_dim).astype(np.float64)
     exact = oc.spmm_csr(dec, indptr, indices)
     assert_mean_aggregate(got.cpu().numpy(), want, exact, float(np.abs(dec).max()))
+    # the streaming store mode turns the results round in LDS at these row lengths too: same sums, bit for bit
+    was = capi.set_store_mode(capi.STORE_STREAM)
+    try:
+        streamed = capi.vq_decompress_spmm_csr(dev(codes), dev(cbs), dev(indptr.astype(idx)), dev(indices.astype(idx)),
+                                               feat_dim)
+        torch.cuda.synchronize()
+    finally:
+        capi.set_store_mode(was)
+    assert torch.equal(got, streamed)
 
 
 @pytest.mark.parametrize("idx", [np.int64, np.int32])
