@@ -1341,11 +1341,14 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
   // Above that (up to 16 edges per row, four-row mini-blocks) the form is chosen by what binds the launch:
   //  * the code table beyond the caches (over 192 MB) or rows of more than four column tiles: the gather binds, the
   //    results are stored as they are (24 x 32 from a 5.8 GB table: 423 us; 446 through LDS, 454 with the exchange);
-  //  * an output of 200 MB and more from a cached table: through LDS as for sparse rows, the form whose store
-  //    instructions write whole lines.  Warm it is level with the exchange (7.5e6 edges at 15 per row from a 160 MB
-  //    table, 16 x 8: 79.1 against 79.4 us; plain 80.7), with graphs and outputs in rotation, where the output's
-  //    lines are not in the last-level cache when they are written, well ahead (108.7 against 125.8 us, plain 120);
-  //  * a smaller output at up to 11 edges per row: the halves of a lane's eight columns are exchanged inside lane
+  //  * an output of 200 MB and more from a table of 64 to 192 MB, which shares the last-level cache with it: through
+  //    LDS as for sparse rows, the form whose store instructions write whole lines.  Warm it is level with the exchange
+  //    (7.5e6 edges at 15 per row from a 160 MB table, 16 x 8: 79.1 against 79.4 us; plain 80.7), with graphs and
+  //    outputs in rotation, where the output's lines are not in the last-level cache when they are written, well
+  //    ahead (108.7 against 125.8 us, plain 120; 16 x 16 at 10 edges per row 73 / 99 against 79 / 102);
+  //  * from a smaller table, such an output or up to 11 edges per row (an output of 340 MB from 32 MB of codes,
+  //    32 x 16 at 12 edges per row: 130 / 131 us warm / in rotation against 135 / 136 through LDS): the halves of a
+  //    lane's eight columns are exchanged inside lane
   //    quads so that every store instruction writes whole 64-byte pieces (dense_store 4; 1e6 source rows, 3e6 edges
   //    at 10 per row, plain -> exchange: 16 x 16 121 -> 87 us, 32 x 16 166 -> 90, 8 x 32 126 -> 90, 64 x 8 150 -> 93,
   //    16 x 8 49 -> 42; the plain form's time at these shapes varies by a factor of two between builds and boxes,
@@ -1358,8 +1361,9 @@ int launch_vq(VqArgs a, const void* indptr, const void* indices, int idx_dtype, 
     if (store_mode() == F2CGT_STORE_STREAM) {
       a.dense_store = 1;
     } else if (cached_table && a.feat_dim >= 128 && a.n_tiles <= 4) {
-      if (a.R * (int64_t)a.feat_dim * 4 >= (200ll << 20)) a.dense_store = 1;
-      else if (avg_deg <= 11.0) a.dense_store = 4;
+      const bool big_out = a.R * (int64_t)a.feat_dim * 4 >= (200ll << 20);
+      if (big_out && a.N * (int64_t)a.n_cb >= (64ll << 20)) a.dense_store = 1;
+      else if (big_out || avg_deg <= 11.0) a.dense_store = 4;
     }
   }
 #ifdef F2CGT_EXPERIMENTS

@@ -150,8 +150,8 @@ def test_rows_per_block_follow_the_launch_size():
 
 def test_fused_vq_store_form_by_shape():
     """aux[2] of a vq_wave_kernel plan is the store form: 1 = results turned round in LDS (up to 8 edges per row, and up
-    to 16 for an output of 200 MB and more from a cached code table, or throughout in the streaming store mode), 4 =
-    halves exchanged inside lane quads (a cached table, a smaller output, up to 11 edges per row), 0 = stored as they
+    to 16 for an output of 200 MB and more from a code table of 64 to 192 MB, or throughout in the streaming store mode),
+    4 = halves exchanged inside lane quads (a cached table: up to 11 edges per row, or a large output), 0 = stored as they
     are; aux[3] is the binary logarithm of the number of lanes that own the columns of a code together (2 for
     codebooks of 32 columns from a cached table where neither of the other forms is taken)."""
     def form(rows, fanout, d, n_cb, w, n_src):
@@ -163,10 +163,11 @@ def test_fused_vq_store_form_by_shape():
     assert form(300_000, 5, 128, 4, 32, 1_000_000) == (1, 0)
     assert form(300_000, 10, 128, 16, 8, 1_000_000) == (4, 0)
     assert form(150_000, 10, 256, 16, 16, 1_000_000) == (4, 0)
-    assert form(300_000, 10, 256, 16, 16, 1_000_000) == (1, 0)      # 307 MB of output
-    assert form(300_000, 14, 256, 16, 16, 1_000_000) == (1, 0)
+    assert form(300_000, 10, 256, 16, 16, 1_000_000) == (4, 0)      # 307 MB of output from 16 MB of codes
+    assert form(300_000, 14, 256, 16, 16, 1_000_000) == (4, 0)
+    assert form(300_000, 14, 256, 16, 16, 10_000_000) == (1, 0)     # from 160 MB of codes
     assert form(100_000, 14, 256, 16, 16, 1_000_000) == (0, 0)
-    assert form(300_000, 10, 512, 16, 32, 1_000_000) == (1, 0)
+    assert form(300_000, 10, 512, 16, 32, 1_000_000) == (4, 0)
     assert form(100_000, 14, 512, 16, 32, 1_000_000) == (0, 2)
     assert form(200_000, 10, 768, 24, 32, 1_000_000) == (0, 2)       # six column tiles
     assert form(500_000, 15, 128, 16, 8, 10_000_000) == (1, 0)      # 256 MB of output from a 160 MB table
