@@ -329,6 +329,36 @@ def _others(idx):
                                      "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
     del wl, out, feat
     torch.cuda.empty_cache()
+    # Reddit's width, 602 columns: rows of 4 k + 2 columns start at multiples of 8 bytes only and end with a group of two
+    # columns.  2e6 edges at 10 per row from 1e6 source rows, next to the same launch at 600 columns.
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    rows602, fan602, src602 = 200_000, 10, 1_000_000
+    ptr602 = synth.csc_from_degrees(torch.full((rows602,), fan602, dtype=torch.int64, device="cuda"), torch.int64)
+    ids602 = synth.zipf_ids(src602, (rows602 * fan602,), 1.1, gen, "cuda", torch.int64)
+    cb5 = torch.tensor([[0.01, 3.0, -6.643856, 1.5849625, 0.4]], device="cuda")
+    for dim in (602, 600):
+        o = torch.empty((rows602, dim), dtype=torch.float32, device="cuda")
+        c4 = torch.randint(0, 256, (src602, dim // 2), generator=gen, device="cuda", dtype=torch.uint8)
+        par = torch.stack([torch.randn(dim, device="cuda"), torch.rand(dim, device="cuda")]).contiguous()
+        vc = torch.randint(0, 256, (src602, 19), generator=gen, device="cuda", dtype=torch.uint8)
+        vcb = torch.randn((19, 256, 32), device="cuda")
+        entry = {}
+        _, ms = _time_steps(lambda: capi.sq_affine_decompress_spmm_csr(c4, par, ptr602, ids602, 4, dim, out=o), 30, 10)
+        entry["affine_sq4_us"] = ms * 1e3
+        _, ms = _time_steps(lambda: capi.sq_decompress_spmm_csr(c4, cb5, ptr602, ids602, 4, dim, dim, out=o), 30, 10)
+        entry["log_sq4_us"] = ms * 1e3
+        _, ms = _time_steps(lambda: capi.vq_decompress_spmm_csr(vc, vcb, ptr602, ids602, dim, out=o), 30, 10)
+        entry["vq_19x32_us"] = ms * 1e3
+        f32 = torch.randn((src602, dim), device="cuda")
+        _, ms = _time_steps(lambda: capi.spmm_csr(f32, ptr602, ids602, out=o), 30, 10)
+        entry["spmm_csr_fp32_us"] = ms * 1e3
+        del f32
+        _, ms = _time_steps(lambda: capi.sq_decompress(c4[:400_000], cb5, 4, dim, dim), 30, 10)
+        entry["sq_decompress4_4e5_rows_us"] = ms * 1e3
+        res["fused_and_decode_at_%d_columns" % dim] = entry
+        del o, c4, par, vc, vcb
+        torch.cuda.empty_cache()
     # the aggregation together with the dense layer that consumes it, at the widest shape (768
     # features -> 256 hidden units, fp32 like the reference's model): the aggregation alone, the GEMM
     # alone, the module's *_linear op (one aggregation, one GEMM), its row-blocked form (bounded
